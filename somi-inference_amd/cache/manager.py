@@ -1,0 +1,218 @@
+"""The cache manager: paged keys/values per group of layers, block tables per request,
+and slots for fixed-size per-request state.
+
+Reference: ``KVCacheManager`` (somi_inference/core/paged_attention.py:112-296):
+one allocator, one tensor per layer, per-sequence page lists and token counts;
+``allocate_slots`` before the forward and ``advance_tokens`` after it
+(:202-221, :294-296); ``free_sequence`` returns every page (:195-200); a
+duplicate ``register_sequence`` raises "already registered" (:150-156).
+
+Beyond the reference: layers are put into *groups* by what they need.  Layers
+that keep every key share one page pool and one block table per request; layers
+that see a window of keys form a group of their own whose pages are released as
+soon as the window has passed them, while the request is still live.  Mixers
+with fixed-size state get one slot per request in a state tensor (this
+architecture has none; the slot is assigned all the same so nothing changes
+when one is added).
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Hashable
+
+import torch
+
+from ..parts.base import FixedStateSpec, LayerCache, PagedKVSpec
+from .pool import CacheError, OutOfPages, PagePool
+
+RELEASED = -1     # host-side mark of a logical page a window has passed
+
+
+@dataclass
+class PagedGroup:
+    window: int | None
+    pool: PagePool
+    runs: list[int] = field(default_factory=list)      # layer runs whose tensors use this group's page ids
+
+
+@dataclass
+class RequestCache:
+    num_tokens: int = 0
+    pages: list[list[int]] = field(default_factory=list)   # per group: logical page -> physical page or RELEASED
+    state_slot: int = -1
+
+
+class CacheManager:
+    def __init__(self, needs: list[PagedKVSpec | FixedStateSpec | int | None], *, block_size: int,
+                 num_blocks: int, max_requests: int, dtype: torch.dtype, device: torch.device | str,
+                 allocate_tensors: bool = True) -> None:
+        if block_size < 1 or num_blocks < 1 or max_requests < 1:
+            raise ValueError("block_size, num_blocks and max_requests must be >= 1")
+        self.block_size, self.num_blocks, self.max_requests = int(block_size), int(num_blocks), int(max_requests)
+        self.dtype, self.device = dtype, torch.device(device)
+        self.groups: list[PagedGroup] = []
+        self.layer_caches: list[LayerCache | None] = [None] * len(needs)
+        by_window: dict[int | None, int] = {}
+        for run, need in enumerate(needs):
+            if isinstance(need, PagedKVSpec):
+                if need.window not in by_window:
+                    by_window[need.window] = len(self.groups)
+                    self.groups.append(PagedGroup(need.window, PagePool(self.num_blocks)))
+                group = by_window[need.window]
+                self.groups[group].runs.append(run)
+                k = v = None
+                if allocate_tensors:
+                    shape = (self.num_blocks, need.num_kv_heads, self.block_size, need.head_dim)
+                    k = torch.zeros(shape, dtype=dtype, device=self.device)
+                    v = torch.zeros(shape, dtype=dtype, device=self.device)
+                self.layer_caches[run] = LayerCache(need, group, k=k, v=v)
+            elif isinstance(need, FixedStateSpec):
+                state = None
+                if allocate_tensors:
+                    state = torch.zeros((self.max_requests, *need.shape), dtype=need.dtype, device=self.device)
+                self.layer_caches[run] = LayerCache(need, -1, state=state)
+        for run, need in enumerate(needs):          # runs that read an earlier run's cache
+            if isinstance(need, int) and not isinstance(need, bool):
+                source = self.layer_caches[need]
+                if source is None:
+                    raise CacheError(f"run {run} reads the cache of run {need}, which has none")
+                self.layer_caches[run] = LayerCache(source.spec, source.group, k=source.k, v=source.v,
+                                                    state=source.state, writes=False)
+        self._requests: dict[Hashable, RequestCache] = {}
+        self._free_slots = list(range(self.max_requests - 1, -1, -1))
+
+    # --------------------------------------------------------------- requests
+    def has(self, request_id: Hashable) -> bool:
+        return request_id in self._requests
+
+    def live_requests(self) -> list[Hashable]:
+        return list(self._requests)
+
+    def register(self, request_id: Hashable) -> None:
+        if request_id in self._requests:
+            raise CacheError(f"request {request_id!r} is already registered")
+        if not self._free_slots:
+            raise CacheError(f"all {self.max_requests} request slots are in use")
+        slot = self._free_slots.pop()
+        self._requests[request_id] = RequestCache(0, [[] for _ in self.groups], slot)
+        for cache in self.layer_caches:
+            if cache is not None and cache.state is not None and cache.writes:
+                cache.state[slot].zero_()
+
+    def free(self, request_id: Hashable) -> None:
+        """Give back every page and the state slot of a request."""
+        record = self._get(request_id)
+        for group, pages in zip(self.groups, record.pages):
+            for page in pages:
+                if page != RELEASED:
+                    group.pool.release(page)
+        self._free_slots.append(record.state_slot)
+        del self._requests[request_id]
+
+    def _get(self, request_id: Hashable) -> RequestCache:
+        if request_id not in self._requests:
+            raise CacheError(f"request {request_id!r} is not registered")
+        return self._requests[request_id]
+
+    def num_tokens(self, request_id: Hashable) -> int:
+        return self._get(request_id).num_tokens
+
+    def state_slot(self, request_id: Hashable) -> int:
+        return self._get(request_id).state_slot
+
+    # ------------------------------------------------------------------ pages
+    def _pages_for(self, length: int) -> int:
+        return (length + self.block_size - 1) // self.block_size
+
+    def pages_needed(self, request_id: Hashable, new_tokens: int) -> list[int]:
+        """Per group, how many pages a portion of ``new_tokens`` more tokens has to take."""
+        record = self._get(request_id)
+        total = self._pages_for(record.num_tokens + new_tokens)
+        return [max(0, total - len(pages)) for pages in record.pages]
+
+    def free_pages(self) -> list[int]:
+        return [group.pool.num_free for group in self.groups]
+
+    def can_reserve(self, portions: list[tuple[Hashable, int]]) -> bool:
+        want = [0] * len(self.groups)
+        for request_id, new_tokens in portions:
+            for g, n in enumerate(self.pages_needed(request_id, new_tokens)):
+                want[g] += n
+        return all(w <= f for w, f in zip(want, self.free_pages()))
+
+    def reserve(self, request_id: Hashable, new_tokens: int) -> None:
+        """Take the pages that positions ``num_tokens .. num_tokens + new_tokens - 1`` fall in.
+
+        Either every group gets its pages or nothing changes (then :class:`OutOfPages`).
+        """
+        if new_tokens < 1:
+            raise CacheError("a portion holds at least one token")
+        record = self._get(request_id)
+        needed = self.pages_needed(request_id, new_tokens)
+        for group, n in zip(self.groups, needed):
+            if n > group.pool.num_free:
+                raise OutOfPages(f"request {request_id!r} needs {n} more pages, {group.pool.num_free} are free")
+        for group, pages, n in zip(self.groups, record.pages, needed):
+            for _ in range(n):
+                pages.append(group.pool.allocate())
+
+    def commit(self, request_id: Hashable, new_tokens: int) -> None:
+        """Count the tokens a step wrote, and give back pages a window has passed."""
+        record = self._get(request_id)
+        record.num_tokens += new_tokens
+        for group, pages in zip(self.groups, record.pages):
+            if self._pages_for(record.num_tokens) > len(pages):
+                raise CacheError(f"request {request_id!r}: tokens committed beyond the reserved pages")
+            if group.window is None:
+                continue
+            # The next token sits at position num_tokens and sees keys from
+            # num_tokens - window + 1 on; pages wholly below that are done.
+            first_visible = record.num_tokens - group.window + 1
+            for logical in range(min(len(pages), max(0, first_visible) // self.block_size)):
+                if pages[logical] != RELEASED:
+                    group.pool.release(pages[logical])
+                    pages[logical] = RELEASED
+
+    # ------------------------------------------------------- tables for a step
+    def page_list(self, group: int, request_id: Hashable) -> list[int]:
+        return self._get(request_id).pages[group]
+
+    def slots(self, group: int, request_id: Hashable, start: int, count: int) -> list[int]:
+        """Physical slot (page * block_size + offset) of positions start .. start + count - 1."""
+        pages = self._get(request_id).pages[group]
+        out = []
+        for pos in range(start, start + count):
+            page = pages[pos // self.block_size]
+            if page == RELEASED:
+                raise CacheError(f"position {pos} of request {request_id!r} lies in a released page")
+            out.append(page * self.block_size + pos % self.block_size)
+        return out
+
+    # -------------------------------------------------------------- invariants
+    def check_invariants(self) -> None:
+        """No page lost, held twice or free while held; slots likewise."""
+        for g, group in enumerate(self.groups):
+            held: dict[int, Hashable] = {}
+            for request_id, record in self._requests.items():
+                for page in record.pages[g]:
+                    if page == RELEASED:
+                        continue
+                    if page in held:
+                        raise CacheError(f"group {g}: page {page} held by {held[page]!r} and {request_id!r}")
+                    held[page] = request_id
+            free = group.pool.free_pages()
+            if len(set(free)) != len(free):
+                raise CacheError(f"group {g}: a page is on the free list twice")
+            if set(free) & set(held):
+                raise CacheError(f"group {g}: pages both free and held: {sorted(set(free) & set(held))}")
+            if len(free) + len(held) != group.pool.num_pages:
+                raise CacheError(f"group {g}: {group.pool.num_pages - len(free) - len(held)} pages lost")
+            for page in held:
+                if group.pool.refcount(page) != 1:
+                    raise CacheError(f"group {g}: page {page} has refcount {group.pool.refcount(page)}")
+        slots = [r.state_slot for r in self._requests.values()]
+        if len(set(slots)) != len(slots) or set(slots) & set(self._free_slots):
+            raise CacheError("a state slot is held twice or both free and held")
+        if len(slots) + len(self._free_slots) != self.max_requests:
+            raise CacheError("a state slot is lost")

@@ -1,0 +1,134 @@
+"""One step's batch: portions of requests as flat device arrays.
+
+The reference passes ``input_ids[1, T]`` for one whole prompt or ``[B, 1]`` for
+decoded tokens and derives positions from ``arange(T)`` or the token counts
+(somi_inference/models/qwen2_adapter.py:91, 134-137), and rebuilds block tables
+in every layer (somi_inference/core/paged_attention.py:173-193 via
+qwen2_adapter.py:117).  Here every token carries its request's entry index and
+its position explicitly, the tables are built once per step on the host as
+int32 and reach the device in one copy.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Hashable
+
+import numpy as np
+import torch
+
+from ..cache.manager import RELEASED, CacheManager
+
+
+@dataclass
+class StepEntry:
+    """A request's next tokens and the places among them whose logits are wanted."""
+
+    request_id: Hashable
+    tokens: list[int]
+    want: list[int] = field(default_factory=list)
+
+
+@dataclass
+class EntryInfo:
+    request_id: Hashable
+    start: int          # index of the entry's first token in the flat batch
+    length: int
+    first_position: int  # position of that token in its request (= tokens cached before the step)
+    state_slot: int
+
+
+@dataclass
+class PagedView:
+    """A cache group's view of the step."""
+
+    slot_mapping: torch.Tensor      # [N] int32: page * block_size + offset where token t's k/v go
+    block_table: torch.Tensor       # [E, max_blocks] int32 physical pages of each entry's request
+
+
+@dataclass
+class StepBatch:
+    num_tokens: int
+    num_entries: int
+    num_logit_rows: int
+    token_ids: torch.Tensor         # [N] int32
+    positions: torch.Tensor         # [N] int32
+    token_entry: torch.Tensor       # [N] int32: entry index of each token
+    entry_start: torch.Tensor       # [E + 1] int32: offsets of the entries in the flat batch
+    entry_first_position: torch.Tensor   # [E] int32
+    context_lens: torch.Tensor      # [E] int32: tokens of each request after this step
+    state_slots: torch.Tensor       # [E] int32
+    logit_rows: torch.Tensor        # [R] int32 flat token indices whose logits are wanted
+    paged: list[PagedView]
+    entries: list[EntryInfo]        # host mirror
+    max_entry_len: int
+    max_context: int
+    block_size: int
+
+
+def build_step(entries: list[StepEntry], cache: CacheManager, device: torch.device) -> StepBatch:
+    """Lay out the step on the host and copy it to the device in one transfer.
+
+    Pages for the new tokens must already be reserved: slot mappings and block
+    tables are read from the cache manager as they stand.
+    """
+    infos: list[EntryInfo] = []
+    token_ids: list[int] = []
+    positions: list[int] = []
+    token_entry: list[int] = []
+    logit_rows: list[int] = []
+    for index, entry in enumerate(entries):
+        first = cache.num_tokens(entry.request_id)
+        infos.append(EntryInfo(entry.request_id, len(token_ids), len(entry.tokens), first,
+                               cache.state_slot(entry.request_id)))
+        logit_rows.extend(len(token_ids) + w for w in entry.want)
+        token_ids.extend(entry.tokens)
+        positions.extend(range(first, first + len(entry.tokens)))
+        token_entry.extend([index] * len(entry.tokens))
+    n, e = len(token_ids), len(entries)
+    bs = cache.block_size
+    tables, slot_maps, widths = [], [], []
+    for g in range(len(cache.groups)):
+        rows = [cache.page_list(g, info.request_id) for info in infos]
+        width = max(1, max((len(r) for r in rows), default=1))
+        table = np.zeros((e, width), dtype=np.int32)
+        for r, pages in enumerate(rows):
+            # released pages read as page 0: the kernels never look below a window
+            table[r, :len(pages)] = [0 if p == RELEASED else p for p in pages]
+        slots: list[int] = []
+        for info in infos:
+            slots.extend(cache.slots(g, info.request_id, info.first_position, info.length))
+        tables.append(table)
+        slot_maps.append(np.asarray(slots, dtype=np.int32))
+        widths.append(width)
+
+    sections = [
+        np.asarray(token_ids, dtype=np.int32), np.asarray(positions, dtype=np.int32),
+        np.asarray(token_entry, dtype=np.int32),
+        np.asarray([i.start for i in infos] + [n], dtype=np.int32),
+        np.asarray([i.first_position for i in infos], dtype=np.int32),
+        np.asarray([i.first_position + i.length for i in infos], dtype=np.int32),
+        np.asarray([i.state_slot for i in infos], dtype=np.int32),
+        np.asarray(logit_rows, dtype=np.int32),
+    ]
+    for table, slots in zip(tables, slot_maps):
+        sections += [slots, table.reshape(-1)]
+    offsets = np.cumsum([0] + [s.size for s in sections])
+    packed = torch.from_numpy(np.concatenate(sections) if sections else np.zeros(0, np.int32))
+    on_device = packed.to(device)
+
+    def part(i: int) -> torch.Tensor:
+        return on_device[int(offsets[i]):int(offsets[i + 1])]
+
+    paged = []
+    for g in range(len(cache.groups)):
+        paged.append(PagedView(part(8 + 2 * g), part(9 + 2 * g).view(e, widths[g])))
+    return StepBatch(
+        num_tokens=n, num_entries=e, num_logit_rows=len(logit_rows),
+        token_ids=part(0), positions=part(1), token_entry=part(2), entry_start=part(3),
+        entry_first_position=part(4), context_lens=part(5), state_slots=part(6), logit_rows=part(7),
+        paged=paged, entries=infos,
+        max_entry_len=max((i.length for i in infos), default=0),
+        max_context=max((i.first_position + i.length for i in infos), default=0),
+        block_size=bs,
+    )

@@ -1,0 +1,206 @@
+"""Python faces of the HIP entry points.
+
+Each function checks on the host what its kernel assumes (device, dtype,
+contiguity, shapes), launches on torch's current stream and raises
+:class:`KernelError` with the library's message on failure.  There is no
+fallback to a library or CPU implementation: the product path fails loudly
+when the extension cannot be built or loaded.
+"""
+
+from __future__ import annotations
+
+import ctypes
+
+import torch
+
+from ..csrc import build as _build
+
+F32, BF16 = 0, 1
+
+
+class KernelError(RuntimeError):
+    """A kernel entry point refused its arguments or failed to launch."""
+
+
+def library() -> ctypes.CDLL:
+    return _build.load()
+
+
+def dtype_code(dtype: torch.dtype) -> int:
+    if dtype == torch.float32:
+        return F32
+    if dtype == torch.bfloat16:
+        return BF16
+    raise KernelError(f"unsupported dtype {dtype}; kernels take float32 and bfloat16")
+
+
+def _stream() -> ctypes.c_void_p:
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _ptr(t: torch.Tensor | None) -> ctypes.c_void_p:
+    return ctypes.c_void_p(0 if t is None else t.data_ptr())
+
+
+def _check(code: int) -> None:
+    if code != 0:
+        raise KernelError(library().somi_last_error().decode("utf-8", "replace"))
+
+
+def _need(t: torch.Tensor, name: str, dtype: torch.dtype | None = None, shape: tuple | None = None) -> None:
+    if not isinstance(t, torch.Tensor):
+        raise KernelError(f"{name}: expected a tensor, got {type(t).__name__}")
+    if not t.is_cuda:
+        raise KernelError(f"{name}: must live on the GPU (there is no CPU path), got {t.device}")
+    if not t.is_contiguous():
+        raise KernelError(f"{name}: must be contiguous")
+    if dtype is not None and t.dtype != dtype:
+        raise KernelError(f"{name}: expected {dtype}, got {t.dtype}")
+    if shape is not None and tuple(t.shape) != tuple(shape):
+        raise KernelError(f"{name}: expected shape {tuple(shape)}, got {tuple(t.shape)}")
+
+
+def embedding(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+    """h[t] = table[ids[t]] as float32.  table: [V, H]; ids: [N] int32."""
+    _need(table, "embedding table")
+    _need(ids, "token ids", torch.int32)
+    vocab, hidden = table.shape
+    n = ids.numel()
+    if out is None:
+        out = torch.empty((n, hidden), dtype=torch.float32, device=table.device)
+    _need(out, "embedding out", torch.float32, (n, hidden))
+    _check(library().somi_embedding(_ptr(table), dtype_code(table.dtype), _ptr(ids), _ptr(out),
+                                    n, hidden, vocab, _stream()))
+    return out
+
+
+def gather_rows(src: torch.Tensor, rows: torch.Tensor) -> torch.Tensor:
+    """out[r] = src[rows[r]] for a float32 matrix."""
+    _need(src, "gather source", torch.float32)
+    _need(rows, "row indices", torch.int32)
+    out = torch.empty((rows.numel(), src.shape[1]), dtype=torch.float32, device=src.device)
+    _check(library().somi_gather_rows_f32(_ptr(src), _ptr(rows), _ptr(out), rows.numel(), src.shape[1], _stream()))
+    return out
+
+
+def rmsnorm(h: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype: torch.dtype,
+            delta: torch.Tensor | None = None, out: torch.Tensor | None = None) -> torch.Tensor:
+    """out = rmsnorm(h (+ delta)) * weight; with delta, h is updated in place (h += delta)."""
+    _need(h, "residual stream", torch.float32)
+    n, hidden = h.shape
+    _need(weight, "norm weight", torch.float32, (hidden,))
+    if delta is not None:
+        _need(delta, "residual delta", out_dtype, (n, hidden))
+    if out is None:
+        out = torch.empty((n, hidden), dtype=out_dtype, device=h.device)
+    _need(out, "norm out", out_dtype, (n, hidden))
+    _check(library().somi_rmsnorm(_ptr(h), _ptr(delta), _ptr(weight), ctypes.c_float(eps), _ptr(out),
+                                  dtype_code(out_dtype), n, hidden, _stream()))
+    return out
+
+
+def residual_add(h: torch.Tensor, delta: torch.Tensor) -> None:
+    _need(h, "residual stream", torch.float32)
+    _need(delta, "residual delta", None, tuple(h.shape))
+    _check(library().somi_residual_add(_ptr(h), _ptr(delta), dtype_code(delta.dtype),
+                                       ctypes.c_int64(h.numel()), _stream()))
+
+
+def linear_plain(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None,
+                 out_dtype: torch.dtype | None = None) -> torch.Tensor:
+    """x @ weight.T (+ bias) with the plain float32-accumulating kernel.  weight: [N, K]."""
+    _need(x, "linear input")
+    m, k = x.shape
+    _need(weight, "linear weight", x.dtype)
+    n = weight.shape[0]
+    if weight.shape[1] != k:
+        raise KernelError(f"linear: input has {k} features, weight expects {weight.shape[1]}")
+    if bias is not None:
+        _need(bias, "linear bias", torch.float32, (n,))
+    out_dtype = out_dtype or x.dtype
+    out = torch.empty((m, n), dtype=out_dtype, device=x.device)
+    _check(library().somi_linear_plain(_ptr(x), _ptr(weight), _ptr(bias), _ptr(out), dtype_code(x.dtype),
+                                       dtype_code(out_dtype), m, n, k, _stream()))
+    return out
+
+
+def rope_kv_store(qkv: torch.Tensor, positions: torch.Tensor, slots: torch.Tensor | None,
+                  inv_freq: torch.Tensor | None, rotary_dim: int, nq: int, nkv: int, head_dim: int,
+                  k_cache: torch.Tensor | None, v_cache: torch.Tensor | None) -> None:
+    """Rotate q (in place) and k, and store k and v in their cache pages.
+
+    qkv: [N, (nq + 2 nkv) * D]; caches: [pages, nkv, page_size, D]; slots: [N] int32.
+    """
+    _need(qkv, "qkv")
+    n = qkv.shape[0]
+    if qkv.shape[1] != (nq + 2 * nkv) * head_dim:
+        raise KernelError(f"rope_kv_store: qkv width {qkv.shape[1]} != (nq + 2 nkv) * D = {(nq + 2 * nkv) * head_dim}")
+    _need(positions, "positions", torch.int32, (n,))
+    page_size = 0
+    if nkv > 0:
+        _need(slots, "slot mapping", torch.int32, (n,))
+        _need(k_cache, "k cache", qkv.dtype)
+        _need(v_cache, "v cache", qkv.dtype, tuple(k_cache.shape))
+        if k_cache.dim() != 4 or k_cache.shape[1] != nkv or k_cache.shape[3] != head_dim:
+            raise KernelError(f"rope_kv_store: cache shape {tuple(k_cache.shape)} != [pages, {nkv}, page, {head_dim}]")
+        page_size = k_cache.shape[2]
+    if inv_freq is not None:
+        _need(inv_freq, "inv_freq", torch.float32, (rotary_dim // 2,))
+    _check(library().somi_rope_kv_store(_ptr(qkv), dtype_code(qkv.dtype), ctypes.c_int64(qkv.shape[1]),
+                                        _ptr(positions), _ptr(slots), _ptr(inv_freq), rotary_dim, n, nq, nkv,
+                                        head_dim, _ptr(k_cache), _ptr(v_cache), page_size, _stream()))
+
+
+def paged_attention_plain(q: torch.Tensor, q_stride: int, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                          block_table: torch.Tensor, token_entry: torch.Tensor, positions: torch.Tensor,
+                          nq: int, window: int, scale: float) -> torch.Tensor:
+    """Causal attention of every token over its request's cached keys (plain float32 kernel).
+
+    q: a tensor whose row t holds the nq query heads of token t first (row stride q_stride elements).
+    """
+    _need(q, "q")
+    n = q.shape[0]
+    _need(k_cache, "k cache", q.dtype)
+    _need(v_cache, "v cache", q.dtype, tuple(k_cache.shape))
+    _, nkv, page_size, head_dim = k_cache.shape
+    if q_stride < nq * head_dim or q.shape[1] < nq * head_dim:
+        raise KernelError("paged_attention: q rows are narrower than nq * head_dim")
+    _need(block_table, "block table", torch.int32)
+    _need(token_entry, "token entries", torch.int32, (n,))
+    _need(positions, "positions", torch.int32, (n,))
+    out = torch.empty((n, nq * head_dim), dtype=q.dtype, device=q.device)
+    _check(library().somi_paged_attention_plain(
+        _ptr(q), dtype_code(q.dtype), ctypes.c_int64(q_stride), _ptr(k_cache), _ptr(v_cache), _ptr(block_table),
+        block_table.shape[1], _ptr(token_entry), _ptr(positions), n, nq, nkv, head_dim, page_size, window,
+        ctypes.c_float(scale), _ptr(out), _stream()))
+    return out
+
+
+def silu_mul(gate_up: torch.Tensor) -> torch.Tensor:
+    """silu(gate_up[:, :I]) * gate_up[:, I:]."""
+    _need(gate_up, "gate_up")
+    n, two_i = gate_up.shape
+    if two_i % 2:
+        raise KernelError(f"silu_mul: width {two_i} is odd")
+    out = torch.empty((n, two_i // 2), dtype=gate_up.dtype, device=gate_up.device)
+    _check(library().somi_silu_mul(_ptr(gate_up), _ptr(out), dtype_code(gate_up.dtype), n, two_i // 2, _stream()))
+    return out
+
+
+def sample(logits: torch.Tensor, temperature: torch.Tensor, uniform: torch.Tensor) -> torch.Tensor:
+    """One token per row: argmax where temperature is 0, else an inverse-CDF draw from softmax(logits / T)."""
+    _need(logits, "logits", torch.float32)
+    rows, vocab = logits.shape
+    _need(temperature, "temperature", torch.float32, (rows,))
+    _need(uniform, "uniform", torch.float32, (rows,))
+    out = torch.empty((rows,), dtype=torch.int32, device=logits.device)
+    _check(library().somi_sample(_ptr(logits), rows, vocab, _ptr(temperature), _ptr(uniform), _ptr(out), _stream()))
+    return out
+
+
+def repetition_penalty(logits_row: torch.Tensor, ids: torch.Tensor, penalty: float) -> None:
+    """In place on one row of float32 logits; ids: distinct int32 token ids."""
+    _need(logits_row, "logits row", torch.float32)
+    _need(ids, "penalised ids", torch.int32)
+    _check(library().somi_repetition_penalty(_ptr(logits_row), logits_row.numel(), _ptr(ids), ids.numel(),
+                                             ctypes.c_float(penalty), _stream()))

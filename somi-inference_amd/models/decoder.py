@@ -1,0 +1,81 @@
+"""Builds and runs any :class:`ModelPlan`: embedding, layers in plan order, final norm, head.
+
+Reference: somi_inference/models/qwen2.py:342-386 (embedding, N layers, final
+norm) and somi_inference/models/qwen2_adapter.py:60-62, 95, 146 (head applied to
+the selected rows only).
+"""
+
+from __future__ import annotations
+
+import torch
+
+from ..kernels import ops
+from ..parts.base import FixedStateSpec, LayerCache, PagedKVSpec, Runtime
+from ..parts.registry import build_part
+from ..parts.residual import ResidualStream
+from ..weights.loader import WeightFetcher, check_weights
+from ..weights.source import WeightSource
+from ..weights.spec import WeightSpec
+from .plan import ModelPlan
+
+
+class DecoderModel:
+    def __init__(self, plan: ModelPlan, runtime: Runtime) -> None:
+        self.plan = plan
+        self.runtime = runtime
+        self.embedding = build_part("embedding", plan.embedding, prefix=plan.embedding_prefix)
+        self.layers = [build_part("block", layer.block, prefix=layer.prefix) for layer in plan.layers]
+        self.final_norm = build_part("norm", plan.final_norm, prefix=plan.final_norm_prefix)
+        self.head = build_part("head", plan.head, prefix=plan.head_prefix)
+        self.order = plan.run_order()
+        self.vocab_size = plan.vocab_size or getattr(self.head, "vocab_size")
+        self.loaded = False
+
+    # ------------------------------------------------------------------ weights
+    def weight_specs(self) -> list[WeightSpec]:
+        specs: dict[str, WeightSpec] = {}
+        for part in [self.embedding, *self.layers, self.final_norm, self.head]:
+            for spec in part.weight_specs():
+                specs[spec.name] = spec
+        return list(specs.values())
+
+    def load(self, source: WeightSource) -> None:
+        """Check the source against the declared tensors (one error for everything), then place them."""
+        specs = self.weight_specs()
+        check_weights(specs, source, self.plan.ignore_weights)
+        fetch = WeightFetcher(specs, source, self.runtime.dtype, self.runtime.device)
+        self.embedding.load(fetch, self.runtime)
+        for layer in self.layers:
+            layer.load(fetch, self.runtime)
+        self.final_norm.load(fetch, self.runtime)
+        self.head.load(fetch, self.runtime)
+        if getattr(self.head, "tied", False):
+            self.head.tie(self.embedding)
+        self.loaded = True
+
+    # -------------------------------------------------------------------- cache
+    def cache_needs(self) -> list[PagedKVSpec | FixedStateSpec | int | None]:
+        """For each run of a layer: the cache its mixer needs, the index of the earlier
+        run whose cache it reads, or None."""
+        needs: list[PagedKVSpec | FixedStateSpec | int | None] = []
+        for run, index in enumerate(self.order):
+            if run in self.plan.cache_from:
+                needs.append(self.plan.cache_from[run])
+            else:
+                needs.append(self.layers[index].mixer.cache_spec())
+        return needs
+
+    # ------------------------------------------------------------------ forward
+    def forward(self, step, caches: list[LayerCache | None]) -> torch.Tensor:
+        """Run the step's tokens; float32 logits ``[len(step.logit_rows), vocab]``."""
+        if not self.loaded:
+            raise RuntimeError("model weights are not loaded")
+        h = self.embedding.forward(step.token_ids)
+        stream = ResidualStream(h)
+        for run, index in enumerate(self.order):
+            self.layers[index].forward(stream, step, caches[run])
+        h = stream.settle()
+        if step.num_logit_rows == 0:
+            return torch.empty((0, self.vocab_size), dtype=torch.float32, device=h.device)
+        rows = ops.gather_rows(h, step.logit_rows)
+        return self.head.forward(self.final_norm.forward(rows))

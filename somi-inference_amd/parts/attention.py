@@ -1,0 +1,95 @@
+"""Grouped-query attention over the paged cache.
+
+Reference: somi_inference/models/qwen2.py:252-300 (q/k/v projections with bias,
+o projection without, heads as contiguous head_dim blocks of the projection,
+rotary encoding on q and k before k is cached), :158-186 (causal softmax
+attention, scale head_dim^-0.5, query head h reads key/value head
+h // (nq / nkv)) and somi_inference/core/paged_attention.py:352-413 (the same
+over cache pages).  The reference has one function for whole prompts that never
+reads the cache and one for single decoded tokens; here one kernel contract
+serves any mix: keys and values of the step's tokens are written to their pages
+first, then every token attends over its request's pages up to its own position.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from ..kernels import attention as attention_kernels
+from ..kernels import ops
+from ..weights.spec import MATRIX, VECTOR, WeightSpec
+from .base import Fetch, LayerCache, Mixer, PagedKVSpec, PartSpec, Runtime
+from .linear import Projection
+from .registry import build_part
+
+
+class GroupedQueryAttention(Mixer):
+    def __init__(self, prefix: str, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
+                 position: PartSpec, qkv_bias: bool = True, out_bias: bool = False,
+                 window: int | None = None, scale: float | None = None, shares_cache: bool = False) -> None:
+        super().__init__(prefix)
+        if num_heads % num_kv_heads != 0:
+            # the reference's message (qwen2.py:116-123)
+            raise ValueError(f"num_q_heads ({num_heads}) must be divisible by num_kv_heads ({num_kv_heads})")
+        self.hidden_size, self.num_heads, self.num_kv_heads = int(hidden_size), int(num_heads), int(num_kv_heads)
+        self.head_dim = int(head_dim)
+        self.qkv_bias, self.out_bias = bool(qkv_bias), bool(out_bias)
+        self.window = int(window) if window else None
+        self.scale = float(scale) if scale is not None else self.head_dim ** -0.5
+        self.shares_cache = bool(shares_cache)     # reads the cache another layer writes: no k/v of its own
+        self.position = build_part("position", position, prefix=self.name("rotary_emb"))
+
+    # ------------------------------------------------------------------ weights
+    def _projections(self) -> list[tuple[str, int]]:
+        names = [("q_proj", self.num_heads * self.head_dim)]
+        if not self.shares_cache:
+            names += [("k_proj", self.num_kv_heads * self.head_dim), ("v_proj", self.num_kv_heads * self.head_dim)]
+        return names
+
+    def weight_specs(self) -> list[WeightSpec]:
+        specs = []
+        for proj, width in self._projections():
+            specs.append(WeightSpec(self.name(f"{proj}.weight"), (width, self.hidden_size), MATRIX))
+            if self.qkv_bias:
+                specs.append(WeightSpec(self.name(f"{proj}.bias"), (width,), VECTOR))
+        specs.append(WeightSpec(self.name("o_proj.weight"), (self.hidden_size, self.num_heads * self.head_dim), MATRIX))
+        if self.out_bias:
+            specs.append(WeightSpec(self.name("o_proj.bias"), (self.hidden_size,), VECTOR))
+        return specs + self.position.weight_specs()
+
+    def load(self, fetch: Fetch, runtime: Runtime) -> None:
+        super().load(fetch, runtime)
+        names = [p for p, _ in self._projections()]
+        self.qkv = Projection.stacked(
+            [fetch(self.name(f"{p}.weight")) for p in names],
+            [fetch(self.name(f"{p}.bias")) for p in names] if self.qkv_bias else None)
+        self.out = Projection(fetch(self.name("o_proj.weight")),
+                              fetch(self.name("o_proj.bias")) if self.out_bias else None)
+        self.position.load(fetch, runtime)
+
+    # -------------------------------------------------------------------- cache
+    def cache_spec(self) -> PagedKVSpec | None:
+        if self.shares_cache:
+            return None
+        return PagedKVSpec(self.num_kv_heads, self.head_dim, self.window)
+
+    # ------------------------------------------------------------------ forward
+    def forward(self, x: torch.Tensor, step, cache: LayerCache | None) -> torch.Tensor:
+        if cache is None or cache.k is None:
+            raise ValueError(f"{self.prefix}: attention needs a paged cache")
+        view = step.paged[cache.group]
+        nkv_new = 0 if self.shares_cache else self.num_kv_heads
+        qkv = self.qkv(x)                                   # [N, (nq + 2 nkv) * D]
+        rotation = self.position.rotation_table()
+        if rotation is None:
+            self.position.encode_qk(qkv, step, self.num_heads, nkv_new, self.head_dim)
+            inv_freq, rotary_dim = None, 0
+        else:
+            inv_freq, rotary_dim = rotation
+        ops.rope_kv_store(qkv, step.positions, view.slot_mapping if nkv_new else None, inv_freq, rotary_dim,
+                          self.num_heads, nkv_new, self.head_dim,
+                          cache.k if nkv_new else None, cache.v if nkv_new else None)
+        attended = attention_kernels.paged_attention(
+            qkv, self.num_heads, cache.k, cache.v, view.block_table, step,
+            window=self.window or 0, scale=self.scale)
+        return self.out(attended)
