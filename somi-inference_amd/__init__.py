@@ -9,6 +9,8 @@ mixed batches, a scheduler, sampling, and hand-written HIP kernels for gfx950.
 from . import config as config
 from . import models as _models            # registers the architectures  # noqa: F401
 from .config import ConfigError, EngineConfig, Qwen2Config
+from .entrypoints import LLM
+from .sampling import SamplingParams
 
 __version__ = "0.1.0"
-__all__ = ["ConfigError", "EngineConfig", "Qwen2Config", "config"]
+__all__ = ["ConfigError", "EngineConfig", "LLM", "Qwen2Config", "SamplingParams", "config"]

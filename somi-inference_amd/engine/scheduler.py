@@ -1,0 +1,179 @@
+"""Continuous-batching scheduler with a token budget and prompt portions.
+
+Reference: ``Scheduler`` (somi_inference/core/continuous_batching.py:46-120):
+three queues (waiting FIFO, running, finished), first come first served with
+head-of-line blocking, at most ``max_concurrent`` running, finished requests
+give their pages back before new ones are admitted.  The reference admits a
+request only if the pages of its whole life fit (``ceil((prompt + max_new - 1) /
+block_size)``, :64-67) and then runs the whole prompt at once.
+
+Here a step has a budget of tokens.  Running requests that decode come first
+(one token each), then running requests with prompt left, then new admissions;
+a prompt is cut into portions of at most ``chunk`` tokens, or what is left of
+the budget.  Pages are taken portion by portion, so they can run out:
+
+* a request whose whole life can never fit the pool is refused when it is added;
+* a new request is admitted only if the pages of its first portion are free
+  (the head of the queue blocks those behind it);
+* if a running request cannot get the pages for its next token(s), the most
+  recently admitted running request is preempted: its pages are given back, it
+  returns to the head of the waiting queue and is recomputed from its first
+  token later (prompt and the tokens it already produced).  The oldest running
+  request is never starved, because the admission check above guarantees that
+  it fits the pool alone.
+"""
+
+from __future__ import annotations
+
+from collections import deque
+from dataclasses import dataclass, field
+
+from ..cache.manager import CacheManager
+from .request import Request, RequestStatus
+
+
+class SchedulerError(ValueError):
+    """A request cannot be accepted."""
+
+
+@dataclass
+class ScheduledPortion:
+    request: Request
+    start: int                    # index of the portion's first token in request.all_tokens
+    tokens: list[int]
+    samples: bool                 # the portion reaches the request's last token: its last logits are sampled
+
+
+@dataclass
+class SchedulerOutput:
+    portions: list[ScheduledPortion] = field(default_factory=list)
+    admitted: list[Request] = field(default_factory=list)
+    preempted: list[Request] = field(default_factory=list)
+
+    @property
+    def num_tokens(self) -> int:
+        return sum(len(p.tokens) for p in self.portions)
+
+
+class Scheduler:
+    def __init__(self, cache: CacheManager, *, max_concurrent: int, max_num_batched_tokens: int,
+                 chunk: int | None = None) -> None:
+        if max_concurrent < 1 or max_num_batched_tokens < 1:
+            raise SchedulerError("max_concurrent and max_num_batched_tokens must be >= 1")
+        self.cache = cache
+        self.max_concurrent = int(max_concurrent)
+        self.max_num_batched_tokens = int(max_num_batched_tokens)
+        self.chunk = int(min(chunk or max_num_batched_tokens, max_num_batched_tokens))
+        self.waiting: deque[Request] = deque()
+        self.running: list[Request] = []          # in admission order
+        self.finished: list[Request] = []
+
+    # -------------------------------------------------------------- requests
+    def add_request(self, request: Request) -> None:
+        pages = (request.max_cached_tokens + self.cache.block_size - 1) // self.cache.block_size
+        if pages > self.cache.num_blocks:
+            raise SchedulerError(
+                f"request {request.request_id!r} needs {pages} pages for {request.max_cached_tokens} tokens "
+                f"(prompt {len(request.prompt_tokens)} + max_new_tokens {request.max_new_tokens} - 1), "
+                f"the cache has {self.cache.num_blocks}")
+        request.status = RequestStatus.WAITING
+        self.waiting.append(request)
+
+    def has_unfinished(self) -> bool:
+        return bool(self.waiting) or bool(self.running)
+
+    def drain_finished(self) -> list[Request]:
+        done, self.finished = self.finished, []
+        return done
+
+    def finish(self, request: Request, reason: str) -> None:
+        """Retire a running request now: its pages and state slot are free for the next step."""
+        request.status = RequestStatus.FINISHED
+        request.finish_reason = reason
+        self.running.remove(request)
+        self.cache.free(request.request_id)
+        self.finished.append(request)
+
+    # ------------------------------------------------------------- scheduling
+    def _preempt_newest(self, output: SchedulerOutput) -> Request:
+        victim = self.running.pop()
+        self.cache.free(victim.request_id)
+        victim.status = RequestStatus.WAITING
+        victim.num_computed = 0
+        victim.num_preemptions += 1
+        self.waiting.appendleft(victim)
+        output.preempted.append(victim)
+        output.portions = [p for p in output.portions if p.request is not victim]
+        return victim
+
+    def _fit(self, request: Request, want: int, taken: list[int]) -> int:
+        """Largest portion <= want whose pages are free after what this step already took."""
+        free = [f - t for f, t in zip(self.cache.free_pages(), taken)]
+        count = want
+        while count > 0:
+            need = self.cache.pages_needed(request.request_id, count)
+            if all(n <= f for n, f in zip(need, free)):
+                return count
+            # shrink to the end of the last page that still fits
+            cached = self.cache.num_tokens(request.request_id)
+            pages_ok = min(len(self.cache.page_list(g, request.request_id)) + free[g]
+                           for g in range(len(free)))
+            count = min(count - 1, pages_ok * self.cache.block_size - cached)
+        return 0
+
+    def schedule(self) -> SchedulerOutput:
+        output = SchedulerOutput()
+        budget = self.max_num_batched_tokens
+        taken = [0] * len(self.cache.groups)
+
+        def take(request: Request, count: int) -> None:
+            nonlocal budget
+            need = self.cache.pages_needed(request.request_id, count)
+            for g, n in enumerate(need):
+                taken[g] += n
+            start = request.num_computed
+            tokens = request.all_tokens[start:start + count]
+            output.portions.append(ScheduledPortion(request, start, tokens,
+                                                    samples=start + count == len(request.all_tokens)))
+            budget -= count
+
+        # 1. running requests: those that decode first, then those with prompt left
+        order = [r for r in self.running if r.num_pending == 1] + [r for r in self.running if r.num_pending > 1]
+        for request in order:
+            if request not in self.running or budget <= 0:
+                continue
+            want = min(request.num_pending, self.chunk, budget)
+            while True:
+                count = self._fit(request, want, taken)
+                if count > 0:
+                    take(request, count)
+                    break
+                if self.running[-1] is request and len(self.running) == 1:
+                    raise SchedulerError(
+                        f"request {request.request_id!r} cannot get a page although it runs alone")
+                victim = self._preempt_newest(output)
+                # what the victim had taken in this step is free again: recount
+                budget = self.max_num_batched_tokens - output.num_tokens
+                for g in range(len(taken)):
+                    taken[g] = 0
+                for portion in output.portions:
+                    for g, n in enumerate(self.cache.pages_needed(portion.request.request_id, len(portion.tokens))):
+                        taken[g] += n
+                if victim is request:
+                    break
+
+        # 2. admissions, first come first served; the head of the queue blocks the rest
+        while self.waiting and len(self.running) < self.max_concurrent and budget > 0 and not output.preempted:
+            request = self.waiting[0]
+            self.cache.register(request.request_id)
+            want = min(request.num_pending, self.chunk, budget)
+            count = self._fit(request, want, taken)
+            if count < want:
+                self.cache.free(request.request_id)     # the pages of its first portion are not free: wait
+                break
+            self.waiting.popleft()
+            request.status = RequestStatus.RUNNING
+            self.running.append(request)
+            output.admitted.append(request)
+            take(request, count)
+        return output

@@ -1,0 +1,116 @@
+"""Shared by the tests: tiny configurations, traces and comparisons."""
+
+from __future__ import annotations
+
+import os
+import random
+
+import torch
+
+from somi_inference_amd.config import Qwen2Config
+
+# Three tiny configurations that differ in every size and option.  A and B are the two of the build's
+# baseline (A is the reference's own test model, tests/conftest.py:27-54 of the reference, with another
+# vocabulary); C adds a window on its upper layers, more kv heads and sizes that are no power of two.
+TINY = {
+    "A": dict(config=Qwen2Config(vocab_size=256, hidden_size=64, intermediate_size=128, num_hidden_layers=2,
+                                 num_attention_heads=4, num_key_value_heads=2, head_dim=16, rope_theta=10000.0,
+                                 rms_norm_eps=1e-6, tie_word_embeddings=True),
+              block_size=16, seed=11),
+    "B": dict(config=Qwen2Config(vocab_size=503, hidden_size=192, intermediate_size=512, num_hidden_layers=3,
+                                 num_attention_heads=6, num_key_value_heads=1, head_dim=32, rope_theta=1e6,
+                                 rms_norm_eps=1e-5, tie_word_embeddings=False),
+              block_size=8, seed=22),
+    "C": dict(config=Qwen2Config(vocab_size=301, hidden_size=120, intermediate_size=200, num_hidden_layers=4,
+                                 num_attention_heads=6, num_key_value_heads=3, head_dim=48, rope_theta=5e4,
+                                 rms_norm_eps=3e-6, tie_word_embeddings=False, attention_bias=True,
+                                 use_sliding_window=True, sliding_window=20, max_window_layers=2),
+              block_size=16, seed=33),
+}
+
+# float32 engine against the float32 plain implementation: rounding of sums in another order only.
+F32_TOL = dict(atol=2e-5, rtol=1e-4)
+# bfloat16 engine against the float32 plain implementation (same bfloat16-rounded weights): activations
+# are rounded to 8 bits of mantissa between kernels; logits of the tiny models are of order 1.
+BF16_TOL = dict(atol=3e-2, rtol=3e-2)
+
+
+def write_tiny(name: str, folder: str) -> str:
+    from somi_inference_amd.weights import write_random_model
+    return write_random_model(folder, TINY[name]["config"], seed=TINY[name]["seed"])
+
+
+def token_ids(vocab: int, length: int, seed: int) -> list[int]:
+    gen = torch.Generator().manual_seed(seed)
+    return torch.randint(0, vocab, (length,), generator=gen).tolist()
+
+
+def tolerance(dtype: str) -> dict:
+    return F32_TOL if dtype == "float32" else BF16_TOL
+
+
+def assert_close(got: torch.Tensor, want: torch.Tensor, dtype: str, what: str = "") -> None:
+    tol = tolerance(dtype)
+    got, want = got.float().cpu(), want.float().cpu()
+    assert got.shape == want.shape, f"{what}: shape {tuple(got.shape)} != {tuple(want.shape)}"
+    bad = (got - want).abs() > tol["atol"] + tol["rtol"] * want.abs()
+    if bad.any():
+        row = int(bad.any(dim=-1).nonzero()[0]) if got.dim() == 2 else int(bad.nonzero()[0])
+        raise AssertionError(f"{what}: first wrong row {row}, max abs error {(got - want).abs().max():.3e} "
+                             f"(tolerance {tol})")
+
+
+def make_engine(folder: str, dtype: str, block_size: int, num_blocks: int, max_requests: int = 8):
+    from somi_inference_amd.models import load_model, make_runner
+    model, config = load_model(folder, dtype=dtype)
+    return make_runner(model, block_size=block_size, num_blocks=num_blocks, max_requests=max_requests), config
+
+
+def run_portions(runner, request_id, tokens: list[int], sizes: list[int]) -> torch.Tensor:
+    """Feed ``tokens`` of one request in portions of the given sizes (cycled), wanting every logit."""
+    from somi_inference_amd.engine import StepEntry
+    runner.begin(request_id)
+    outs, at, i = [], 0, 0
+    while at < len(tokens):
+        size = max(1, sizes[i % len(sizes)])
+        portion = tokens[at:at + size]
+        outs.append(runner.step([StepEntry(request_id, portion, list(range(len(portion))))]).cpu())
+        at += len(portion)
+        i += 1
+    runner.end(request_id)
+    return torch.cat(outs)
+
+
+def mixed_trace(requests: dict[str, list[int]], seed: int, max_live: int = 4, portion_sizes=(7, 2, 5, 3, 11, 1)):
+    """A schedule over several requests: up to ``max_live`` live at once, prompt portions of changing
+    size for some beside single tokens of others, requests ending and new ones starting mid-way.
+
+    Yields steps as ``(entries, ends)`` with entries ``[(id, start, count)]``.
+    """
+    rng = random.Random(seed)
+    pending = list(requests)
+    live: dict[str, int] = {}            # id -> tokens fed so far
+    steps = []
+    while pending or live:
+        while pending and len(live) < max_live and (not live or rng.random() < 0.6):
+            live[pending.pop(0)] = 0
+        entries, ends = [], []
+        for rid in list(live):
+            if len(live) > 1 and rng.random() < 0.25:
+                continue                  # a request may sit a step out
+            fed, total = live[rid], len(requests[rid])
+            tail = total - min(32, total // 2)       # the last tokens go one by one
+            if fed >= tail:
+                count = 1
+            else:
+                count = min(rng.choice(portion_sizes), tail - fed)
+                if count == 1 and tail - fed >= 2:
+                    count = 2
+            entries.append((rid, fed, count))
+            live[rid] = fed + count
+            if live[rid] == total:
+                ends.append(rid)
+                del live[rid]
+        if entries:
+            steps.append((entries, ends))
+    return steps

@@ -1,0 +1,205 @@
+"""The scheduler's decisions and the generation loop, with a scripted model (no GPU).
+
+Scenarios follow the reference's tests/core/test_continuous_batching.py (mock runner with scripted
+tokens, :35-75): admission order, a full pool blocks admission, finishing frees before admitting,
+max_concurrent, EOS at the first token, per-request parameters and histories.
+"""
+
+from collections import deque
+
+import pytest
+import torch
+
+from somi_inference_amd.cache import CacheManager
+from somi_inference_amd.engine import Engine, Request, RequestStatus, Scheduler, SchedulerError
+from somi_inference_amd.parts import PagedKVSpec
+from somi_inference_amd.sampling import SamplingParams
+
+
+def make_cache(num_blocks=8, block_size=4, max_requests=8):
+    return CacheManager([PagedKVSpec(1, 8)], block_size=block_size, num_blocks=num_blocks,
+                        max_requests=max_requests, dtype=torch.float32, device="cpu", allocate_tensors=False)
+
+
+class ScriptedRunner:
+    """Stands in for the model step: does the cache bookkeeping and records what it was given."""
+
+    def __init__(self, cache):
+        self.cache = cache
+        self.calls = []
+
+    def step(self, entries):
+        self.calls.append([(e.request_id, list(e.tokens), list(e.want)) for e in entries])
+        for e in entries:
+            self.cache.reserve(e.request_id, len(e.tokens))
+        for e in entries:
+            self.cache.commit(e.request_id, len(e.tokens))
+        self.cache.check_invariants()
+        return torch.zeros((sum(len(e.want) for e in entries), 4))
+
+
+class ScriptedSampler:
+    """Returns the next scripted token of each request (keyed by its seed, which tests set to its id)."""
+
+    def __init__(self, scripts):
+        self.scripts = {k: list(v) for k, v in scripts.items()}
+        self.seen = []
+        self.draws = []
+
+    def sample(self, logits, params, token_histories=None, seeds=None, counters=None):
+        self.seen.append((list(params), [list(h) for h in token_histories], list(counters)))
+        assert logits.shape[0] == len(params)
+        self.draws.extend(zip(seeds, counters))
+        return [self.scripts[s][c] for s, c in zip(seeds, counters)]
+
+
+def request(rid, prompt_len, max_new, **kw):
+    return Request(rid, list(range(100, 100 + prompt_len)), max_new, seed=rid, **kw)
+
+
+def make_engine(cache, scripts, *, max_concurrent=4, budget=64, chunk=None, eos=None):
+    scheduler = Scheduler(cache, max_concurrent=max_concurrent, max_num_batched_tokens=budget, chunk=chunk)
+    runner, sampler = ScriptedRunner(cache), ScriptedSampler(scripts)
+    return Engine(runner, scheduler, sampler, eos), scheduler, runner, sampler
+
+
+def test_three_new_tokens_are_one_prompt_step_and_two_decodes_and_the_pool_is_empty_after():
+    # /root/reference/tests/core/test_continuous_batching.py:231-261
+    cache = make_cache()
+    engine, _, runner, _ = make_engine(cache, {0: [7, 8, 9]})
+    done = engine.run(deque([(0, request(0, 5, 3))]))
+    assert [r.output_tokens for r in done] == [[7, 8, 9]] and done[0].finish_reason == "length"
+    assert runner.calls == [[(0, [100, 101, 102, 103, 104], [4])], [(0, [7], [0])], [(0, [8], [0])]]
+    assert cache.free_pages() == [8] and not cache.live_requests()
+
+
+def test_eos_at_the_first_token_ends_without_decoding_and_is_kept():
+    # /root/reference/tests/core/test_continuous_batching.py:263-281
+    cache = make_cache()
+    engine, _, runner, _ = make_engine(cache, {0: [2, 5]}, eos=2)
+    done = engine.run(deque([(0, request(0, 3, 4))]))
+    assert done[0].output_tokens == [2] and done[0].finish_reason == "eos" and len(runner.calls) == 1
+    assert done[0].status == RequestStatus.FINISHED
+
+
+def test_prompt_is_cut_into_portions_under_the_token_budget_beside_decodes():
+    cache = make_cache(num_blocks=16)
+    engine, _, runner, _ = make_engine(cache, {0: [1, 2, 3, 4], 1: [5, 6]}, budget=8, chunk=7)
+    done = engine.run(deque([(0, request(0, 3, 4)), (1, request(1, 17, 2))]))
+    assert {r.request_id: r.output_tokens for r in done} == {0: [1, 2, 3, 4], 1: [5, 6]}
+    sizes = [[(rid, len(tokens), want) for rid, tokens, want in call] for call in runner.calls]
+    # step 0: request 0's whole prompt; step 1: 0 decodes, 1 gets its first portion of 7 (chunk);
+    # step 2: decode + 7 more; step 3: decode first, then the last 3 prompt tokens, whose last logits are sampled
+    assert sizes[0] == [(0, 3, [2])]
+    assert sizes[1] == [(0, 1, [0]), (1, 7, [])]
+    assert sizes[2] == [(0, 1, [0]), (1, 7, [])]
+    assert sizes[3] == [(0, 1, [0]), (1, 3, [2])]
+    assert all(sum(n for _, n, _ in call) <= 8 for call in sizes)
+    assert sizes[4] == [(1, 1, [0])]
+
+
+def test_first_come_first_served_and_max_concurrent():
+    # /root/reference/tests/core/test_continuous_batching.py:120-156, 209-225
+    cache = make_cache(num_blocks=32)
+    engine, scheduler, runner, _ = make_engine(cache, {i: [1] * 3 for i in range(4)}, max_concurrent=2)
+    for i in range(4):
+        engine.add_request(request(i, 2, 3))
+    engine.step()
+    assert [r.request_id for r in scheduler.running] == [0, 1] and [r.request_id for r in scheduler.waiting] == [2, 3]
+    done = engine.run()
+    assert sorted(r.request_id for r in done) == [0, 1, 2, 3]
+    assert max(len(call) for call in runner.calls) == 2
+
+
+def test_head_of_queue_blocks_those_behind_it_when_its_pages_are_not_free():
+    # /root/reference/tests/core/test_continuous_batching.py:158-207
+    cache = make_cache(num_blocks=4, block_size=4)
+    engine, scheduler, _, _ = make_engine(cache, {0: [1] * 6, 1: [1] * 2, 2: [1] * 2})
+    engine.add_request(request(0, 10, 6))     # 3 pages now, a 4th later
+    engine.add_request(request(1, 8, 2))      # first portion needs 2 pages: does not fit beside request 0
+    engine.add_request(request(2, 2, 2))      # would fit, but must not overtake
+    engine.step()
+    assert [r.request_id for r in scheduler.running] == [0]
+    assert [r.request_id for r in scheduler.waiting] == [1, 2]
+    done = engine.run()
+    assert [r.request_id for r in done] == [0, 1, 2]
+    assert cache.free_pages() == [4]
+
+
+def test_request_that_can_never_fit_is_refused_when_added():
+    cache = make_cache(num_blocks=2, block_size=4)
+    engine, _, _, _ = make_engine(cache, {})
+    with pytest.raises(SchedulerError, match="needs 3 pages"):
+        engine.add_request(request(0, 8, 2))
+    engine.add_request(request(1, 8, 1))       # 8 cached tokens at most: fits exactly
+
+
+def test_when_pages_run_out_the_newest_request_is_preempted_and_recomputed():
+    cache = make_cache(num_blocks=4, block_size=4)
+    scripts = {0: list(range(10, 20)), 1: list(range(30, 40))}
+    engine, scheduler, runner, sampler = make_engine(cache, scripts)
+    engine.add_request(request(0, 6, 7))       # grows to 12 tokens = 3 pages
+    engine.add_request(request(1, 6, 6))       # 2 pages each at first; both want a third at the same step
+    done = engine.run()
+    assert {r.request_id: r.output_tokens for r in done} == {0: scripts[0][:7], 1: scripts[1][:6]}
+    victim = next(r for r in done if r.request_id == 1)
+    assert victim.num_preemptions >= 1
+    # the recomputation feeds prompt and the tokens made so far in one portion and samples at its end
+    recompute = [call for call in runner.calls for rid, tokens, want in call
+                 if rid == 1 and len(tokens) > 6]
+    assert recompute, "request 1 was never recomputed"
+    assert cache.free_pages() == [4] and not cache.live_requests()
+    # a request's random stream goes on where it stopped: every counter 0..5 is drawn exactly once
+    assert [c for s, c in sampler.draws if s == 1] == list(range(6))
+    assert [c for s, c in sampler.draws if s == 0] == list(range(7))
+    assert all(r.finish_reason == "length" for r in done)
+
+
+def test_oldest_request_is_never_the_victim():
+    cache = make_cache(num_blocks=3, block_size=4)
+    engine, scheduler, _, _ = make_engine(cache, {0: [1] * 8, 1: [1] * 8})
+    engine.add_request(request(0, 4, 8))
+    engine.add_request(request(1, 4, 4))
+    done = engine.run()
+    assert next(r for r in done if r.request_id == 0).num_preemptions == 0
+    assert sorted(r.request_id for r in done) == [0, 1]
+
+
+def test_sampler_sees_each_requests_parameters_history_and_counter():
+    # /root/reference/tests/core/test_continuous_batching.py:304-362
+    cache = make_cache(num_blocks=16)
+    engine, _, _, sampler = make_engine(cache, {0: [50, 51], 1: [60, 61]})
+    a = request(0, 3, 2, sampling_params=SamplingParams(temperature=0.0))
+    b = request(1, 2, 2, sampling_params=SamplingParams(temperature=0.8, top_k=5))
+    engine.run(deque([(0, a), (0, b)]))
+    params, histories, counters = sampler.seen[0]
+    assert [p.temperature for p in params] == [0.0, 0.8] and counters == [0, 0]
+    assert histories == [[100, 101, 102], [100, 101]]            # the prompt alone at the first token (model_runner.py:36)
+    params, histories, counters = sampler.seen[1]
+    assert histories == [[100, 101, 102, 50], [100, 101, 60]] and counters == [1, 1]   # prompt + outputs (continuous_batching.py:167)
+
+
+def test_finished_requests_do_not_leak_into_the_next_run():
+    # /root/reference/tests/core/test_continuous_batching.py:283-302
+    cache = make_cache()
+    engine, _, _, _ = make_engine(cache, {0: [1], 1: [2]})
+    assert [r.request_id for r in engine.run(deque([(0, request(0, 2, 1))]))] == [0]
+    assert [r.request_id for r in engine.run(deque([(0, request(1, 2, 1))]))] == [1]
+
+
+def test_arrivals_are_injected_by_step():
+    cache = make_cache(num_blocks=16)
+    engine, _, runner, _ = make_engine(cache, {0: [1] * 4, 1: [2] * 2})
+    engine.run(deque([(0, request(0, 2, 4)), (2, request(1, 2, 2))]))
+    assert [rid for rid, _, _ in runner.calls[0]] == [0] and [rid for rid, _, _ in runner.calls[1]] == [0]
+    assert [rid for rid, _, _ in runner.calls[2]] == [0, 1]
+
+
+def test_bad_requests_are_refused():
+    with pytest.raises(ValueError, match="max_new_tokens"):     # asserted by the reference (continuous_batching.py:34)
+        Request(0, [1], 0)
+    with pytest.raises(ValueError, match="prompt"):
+        Request(0, [], 1)
+    for bad in (dict(temperature=-1.0), dict(top_k=0), dict(top_p=0.0), dict(top_p=1.5), dict(repetition_penalty=0.0)):
+        with pytest.raises(ValueError):                           # reference: sampler.py:20-25
+            SamplingParams(**bad)
