@@ -31,8 +31,12 @@ TINY = {
 # float32 engine against the float32 plain implementation: rounding of sums in another order only.
 F32_TOL = dict(atol=2e-5, rtol=1e-4)
 # bfloat16 engine against the float32 plain implementation (same bfloat16-rounded weights): activations
-# are rounded to 8 bits of mantissa between kernels; logits of the tiny models are of order 1.
-BF16_TOL = dict(atol=3e-2, rtol=3e-2)
+# are rounded to 8 bits of mantissa between kernels; logits of the tiny models are of order 1.  The bound
+# on single elements is the one the reference uses for half precision (atol = rtol = 5e-2,
+# /root/reference/tests/core/test_paged_attention.py:338); rounding noise is random, so on top of it the
+# root mean square error over all logits must stay an order of magnitude below that.
+BF16_TOL = dict(atol=5e-2, rtol=5e-2)
+BF16_RMS = 8e-3
 
 
 def write_tiny(name: str, folder: str) -> str:
@@ -58,6 +62,9 @@ def assert_close(got: torch.Tensor, want: torch.Tensor, dtype: str, what: str = 
         row = int(bad.any(dim=-1).nonzero()[0]) if got.dim() == 2 else int(bad.nonzero()[0])
         raise AssertionError(f"{what}: first wrong row {row}, max abs error {(got - want).abs().max():.3e} "
                              f"(tolerance {tol})")
+    if dtype != "float32":
+        rms = float((got - want).pow(2).mean().sqrt())
+        assert rms < BF16_RMS, f"{what}: root mean square error {rms:.3e} (bound {BF16_RMS})"
 
 
 def make_engine(folder: str, dtype: str, block_size: int, num_blocks: int, max_requests: int = 8):
@@ -114,3 +121,31 @@ def mixed_trace(requests: dict[str, list[int]], seed: int, max_live: int = 4, po
         if entries:
             steps.append((entries, ends))
     return steps
+
+
+def peaky_folder(source: str, target: str, factor: float = 6.0) -> str:
+    """A copy of a model folder whose q and k projections are scaled so that attention scores spread
+    over several units: single keys stand out, and a wrong key, page or window edge changes the logits."""
+    import shutil
+    from safetensors.torch import load_file, save_file
+    os.makedirs(target, exist_ok=True)
+    shutil.copy(os.path.join(source, "config.json"), os.path.join(target, "config.json"))
+    tensors = load_file(os.path.join(source, "model.safetensors"))
+    for name in list(tensors):
+        if ".q_proj." in name or ".k_proj." in name:
+            tensors[name] = (tensors[name].float() * factor).to(tensors[name].dtype)
+    save_file(tensors, os.path.join(target, "model.safetensors"))
+    return target
+
+
+def peak_pages(steps, block_size: int) -> int:
+    """Most pages live requests hold at any time while a mixed trace runs."""
+    held: dict[str, int] = {}
+    peak = 0
+    for entries, ends in steps:
+        for rid, start, count in entries:
+            held[rid] = start + count
+        peak = max(peak, sum((n + block_size - 1) // block_size for n in held.values()))
+        for rid in ends:
+            del held[rid]
+    return peak

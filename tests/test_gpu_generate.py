@@ -1,0 +1,151 @@
+"""Generation through the entry point and the command line: greedy against the plain implementation,
+temperature sampling with a request's own seed, sampler rules on the GPU, and what happens when pages run out."""
+
+import json
+import os
+import subprocess
+import sys
+
+import pytest
+import torch
+
+from helpers import TINY, token_ids
+from plain import qwen2_plain as plain
+from somi_inference_amd import LLM, SamplingParams
+from somi_inference_amd.sampling import Sampler, uniform
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def plain_greedy(folder, prompts, new_tokens):
+    cfg, weights = plain.read_model(folder)
+    return [plain.greedy_generate(cfg, weights, p, new_tokens) for p in prompts], cfg, weights
+
+
+def assert_greedy_matches(got, want, prompts, cfg, weights, exact):
+    for prompt, tokens, expected in zip(prompts, got, want):
+        if tokens == expected:
+            continue
+        assert not exact, f"float32 tokens {tokens} differ from the plain implementation's {expected}"
+        first = next(i for i, (a, b) in enumerate(zip(tokens, expected)) if a != b)
+        logits = plain.model_logits(cfg, weights, prompt + expected[:first])[-1]
+        gap = float(logits[expected[first]] - logits[tokens[first]])
+        assert 0.0 <= gap < 0.03, f"token {tokens[first]} instead of {expected[first]} at {first}: gap {gap}"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_greedy_generation_of_the_small_workload(dtype, model_folders):
+    # prompts of 5, 17 and 33 tokens, 8 greedy tokens each, pages of 16
+    vocab = TINY["A"]["config"].vocab_size
+    prompts = [token_ids(vocab, n, 10 + n) for n in (5, 17, 33)]
+    want, cfg, weights = plain_greedy(model_folders["A"], prompts, 8)
+    llm = LLM(model_folders["A"], dtype=dtype, block_size=16, num_blocks=16, max_concurrent=4, eos_token_id=-1)
+    got = llm.generate(prompts, max_new_tokens=8, temperature=0.0)
+    assert_greedy_matches(got, want, prompts, cfg, weights, exact=dtype == "float32")
+    assert llm.kv_manager.free_pages() == [16]
+    one = llm.generate(prompts[0], max_new_tokens=8, temperature=0.0)       # a single prompt gives a single result
+    assert one == got[0]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_prompts_in_portions_of_seven_beside_decoding(dtype, model_folders):
+    # prompts of 1, 9, 40, 64 and 100 tokens, 12 tokens each, portions of 7 mixed with decoded tokens, pages of 8
+    vocab = TINY["B"]["config"].vocab_size
+    prompts = [token_ids(vocab, n, 20 + n) for n in (1, 9, 40, 64, 100)]
+    want, cfg, weights = plain_greedy(model_folders["B"], prompts, 12)
+    llm = LLM(model_folders["B"], dtype=dtype, block_size=8, num_blocks=64, max_concurrent=5,
+              max_num_batched_tokens=24, max_chunk=7, eos_token_id=-1)
+    got = llm.generate(prompts, max_new_tokens=12, temperature=0.0)
+    assert_greedy_matches(got, want, prompts, cfg, weights, exact=dtype == "float32")
+    assert llm.engine.num_steps > 12                       # the prompts really were cut up
+    # temperature 0.8 with a fixed seed: the same tokens whatever the batch and the portions are
+    sampled = llm.generate(prompts, max_new_tokens=12, temperature=0.8, seed=5)
+    alone = LLM(model_folders["B"], dtype=dtype, block_size=8, num_blocks=64, max_concurrent=1, eos_token_id=-1)
+    for index, prompt in enumerate(prompts):
+        if dtype == "float32":
+            assert alone.generate(prompt, max_new_tokens=12, temperature=0.8, seed=5 + index) == sampled[index]
+    assert sampled != got
+    assert llm.generate(prompts, max_new_tokens=12, temperature=0.8, seed=5) == sampled
+
+
+def test_running_out_of_pages_preempts_and_still_gives_the_same_tokens(model_folders):
+    vocab = TINY["A"]["config"].vocab_size
+    prompts = [token_ids(vocab, n, 30 + n) for n in (30, 28, 25)]
+    roomy = LLM(model_folders["A"], dtype="float32", block_size=16, num_blocks=32, max_concurrent=3, eos_token_id=-1)
+    want = roomy.generate(prompts, max_new_tokens=24, temperature=0.7, seed=1)
+    tight = LLM(model_folders["A"], dtype="float32", block_size=16, num_blocks=7, max_concurrent=3, eos_token_id=-1)
+    got = tight.generate(prompts, max_new_tokens=24, temperature=0.7, seed=1)
+    assert got == want
+    assert tight.kv_manager.free_pages() == [7]
+
+
+def test_eos_ends_a_request_and_is_kept(model_folders):
+    vocab = TINY["A"]["config"].vocab_size
+    prompt = token_ids(vocab, 9, 3)
+    free = LLM(model_folders["A"], dtype="float32", num_blocks=8, eos_token_id=-1).generate(prompt, max_new_tokens=6, temperature=0.0)
+    eos = free[2]
+    stopped = LLM(model_folders["A"], dtype="float32", num_blocks=8, eos_token_id=eos).generate(prompt, max_new_tokens=6, temperature=0.0)
+    assert stopped == free[:free.index(eos) + 1]
+
+
+def test_entry_point_options_and_errors(model_folders):
+    llm = LLM(model_folders["A"], num_blocks=4)
+    assert llm.dtype == "float32"                            # the reference's default dtype (entrypoints/llm.py:66)
+    with pytest.raises(NotImplementedError):                 # reference entrypoints/llm.py:166-170
+        llm.generate_stream("x", max_new_tokens=1)
+    with pytest.raises(ValueError, match="tokenizer"):
+        llm.generate("some text", max_new_tokens=1)
+    with pytest.raises(ValueError, match="max_new_tokens"):
+        llm.generate([1, 2], max_new_tokens=0)
+    with pytest.raises(ValueError, match="pages"):
+        llm.generate(list(range(60)), max_new_tokens=10)
+    with pytest.raises(RuntimeError, match="GPU"):
+        LLM(model_folders["A"], device="cpu")
+
+
+def test_sampler_rules_on_the_gpu():
+    sampler, dev = Sampler(), "cuda:0"
+    t = lambda rows: torch.tensor(rows, dtype=torch.float32, device=dev)
+    greedy = SamplingParams(temperature=0.0)
+    assert sampler.sample(t([[1.0, 3.0, 2.0]]), greedy) == [1]                                     # reference test_sampler.py:58-66
+    assert sampler.sample(t([[2.0, 1.5]]), SamplingParams(temperature=0.0, repetition_penalty=2.0), [[0]]) == [1]   # :85-93
+    assert sampler.sample(t([[-1.0, 0.5, 0.5]]), SamplingParams(temperature=0.0, repetition_penalty=2.0), [[0]])[0] != 0
+    rows = t([[1.0, 2.9, 3.0], [1.0, 2.9, 3.0]])
+    assert sampler.sample(rows, SamplingParams(temperature=0.0, repetition_penalty=1.5), [[2], [1]]) == [1, 2]     # :251-279
+    # temperature 0 ignores top-k and top-p (:131-141)
+    assert sampler.sample(t([[1.0, 5.0, 2.0]]), SamplingParams(temperature=0.0, top_k=1, top_p=0.1)) == [1]
+    # top-k keeps exactly k also under ties; top-p keeps the entry that crosses p (:96-128)
+    for counter in range(50):
+        picked = sampler.sample(t([[5.0, 4.0, 4.0, 1.0]]), SamplingParams(top_k=2), seeds=[3], counters=[counter])[0]
+        assert picked in (0, 1, 2) and picked != 3
+        assert sampler.sample(t([[4.0, 3.0, 2.0, 1.0]]), SamplingParams(top_p=0.5), seeds=[3], counters=[counter]) == [0]
+    # heterogeneous rows in one call (:144-160), and the caller's logits are not modified
+    logits = t([[0.0, 9.0, 1.0], [3.0, 1.0, 2.0]])
+    keep = logits.clone()
+    out = sampler.sample(logits, [SamplingParams(temperature=0.0), SamplingParams(top_k=1, repetition_penalty=3.0)], [[], [1]])
+    assert out == [1, 0] and torch.equal(logits, keep)
+    # the draws follow the softmax: frequencies over the request's own stream
+    probs = torch.softmax(t([1.0, 2.0, 0.5, 3.0]) / 0.8, dim=-1).cpu()
+    n = 3000
+    rows = t([[1.0, 2.0, 0.5, 3.0]]).expand(n, -1).contiguous()
+    picks = torch.tensor(sampler.sample(rows, SamplingParams(temperature=0.8), seeds=[11] * n, counters=list(range(n))))
+    freq = torch.bincount(picks, minlength=4).float() / n
+    assert (freq - probs).abs().max() < 0.03
+    assert 0.0 <= uniform(1, 2) < 1.0 and uniform(1, 2) == uniform(1, 2) != uniform(1, 3)
+
+
+def test_command_line_generates_and_appends_jsonl(model_folders, tmp_path):
+    vocab = TINY["A"]["config"].vocab_size
+    prompt = token_ids(vocab, 6, 1)
+    out_file = tmp_path / "out.jsonl"
+    cmd = [sys.executable, "-m", "somi_inference_amd.entrypoints.cli", "--model-name", model_folders["A"],
+           "--dtype", "float32", "--num-blocks", "8", "--max-new-tokens", "5", "--temperature", "0.0",
+           "--prompt-ids", ",".join(map(str, prompt)), "--output-file", str(out_file)]
+    done = subprocess.run(cmd, cwd=ROOT, capture_output=True, text=True, timeout=300)
+    assert done.returncode == 0, done.stderr[-2000:]
+    record = json.loads(done.stdout.strip().splitlines()[-1])
+    cfg, weights = plain.read_model(model_folders["A"])
+    want = plain.greedy_generate(cfg, weights, prompt, 5, eos=cfg.get("eos_token_id"))
+    assert record["prompt"] == prompt and record["output"] == want
+    assert json.loads(out_file.read_text().strip()) == record

@@ -1,0 +1,219 @@
+"""Each HIP kernel alone against a plain float32 torch reference of the same op, at sizes other than
+the tiny models' (odd widths, many heads and groups, page sizes, tails)."""
+
+import math
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from plain import qwen2_plain as plain
+from somi_inference_amd.kernels import KernelError, ops
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+DT = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+TOL = {"float32": dict(atol=1e-5, rtol=1e-5), "bfloat16": dict(atol=2e-2, rtol=2e-2)}
+
+
+def rnd(*shape, dtype="float32", seed=0, scale=1.0):
+    gen = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=gen) * scale).to(DT[dtype]).to(DEV)
+
+
+def i32(values):
+    return torch.tensor(values, dtype=torch.int32, device=DEV)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_embedding_gathers_rows_as_float32(dtype):
+    table = rnd(301, 72, dtype=dtype)
+    ids = i32([0, 300, 17, 17, 5])
+    out = ops.embedding(table, ids)
+    assert out.dtype == torch.float32
+    assert torch.equal(out, table.float()[ids.long()])
+    assert torch.equal(ops.gather_rows(out, i32([4, 0])), out[[4, 0]])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("hidden", [8, 200, 3584 + 24])
+def test_rmsnorm_and_the_fused_residual_add(dtype, hidden):
+    h = rnd(5, hidden, seed=1) + 0.5
+    w = rnd(hidden, seed=2) + 1.0
+    for eps in (1e-6, 0.1):
+        out = ops.rmsnorm(h.clone(), w, eps, DT[dtype])
+        torch.testing.assert_close(out.float(), F.rms_norm(h, (hidden,), w, eps), **TOL[dtype])
+    delta = rnd(5, hidden, dtype=dtype, seed=3)
+    h2 = h.clone()
+    out = ops.rmsnorm(h2, w, 1e-5, DT[dtype], delta=delta)
+    torch.testing.assert_close(h2, h + delta.float(), atol=1e-6, rtol=1e-6)       # the sum itself is float32
+    torch.testing.assert_close(out.float(), F.rms_norm(h + delta.float(), (hidden,), w, 1e-5), **TOL[dtype])
+    h3 = h.clone()
+    ops.residual_add(h3, delta)
+    assert torch.equal(h3, h2)
+    # the reference's vector: [1,2,3,4], eps 0 -> x / sqrt(7.5) (tests/models/test_qwen2.py:18-26)
+    x = torch.tensor([[1.0, 2.0, 3.0, 4.0]], device=DEV)
+    torch.testing.assert_close(ops.rmsnorm(x, torch.ones(4, device=DEV), 0.0, torch.float32), x / math.sqrt(7.5))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("m, n, k", [(1, 503, 192), (7, 64, 65), (65, 130, 17), (130, 33, 1000)])
+def test_linear_plain_with_bias_and_tails(dtype, m, n, k):
+    x, w, b = rnd(m, k, dtype=dtype, seed=1), rnd(n, k, dtype=dtype, seed=2, scale=0.1), rnd(n, seed=3)
+    want = F.linear(x.float(), w.float(), b)
+    torch.testing.assert_close(ops.linear_plain(x, w, b).float(), want, **TOL[dtype])
+    torch.testing.assert_close(ops.linear_plain(x, w, None, torch.float32), F.linear(x.float(), w.float()),
+                               atol=1e-4, rtol=1e-4)
+    # a row's result does not depend on how many rows are in the launch
+    assert torch.equal(ops.linear_plain(x[:1].contiguous(), w, b), ops.linear_plain(x, w, b)[:1])
+    with pytest.raises(KernelError, match="features"):
+        ops.linear_plain(x, rnd(n, k + 1, dtype=dtype))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("nq, nkv, d, page", [(4, 2, 16, 16), (12, 2, 48, 8), (8, 1, 80, 4), (3, 3, 128, 32)])
+def test_rope_and_cache_write(dtype, nq, nkv, d, page):
+    n, pages, theta = 9, 6, 1e4
+    qkv = rnd(n, (nq + 2 * nkv) * d, dtype=dtype, seed=4)
+    positions = i32([0, 1, 2, 3, 40, 41, 7, 1000, 5])
+    slot_list = [page * 5 + 1, page * 5 + 2, 3, 0, page * 2, page * 2 + 1, page * 4 - 1, page * 3, 2]
+    if page < 4:
+        pytest.skip("needs distinct slots")
+    slots = i32(slot_list)
+    kc = torch.zeros(pages, nkv, page, d, dtype=DT[dtype], device=DEV)
+    vc = torch.zeros_like(kc)
+    inv_freq = plain.rope_inv_freq(d, theta).to(DEV)
+    before = qkv.clone()
+    ops.rope_kv_store(qkv, positions, slots, inv_freq, d, nq, nkv, d, kc, vc)
+    heads = before.float().view(n, nq + 2 * nkv, d).cpu()
+    cos, sin = plain.rope_cos_sin(positions.cpu(), d, theta)
+    want_q = plain.apply_rope(heads[:, :nq].transpose(0, 1), cos, sin).transpose(0, 1)
+    want_k = plain.apply_rope(heads[:, nq:nq + nkv].transpose(0, 1), cos, sin).transpose(0, 1)
+    tol = dict(atol=1e-5, rtol=1e-5) if dtype == "float32" else dict(atol=2e-2, rtol=2e-2)
+    torch.testing.assert_close(qkv.float().view(n, -1, d)[:, :nq].cpu(), want_q, **tol)
+    for t, slot in enumerate(slot_list):
+        pg, off = divmod(slot, page)
+        torch.testing.assert_close(kc[pg, :, off].float().cpu(), want_k[t], **tol)
+        assert torch.equal(vc[pg, :, off].cpu(), before.view(n, -1, d)[t, nq + nkv:].cpu())
+    written = torch.zeros(pages * page, dtype=torch.bool)
+    written[slot_list] = True
+    untouched = kc.float().permute(0, 2, 1, 3).reshape(pages * page, -1).cpu()[~written]
+    assert float(untouched.abs().sum()) == 0.0, "a slot that was not addressed was written"
+    # no rotation table: q unchanged, k and v stored as they are
+    qkv2 = before.clone()
+    ops.rope_kv_store(qkv2, positions, slots, None, 0, nq, nkv, d, kc, vc)
+    assert torch.equal(qkv2, before)
+    assert torch.equal(kc[slot_list[0] // page, :, slot_list[0] % page], before.view(n, -1, d)[0, nq:nq + nkv])
+
+
+def dense_attention_reference(q, keys, values, positions, lens_before, window, scale):
+    """q: [N, nq, D] of one request laid out after its cached tokens; keys/values: [L, nkv, D]."""
+    nq, nkv = q.shape[1], keys.shape[1]
+    out = torch.zeros_like(q)
+    for t in range(q.shape[0]):
+        p = positions[t]
+        lo = max(0, p - window + 1) if window else 0
+        k = keys[lo:p + 1].repeat_interleave(nq // nkv, dim=1)
+        v = values[lo:p + 1].repeat_interleave(nq // nkv, dim=1)
+        scores = torch.einsum("hd,lhd->hl", q[t], k) * scale
+        out[t] = torch.einsum("hl,lhd->hd", torch.softmax(scores, dim=-1), v)
+    return out
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("nq, nkv, d, page, window", [
+    (8, 4, 32, 4, 0),          # the reference's microbenchmark shape (benchmarks/bench_paged_attention.py:88-104)
+    (12, 2, 64, 16, 0), (8, 1, 48, 8, 0), (6, 3, 128, 16, 37), (5, 5, 16, 3, 5), (14, 2, 256, 16, 0)])
+def test_paged_attention_over_permuted_pages_for_portions_and_single_tokens(dtype, nq, nkv, d, page, window):
+    # two requests: one brings a portion of 9 tokens after 30 cached ones, one a single token after 200
+    cached, new = [30, 200], [9, 1]
+    total = [c + n for c, n in zip(cached, new)]
+    n_pages = sum((t + page - 1) // page for t in total) + 3
+    perm = torch.randperm(n_pages, generator=torch.Generator().manual_seed(3)).tolist()
+    tables, at = [], 0
+    for t in total:
+        count = (t + page - 1) // page
+        tables.append(perm[at:at + count])
+        at += count
+    width = max(len(t) for t in tables)
+    block_table = i32([t + [0] * (width - len(t)) for t in tables])
+    keys = [rnd(t, nkv, d, dtype=dtype, seed=10 + i) for i, t in enumerate(total)]
+    values = [rnd(t, nkv, d, dtype=dtype, seed=20 + i) for i, t in enumerate(total)]
+    kc = rnd(n_pages, nkv, page, d, dtype=dtype, seed=99)      # garbage everywhere else must be inert
+    vc = rnd(n_pages, nkv, page, d, dtype=dtype, seed=98)      # (reference tests/core/test_paged_attention.py:243-256)
+    for r, t in enumerate(total):
+        for pos in range(t):
+            kc[tables[r][pos // page], :, pos % page] = keys[r][pos]
+            vc[tables[r][pos // page], :, pos % page] = values[r][pos]
+    n = sum(new)
+    q = rnd(n, nq * d, dtype=dtype, seed=5, scale=2.0)
+    positions = [cached[0] + i for i in range(new[0])] + [cached[1]]
+    entry = [0] * new[0] + [1]
+    scale = d ** -0.5
+    out = ops.paged_attention_plain(q, nq * d, kc, vc, block_table, i32(entry), i32(positions), nq, window, scale)
+    qh = q.float().view(n, nq, d).cpu()
+    want = torch.cat([
+        dense_attention_reference(qh[:new[0]], keys[0].float().cpu(), values[0].float().cpu(), positions[:new[0]], cached[0], window, scale),
+        dense_attention_reference(qh[new[0]:], keys[1].float().cpu(), values[1].float().cpu(), positions[new[0]:], cached[1], window, scale)])
+    tol = dict(atol=2e-5, rtol=1e-4) if dtype == "float32" else dict(atol=2e-2, rtol=2e-2)
+    torch.testing.assert_close(out.float().view(n, nq, d).cpu(), want, **tol)
+
+
+def test_paged_attention_refuses_what_it_cannot_do():
+    q = rnd(1, 5 * 16)
+    kc = rnd(2, 2, 4, 16)
+    with pytest.raises(KernelError, match="divisible"):      # reference: AssertionError on bad GQA (tests/core/test_paged_attention.py:340-350)
+        ops.paged_attention_plain(q, 80, kc, kc.clone(), i32([[0]]), i32([0]), i32([0]), 5, 0, 0.25)
+    big = rnd(1, 2 * 272)
+    kc2 = rnd(2, 2, 4, 272)
+    with pytest.raises(KernelError, match="head_dim"):
+        ops.paged_attention_plain(big, 544, kc2, kc2.clone(), i32([[0]]), i32([0]), i32([0]), 2, 0, 0.1)
+    with pytest.raises(KernelError, match="GPU"):
+        ops.silu_mul(torch.zeros(2, 4))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_silu_mul(dtype):
+    gu = rnd(7, 2 * 203, dtype=dtype, seed=6, scale=3.0)
+    want = F.silu(gu.float()[:, :203]) * gu.float()[:, 203:]
+    torch.testing.assert_close(ops.silu_mul(gu).float(), want, **TOL[dtype])
+    # the reference's vector: gate = up = 10 -> silu(10) * 10 (tests/models/test_qwen2_mlp.py:22-39)
+    ten = torch.full((1, 2), 10.0, device=DEV)
+    assert ops.silu_mul(ten).item() == pytest.approx(10.0 / (1 + math.exp(-10.0)) * 10.0, rel=1e-6)
+
+
+def test_sample_greedy_takes_the_first_maximum():
+    logits = torch.tensor([[1.0, 3.0, 2.0], [5.0, 5.0, 4.0], [-1.0, -3.0, -1.0]], device=DEV)   # reference test_sampler.py:58-66
+    zero = torch.zeros(3, device=DEV)
+    assert ops.sample(logits, zero, zero).tolist() == [1, 0, 0]
+    wide = rnd(4, 152064 // 8 + 5, seed=8)
+    assert ops.sample(wide, torch.zeros(4, device=DEV), torch.zeros(4, device=DEV)).tolist() == wide.argmax(-1).tolist()
+
+
+def test_sample_draws_by_inverse_cdf_of_the_softmax():
+    logits = torch.tensor([[0.0, math.log(2.0), math.log(3.0), -float("inf"), math.log(2.0)]], device=DEV)
+    temp = torch.ones(1, device=DEV)
+    edges = torch.tensor([1, 3, 6, 6, 8]) / 8.0             # cumulative probabilities 1/8, 3/8, 6/8, 6/8, 1
+    for u, want in [(0.0, 0), (0.124, 0), (0.126, 1), (0.374, 1), (0.376, 2), (0.749, 2), (0.751, 4), (0.999999, 4)]:
+        got = ops.sample(logits, temp, torch.tensor([u], device=DEV)).item()
+        assert got == want, f"u={u}: token {got}, expected {want} (edges {edges.tolist()})"
+    # temperature sharpens: at T = 0.5 probabilities are proportional to 1, 4, 9, 0, 4 (of 18)
+    half = torch.full((1,), 0.5, device=DEV)
+    assert ops.sample(logits, half, torch.tensor([1.5 / 18], device=DEV)).item() == 1
+    assert ops.sample(logits, half, torch.tensor([5.5 / 18], device=DEV)).item() == 2
+    # a wide row: the empirical distribution of many uniform draws matches the softmax
+    wide = rnd(1, 1237, seed=9, scale=2.0)
+    probs = torch.softmax(wide[0].float() / 0.8, dim=-1).cpu()
+    us = torch.rand(4000, generator=torch.Generator().manual_seed(1))
+    rows = wide.expand(4000, -1).contiguous()
+    picks = ops.sample(rows, torch.full((4000,), 0.8, device=DEV), us.to(DEV)).cpu().long()
+    want = torch.searchsorted(torch.cumsum(probs.double(), 0), us.double()).clamp(max=1236)
+    assert (picks == want).float().mean() > 0.995          # equal up to float32 rounding at bucket edges
+
+
+def test_repetition_penalty_rule():
+    row = torch.tensor([2.0, 1.5, -1.0, 0.5], device=DEV)   # reference test_sampler.py:85-93, 251-263
+    ops.repetition_penalty(row, i32([0, 2]), 2.0)
+    assert row.tolist() == [1.0, 1.5, -2.0, 0.5]
+    with pytest.raises(KernelError, match="penalty"):
+        ops.repetition_penalty(row, i32([0]), 0.0)

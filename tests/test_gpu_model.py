@@ -1,0 +1,173 @@
+"""The engine against the plain implementation, for every way of cutting the work, in float32 and bfloat16."""
+
+import pytest
+import torch
+
+from helpers import (TINY, assert_close, make_engine, mixed_trace, peak_pages, peaky_folder, run_portions,
+                     token_ids)
+from plain import qwen2_plain as plain
+from somi_inference_amd.cache import OutOfPages
+from somi_inference_amd.engine import StepEntry, StepError
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = ["float32", "bfloat16"]
+NAMES = list(TINY)
+
+
+@pytest.fixture(scope="module")
+def peaky_folders(model_folders, tmp_path_factory):
+    root = tmp_path_factory.mktemp("peaky")
+    return {name: peaky_folder(folder, str(root / name)) for name, folder in model_folders.items()}
+
+
+@pytest.fixture(scope="module")
+def oracle(model_folders, peaky_folders):
+    """Plain logits of (folder kind, config name, token tuple), computed once."""
+    cache = {}
+
+    def get(kind: str, name: str, tokens: list[int]) -> torch.Tensor:
+        key = (kind, name, tuple(tokens))
+        if key not in cache:
+            folder = (model_folders if kind == "plain" else peaky_folders)[name]
+            cfg, weights = plain.read_model(folder)
+            cache[key] = plain.model_logits(cfg, weights, tokens)
+        return cache[key]
+    return get
+
+
+def folder_of(kind, name, model_folders, peaky_folders):
+    return (model_folders if kind == "plain" else peaky_folders)[name]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", NAMES)
+@pytest.mark.parametrize("kind", ["plain", "peaky"])
+def test_each_request_alone_and_whole(kind, name, dtype, model_folders, peaky_folders, oracle):
+    vocab, bs = TINY[name]["config"].vocab_size, TINY[name]["block_size"]
+    runner, _ = make_engine(folder_of(kind, name, model_folders, peaky_folders), dtype, bs, 64)
+    for length, seed in ((1, 1), (5, 2), (17, 3), (33, 4), (64, 5), (100, 6), (257, 7)):
+        tokens = token_ids(vocab, length, seed)
+        got = run_portions(runner, f"r{length}", tokens, [length])
+        assert_close(got, oracle(kind, name, tokens), dtype, f"{name} {dtype} whole prompt of {length}")
+    runner.cache.check_invariants()
+    assert runner.cache.free_pages() == [64] * len(runner.cache.groups)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", NAMES)
+def test_most_in_one_step_then_the_last_32_one_by_one(name, dtype, peaky_folders, oracle):
+    vocab, bs = TINY[name]["config"].vocab_size, TINY[name]["block_size"]
+    runner, _ = make_engine(peaky_folders[name], dtype, bs, 32)
+    for length in (45, 130):
+        tokens = token_ids(vocab, length, 40 + length)
+        got = run_portions(runner, "d", tokens, [length - 32] + [1] * 32)
+        want = oracle("peaky", name, tokens)
+        assert_close(got, want, dtype, f"{name} {dtype} prefill {length - 32} + 32 decoded")
+        if dtype == "float32":
+            whole = run_portions(runner, "w", tokens, [length])
+            assert torch.equal(got, whole), "float32 logits differ between decoding and the whole prompt"
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", NAMES)
+def test_portions_of_changing_size_down_to_two_tokens(name, dtype, peaky_folders, oracle):
+    vocab, bs = TINY[name]["config"].vocab_size, TINY[name]["block_size"]
+    runner, _ = make_engine(peaky_folders[name], dtype, bs, 32)
+    tokens = token_ids(vocab, 150, 77)
+    want = oracle("peaky", name, tokens)
+    whole = run_portions(runner, "w", tokens, [150])
+    for sizes in ([7, 2, 5, 3, 11, 2, 16, 2, 29], [2], [bs, bs + 1, bs - 1, 2 * bs], [3, 64, 2, 50]):
+        got = run_portions(runner, "c", tokens, sizes)
+        assert_close(got, want, dtype, f"{name} {dtype} portions {sizes}")
+        if dtype == "float32":
+            assert torch.equal(got, whole), f"float32 logits depend on the portions {sizes}"
+        else:
+            assert (got - whole).abs().max() < 2e-2, f"bfloat16 logits depend on the portions {sizes} beyond rounding"
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", NAMES)
+def test_mixed_batches_with_so_few_pages_that_they_are_used_again(name, dtype, peaky_folders, oracle):
+    vocab, bs = TINY[name]["config"].vocab_size, TINY[name]["block_size"]
+    lengths = {"a": 70, "b": 45, "c": 100, "d": 33, "e": 64, "f": 90, "g": 2, "h": 51}
+    requests = {rid: token_ids(vocab, n, 100 + i) for i, (rid, n) in enumerate(lengths.items())}
+    steps = mixed_trace(requests, seed=5)
+    pages = peak_pages(steps, bs)
+    assert pages < sum((n + bs - 1) // bs for n in lengths.values()), "the trace does not force pages to be used again"
+    runner, _ = make_engine(peaky_folders[name], dtype, bs, pages, max_requests=4)
+    rows = {rid: [] for rid in requests}
+    seen_pages = set()
+    reused = False
+    for entries, ends in steps:
+        batch = []
+        for rid, start, count in entries:
+            if not runner.cache.has(rid):
+                runner.begin(rid)
+            batch.append(StepEntry(rid, requests[rid][start:start + count], list(range(count))))
+        logits = runner.step(batch).cpu()
+        at = 0
+        for rid, start, count in entries:
+            rows[rid].append(logits[at:at + count])
+            at += count
+        for rid in ends:
+            held = set(p for p in runner.cache.page_list(0, rid) if p >= 0)
+            reused = reused or bool(held & seen_pages)
+            seen_pages |= held
+            runner.end(rid)
+        runner.cache.check_invariants()
+    assert reused, "no page was used by two requests"
+    for rid, tokens in requests.items():
+        assert_close(torch.cat(rows[rid]), oracle("peaky", name, tokens), dtype, f"{name} {dtype} mixed request {rid}")
+    assert runner.cache.free_pages() == [pages] * len(runner.cache.groups)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["B", "C"])
+def test_long_decoding_from_a_short_prompt(name, dtype, peaky_folders, oracle):
+    vocab, bs = TINY[name]["config"].vocab_size, TINY[name]["block_size"]
+    runner, _ = make_engine(peaky_folders[name], dtype, bs, 64)
+    tokens = token_ids(vocab, 300, 9)
+    got = run_portions(runner, "l", tokens, [3] + [1] * 297)
+    assert_close(got, oracle("peaky", name, tokens), dtype, f"{name} {dtype} 297 tokens decoded one by one")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", NAMES)
+def test_the_first_tokens_of_a_sequence(name, dtype, model_folders, oracle):
+    vocab, bs = TINY[name]["config"].vocab_size, TINY[name]["block_size"]
+    runner, _ = make_engine(model_folders[name], dtype, bs, 8)
+    tokens = token_ids(vocab, 4, 3)
+    want = oracle("plain", name, tokens)
+    assert_close(run_portions(runner, "x", tokens[:1], [1]), want[:1], dtype, "a prompt of one token")
+    assert_close(run_portions(runner, "y", tokens, [1, 1, 2]), want, dtype, "token by token from the start")
+    # only the wanted places come back, in the order asked for
+    runner.begin("z")
+    got = runner.step([StepEntry("z", tokens, [3, 0])]).cpu()
+    runner.end("z")
+    assert_close(got, want[[3, 0]], dtype, "wanted places")
+    runner.begin("n")
+    assert runner.step([StepEntry("n", tokens, [])]).shape == (0, vocab)
+    runner.end("n")
+
+
+def test_step_contract_errors(model_folders):
+    runner, config = make_engine(model_folders["A"], "float32", 16, 2)
+    with pytest.raises(StepError, match="not live"):
+        runner.step([StepEntry("q", [1], [0])])
+    runner.begin("q")
+    with pytest.raises(StepError, match="outside"):        # out-of-range ids raise, as in the reference
+        runner.step([StepEntry("q", [config.vocab_size], [0])])
+    with pytest.raises(StepError, match="outside"):
+        runner.step([StepEntry("q", [-1], [0])])
+    with pytest.raises(StepError, match="wanted place"):
+        runner.step([StepEntry("q", [1, 2], [2])])
+    with pytest.raises(StepError, match="twice"):
+        runner.step([StepEntry("q", [1], [0]), StepEntry("q", [2], [0])])
+    with pytest.raises(StepError, match="at least one token"):
+        runner.step([StepEntry("q", [], [])])
+    before = runner.cache.free_pages()
+    with pytest.raises(OutOfPages):
+        runner.step([StepEntry("q", [1] * 33, [0])])       # 3 pages, the pool has 2
+    assert runner.cache.free_pages() == before and runner.cache.num_tokens("q") == 0
+    assert runner.step([StepEntry("q", [1] * 32, [31])]).shape == (1, config.vocab_size)
