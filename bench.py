@@ -1,0 +1,199 @@
+"""Decode and prefill throughput of the engine at Qwen2.5-7B layer sizes on one MI355X.
+
+``python bench.py --gpus 1 --steps K --warmup W`` builds a random-weights model of the 7B layer
+sizes in bfloat16, fills the cache of ``--batch`` requests by running their prompts through the
+engine's own step function, then times exactly K decode steps (one token per request per step:
+model step plus greedy sampling) between two synchronisations.  It prints ONE JSON line; ``value``
+is decoded tokens per second.  The same line carries a 2,048-token prefill measurement, the decode
+step's HBM roofline figures and decode throughput at batch 1 and 64.
+
+The method follows the reference's benchmarks (warm-up, synchronise, wall clock, synchronise:
+benchmarks/common.py:131-156; tokens/s = batch * iterations / time: benchmarks/bench_decode.py:241-247)
+with seeded random weights and seeded uniform token ids in place of a downloaded checkpoint and a
+tokenizer-built workload.  The engine runs on one GPU; for more it says so and exits with 2.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E bandwidth
+PEAK_FLOPS = {"bfloat16": 2.5e15, "float32": 157.3e12}   # dense MFMA peaks
+
+
+def parse_args() -> argparse.Namespace:
+    p = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    p.add_argument("--gpus", type=int, default=1)
+    p.add_argument("--steps", type=int, default=64)
+    p.add_argument("--warmup", type=int, default=8)
+    p.add_argument("--batch", type=int, default=8)
+    p.add_argument("--context", type=int, default=4096, help="context length the timed decode steps end at")
+    p.add_argument("--layers", type=int, default=None, help="run fewer layers than the configuration has")
+    p.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    p.add_argument("--block-size", type=int, default=16)
+    p.add_argument("--prefill-tokens", type=int, default=2048)
+    p.add_argument("--seed", type=int, default=0)
+    p.add_argument("--no-points", action="store_true", help="skip the batch 1 / batch 64 decode points")
+    p.add_argument("--no-prefill", action="store_true", help="skip the prefill measurement")
+    return p.parse_args()
+
+
+def main() -> int:
+    args = parse_args()
+    world = int(os.environ.get("WORLD_SIZE", "1"))
+    if args.gpus != 1 or world != 1:
+        if int(os.environ.get("RANK", "0")) == 0:
+            print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} (WORLD_SIZE {world}) is not supported")
+        return 2
+
+    import torch
+
+    from somi_inference_amd.config import Qwen2Config
+    from somi_inference_amd.engine import StepEntry
+    from somi_inference_amd.models import make_runner, random_model
+    from somi_inference_amd.sampling import Sampler, SamplingParams
+
+    full_layers = 28
+    layers = args.layers or full_layers
+    config = Qwen2Config(vocab_size=152064, hidden_size=3584, intermediate_size=18944, num_hidden_layers=layers,
+                         num_attention_heads=28, num_key_value_heads=4, head_dim=128, rope_theta=1e6,
+                         rms_norm_eps=1e-6, tie_word_embeddings=False, max_position_embeddings=32768)
+    torch.manual_seed(args.seed)
+    model = random_model(config, seed=args.seed, dtype=args.dtype)
+    elem = 2 if args.dtype == "bfloat16" else 4
+    batches = [args.batch] if args.no_points else sorted({1, args.batch, 64})
+    pages_per_request = (args.context + args.block_size - 1) // args.block_size + 1
+    num_blocks = max(max(batches) * pages_per_request,
+                     (args.prefill_tokens + args.block_size - 1) // args.block_size + 1)
+    runner = make_runner(model, block_size=args.block_size, num_blocks=num_blocks, max_requests=max(batches) + 1)
+    sampler, greedy = Sampler(), SamplingParams(temperature=0.0)
+    gen = torch.Generator().manual_seed(args.seed)
+
+    weight_bytes = sum(t.numel() * t.element_size() for t in _decode_weights(model))
+    kv_bytes_per_token = 2 * config.num_key_value_heads * config.head_dim * elem * layers
+
+    def sync() -> None:
+        torch.cuda.synchronize()
+
+    def decode_run(batch: int, steps: int, warmup: int) -> tuple[float, float]:
+        """Fill ``batch`` requests up to context - (warmup + steps), then time ``steps`` decode steps.
+        Returns (seconds, mean context length during the timed steps)."""
+        prompt_len = args.context - (warmup + steps)
+        ids = [f"b{batch}_{i}" for i in range(batch)]
+        for rid in ids:
+            runner.begin(rid)
+            tokens = torch.randint(0, config.vocab_size, (prompt_len,), generator=gen).tolist()
+            for at in range(0, prompt_len, 2048):
+                runner.step([StepEntry(rid, tokens[at:at + 2048], [])])
+        last = torch.randint(0, config.vocab_size, (batch,), generator=gen).tolist()
+
+        def one_step(tokens: list[int]) -> list[int]:
+            logits = runner.step([StepEntry(rid, [tok], [0]) for rid, tok in zip(ids, tokens)])
+            return sampler.sample(logits, greedy)
+
+        for _ in range(warmup):
+            last = one_step(last)
+        sync()
+        start = time.perf_counter()
+        for _ in range(steps):
+            last = one_step(last)
+        sync()
+        seconds = time.perf_counter() - start
+        for rid in ids:
+            runner.end(rid)
+        return seconds, args.context - steps / 2.0
+
+    results = {}
+    for batch in batches:
+        steps = args.steps if batch == args.batch else max(8, args.steps // 2)
+        warmup = args.warmup if batch == args.batch else max(2, args.warmup // 2)
+        seconds, mean_ctx = decode_run(batch, steps, warmup)
+        results[batch] = dict(tok_s=batch * steps / seconds, ms=1000.0 * seconds / steps, steps=steps,
+                              warmup=warmup, mean_ctx=mean_ctx)
+
+    main_run = results[args.batch]
+    step_bytes = weight_bytes + args.batch * main_run["mean_ctx"] * kv_bytes_per_token
+    achieved = step_bytes / (main_run["ms"] / 1000.0) / 1e9
+
+    prefill = None
+    if not args.no_prefill:
+        tokens = torch.randint(0, config.vocab_size, (args.prefill_tokens,), generator=gen).tolist()
+        times = []
+        for rep in range(4):
+            runner.begin("prefill")
+            sync()
+            start = time.perf_counter()
+            runner.step([StepEntry("prefill", tokens, [len(tokens) - 1])])
+            sync()
+            times.append(time.perf_counter() - start)
+            runner.end("prefill")
+        seconds = min(times[1:])
+        flops = _prefill_flops(config, args.prefill_tokens)
+        prefill = {"value": round(args.prefill_tokens / seconds, 1), "tokens": args.prefill_tokens,
+                   "ms": round(seconds * 1000.0, 3), "frac": round(flops / seconds / PEAK_FLOPS[args.dtype], 4)}
+
+    line = {
+        "metric": "decode tok/s at batch 8, Qwen2.5-7B layer sizes (plus prefill tok/s at 2,048 tokens, batch 1/64 points)",
+        "value": round(main_run["tok_s"], 2), "unit": "tokens/s", "n_gpus": 1,
+        "steps": main_run["steps"], "warmup": main_run["warmup"], "ms_per_step": round(main_run["ms"], 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+        "data": "synthetic: seeded random N(0,0.02) weights, seeded uniform token ids; caches filled by running the prompts",
+        "config": {"model": "Qwen2.5-7B layer sizes (random weights)", "global_batch": args.batch,
+                   "seq_len": args.context, "parallelism": "single GPU", "layers": layers,
+                   "layers_of_config": full_layers, "hidden_size": config.hidden_size,
+                   "intermediate_size": config.intermediate_size, "num_attention_heads": config.num_attention_heads,
+                   "num_key_value_heads": config.num_key_value_heads, "head_dim": config.head_dim,
+                   "vocab_size": config.vocab_size, "tie_word_embeddings": False, "block_size": args.block_size,
+                   "context_at_end": args.context},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4)},
+        "points": {f"decode_b{b}": round(r["tok_s"], 2) for b, r in results.items() if b in (1, 64)},
+    }
+    if prefill is not None:
+        line["prefill"] = prefill
+    print(json.dumps(line))
+    return 0
+
+
+def _decode_weights(model):
+    """Every weight a decode step reads once: all layers' matrices, norms, biases and the head
+    (the embedding table is touched for one row per request only)."""
+    seen, out = set(), []
+    for layer in model.layers:
+        for part in layer.parts():
+            for value in vars(part).values():
+                tensors = []
+                if hasattr(value, "weight") and hasattr(value, "bias"):
+                    tensors = [value.weight, value.bias]
+                elif hasattr(value, "data_ptr"):
+                    tensors = [value]
+                for t in tensors:
+                    if t is not None and t.data_ptr() not in seen:
+                        seen.add(t.data_ptr())
+                        out.append(t)
+    for t in (model.final_norm.weight, model.head.weight):
+        if t.data_ptr() not in seen:
+            seen.add(t.data_ptr())
+            out.append(t)
+    return out
+
+
+def _prefill_flops(config, tokens: int) -> float:
+    h, i, d = config.hidden_size, config.intermediate_size, config.head_dim
+    nq, nkv, layers = config.num_attention_heads, config.num_key_value_heads, config.num_hidden_layers
+    linear = 2.0 * tokens * (h * (nq + 2 * nkv) * d + nq * d * h + 3 * h * i) * layers
+    attention = 4.0 * nq * d * (tokens * (tokens + 1) / 2.0) * layers     # q.k and p.v over the causal half
+    head = 2.0 * h * config.vocab_size                                    # logits of the last position only
+    return linear + attention + head
+
+
+if __name__ == "__main__":
+    sys.exit(main())

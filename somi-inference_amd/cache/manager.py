@@ -63,9 +63,11 @@ class CacheManager:
                 self.groups[group].runs.append(run)
                 k = v = None
                 if allocate_tensors:
-                    shape = (self.num_blocks, need.num_kv_heads, self.block_size, need.head_dim)
-                    k = torch.zeros(shape, dtype=dtype, device=self.device)
-                    v = torch.zeros(shape, dtype=dtype, device=self.device)
+                    # V is transposed inside a page: consecutive positions of one channel are adjacent
+                    k = torch.zeros((self.num_blocks, need.num_kv_heads, self.block_size, need.head_dim),
+                                    dtype=dtype, device=self.device)
+                    v = torch.zeros((self.num_blocks, need.num_kv_heads, need.head_dim, self.block_size),
+                                    dtype=dtype, device=self.device)
                 self.layer_caches[run] = LayerCache(need, group, k=k, v=v)
             elif isinstance(need, FixedStateSpec):
                 state = None

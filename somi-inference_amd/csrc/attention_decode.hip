@@ -1,0 +1,260 @@
+// Paged grouped-query attention for decoded tokens and short portions, bfloat16, on the matrix cores.
+//
+// Reference: somi_inference/core/paged_attention.py:352-413 (walk the block table with a running max,
+// running sum and rescaled output; float32 softmax state; weights cast to the value dtype before P.V) and
+// its Triton twin core/paged_attention_triton.py:29-150, which launches one program per (sequence, query
+// head) and so reads every key and value nq/nkv times.  Here one workgroup serves all query heads that
+// share a key/value head, and the keys of a long context are split over workgroups so that a few
+// requests still fill 256 compute units:
+//   grid = (token, kv head x blocks of 16 query heads, split of the context)
+//   a wavefront takes 16-key tiles (aligned to absolute positions) of its split in turn;
+//   S^T[key, head] = K[key, :] . Q^T   (v_mfma_f32_16x16x32_bf16; K rows are the A operand, read 16 B per lane)
+//   online softmax per head over the tile in float32 (the four keys a lane holds, then across lane groups)
+//   O^T[d, head] += V^T[d, key] . P^T (v_mfma_f32_16x16x16_bf16; S^T comes out of the first product in
+//                   exactly the B-operand layout, and V is stored transposed inside a page so a lane reads
+//                   four consecutive keys of one channel with one 8-byte load)
+// The wavefronts of a workgroup are merged through LDS; with several splits the workgroup writes
+// (max, sum, unnormalised output) to a workspace and a second kernel merges the splits in split order.
+#include "common.h"
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(4))) short short4_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+__device__ __forceinline__ bf16x8 ld8(const bf16* p) { return *reinterpret_cast<const bf16x8*>(p); }
+__device__ __forceinline__ short4_t ld4(const bf16* p) { return *reinterpret_cast<const short4_t*>(p); }
+// Four elements in the lower half of an eight-wide operand, zeros above.
+__device__ __forceinline__ bf16x8 half_step(const bf16* p) {
+    union { bf16x8 wide; short4_t half[2]; } u;
+    u.half[0] = ld4(p);
+    u.half[1] = short4_t{0, 0, 0, 0};
+    return u.wide;
+}
+
+template <int DT>
+__global__ void __launch_bounds__(256)
+attention_decode_kernel(const bf16* __restrict__ q, int64_t q_stride, const bf16* __restrict__ kc,
+                        const bf16* __restrict__ vc, const int* __restrict__ block_table, int max_blocks,
+                        const int* __restrict__ token_list, const int* __restrict__ token_entry,
+                        const int* __restrict__ positions, int nq, int nkv, int page_size, int window, float scale,
+                        int split_len, int num_splits, bf16* __restrict__ out, float* __restrict__ part_acc,
+                        float* __restrict__ part_ml) {
+    constexpr int D = DT * 16;
+    extern __shared__ float lds[];
+    const int waves = blockDim.x >> 6;
+    float* lds_acc = lds;                                  // [waves][DT][64][4]
+    float* lds_m = lds + waves * DT * 256;                 // [waves][16]
+    float* lds_l = lds_m + waves * 16;                     // [waves][16]
+
+    const int ti = blockIdx.x;
+    const int t = token_list ? token_list[ti] : ti;
+    const int G = nq / nkv, HB = (G + 15) / 16;
+    const int kvh = blockIdx.y / HB, hb = blockIdx.y % HB;
+    const int split = blockIdx.z;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4;
+
+    const int p = positions[t];
+    const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+    const int* table = block_table + (int64_t)token_entry[t] * max_blocks;
+    const int begin = lo > split * split_len ? lo : split * split_len;
+    const int end = p < (split + 1) * split_len - 1 ? p : (split + 1) * split_len - 1;      // inclusive
+
+    const int hloc = hb * 16 + r;
+    const int head = kvh * G + (hloc < G ? hloc : G - 1);
+    const bf16* qrow = q + (int64_t)t * q_stride + (int64_t)head * D;
+    // The head size is walked in 32-wide steps; an odd number of 16-wide tiles leaves a last step whose
+    // upper half is zero in both operands.  (All products of the chain are the same instruction: a
+    // 16x16x16 product that takes the result of a 16x16x32 one as its addend straight away, without an
+    // instruction in between, has been seen to read it too early.)
+    constexpr int QK_STEPS = (DT + 1) / 2;
+    bf16x8 qf[QK_STEPS];
+#pragma unroll
+    for (int c = 0; c < DT / 2; ++c) qf[c] = ld8(qrow + c * 32 + g * 8);
+    if (DT & 1) qf[QK_STEPS - 1] = half_step(qrow + (DT - 1) * 16 + g * 4);
+
+    float m_run = -INFINITY, l_run = 0.f;
+    f32x4 acc[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) acc[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    if (begin <= end) {
+        for (int tile = begin / 16 + wave; tile <= end / 16; tile += waves) {
+            const int j0 = tile * 16;
+            // keys: lane reads row j0 + r (an address inside the split even where the key is masked)
+            int pos = j0 + r;
+            pos = pos < begin ? begin : (pos > end ? end : pos);
+            const int64_t kpage = table[pos / page_size];
+            const bf16* krow = kc + ((kpage * nkv + kvh) * page_size + pos % page_size) * (int64_t)D;
+            // values: lane reads channel dt * 16 + r at keys j0 + 4 g .. + 3 (one page: page_size % 4 == 0)
+            int vpos = j0 + g * 4;
+            const int vlo = begin & ~3, vhi = end & ~3;
+            vpos = vpos < vlo ? vlo : (vpos > vhi ? vhi : vpos);
+            const int64_t vpage = table[vpos / page_size];
+            const bf16* vbase = vc + (vpage * nkv + kvh) * (int64_t)D * page_size + vpos % page_size;
+            // all loads of the tile are issued before the first product
+            bf16x8 kf[QK_STEPS];
+            short4_t vf[DT];
+#pragma unroll
+            for (int c = 0; c < DT / 2; ++c) kf[c] = ld8(krow + c * 32 + g * 8);
+            if (DT & 1) kf[QK_STEPS - 1] = half_step(krow + (DT - 1) * 16 + g * 4);
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) vf[dt] = ld4(vbase + (int64_t)(dt * 16 + r) * page_size);
+            f32x4 s = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int c = 0; c < QK_STEPS; ++c) s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[c], qf[c], s, 0, 0, 0);
+            // s[i] = S[key j0 + 4 g + i][head r]
+            float mx = -INFINITY;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int pj = j0 + g * 4 + i;
+                s[i] = (pj >= begin && pj <= end) ? s[i] * scale : -INFINITY;
+                mx = fmaxf(mx, s[i]);
+            }
+            mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            const float m_new = fmaxf(m_run, mx);           // finite: every tile holds a visible key
+            const float corr = expf(m_run - m_new);
+            float pr[4], sum = 0.f;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                pr[i] = expf(s[i] - m_new);
+                sum += pr[i];
+            }
+            sum += __shfl_xor(sum, 16, 64);
+            sum += __shfl_xor(sum, 32, 64);
+            l_run = l_run * corr + sum;
+            m_run = m_new;
+            bf16x4 pb = {(bf16)pr[0], (bf16)pr[1], (bf16)pr[2], (bf16)pr[3]};
+            const short4_t pf = *reinterpret_cast<short4_t*>(&pb);
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                acc[dt] *= corr;
+                acc[dt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf[dt], pf, acc[dt], 0, 0, 0);
+            }
+        }
+    }
+
+    // merge the wavefronts: acc[dt][i] = O^T[d = dt * 16 + 4 g + i][head r]
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+        *reinterpret_cast<f32x4*>(lds_acc + ((wave * DT + dt) * 64 + lane) * 4) = acc[dt];
+    if (g == 0) {
+        lds_m[wave * 16 + r] = m_run;
+        lds_l[wave * 16 + r] = l_run;
+    }
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < DT * 256; idx += blockDim.x) {
+        const int dt = idx >> 8, l = (idx >> 2) & 63, i = idx & 3;
+        const int hr = l & 15;
+        const int hl = hb * 16 + hr;
+        if (hl >= G) continue;
+        float m_all = -INFINITY;
+        for (int w = 0; w < waves; ++w) m_all = fmaxf(m_all, lds_m[w * 16 + hr]);
+        float total = 0.f, l_all = 0.f;
+        if (m_all > -INFINITY) {
+            for (int w = 0; w < waves; ++w) {
+                const float f = expf(lds_m[w * 16 + hr] - m_all);
+                total += lds_acc[w * DT * 256 + idx] * f;
+                l_all += lds_l[w * 16 + hr] * f;
+            }
+        }
+        const int d = dt * 16 + (l >> 4) * 4 + i;
+        const int hq = kvh * G + hl;
+        if (num_splits == 1) {
+            out[((int64_t)t * nq + hq) * D + d] = (bf16)(total / l_all);
+        } else {
+            const int64_t slot = ((int64_t)ti * nq + hq) * num_splits + split;
+            part_acc[slot * D + d] = total;
+            if (dt == 0 && (l >> 4) == 0 && i == 0) {
+                part_ml[slot * 2] = m_all;
+                part_ml[slot * 2 + 1] = l_all;
+            }
+        }
+    }
+}
+
+// Merge the splits of one (token, head) in split order.
+__global__ void __launch_bounds__(64)
+attention_combine_kernel(const float* __restrict__ part_acc, const float* __restrict__ part_ml,
+                         const int* __restrict__ token_list, int nq, int D, int num_splits,
+                         bf16* __restrict__ out) {
+    const int ti = blockIdx.x, h = blockIdx.y;
+    const int t = token_list ? token_list[ti] : ti;
+    const int64_t base = ((int64_t)ti * nq + h) * num_splits;
+    float m_all = -INFINITY;
+    for (int s = 0; s < num_splits; ++s)
+        if (part_ml[(base + s) * 2 + 1] > 0.f) m_all = fmaxf(m_all, part_ml[(base + s) * 2]);
+    float l_all = 0.f;
+    for (int s = 0; s < num_splits; ++s) {
+        const float l = part_ml[(base + s) * 2 + 1];
+        if (l > 0.f) l_all += l * expf(part_ml[(base + s) * 2] - m_all);
+    }
+    for (int d = threadIdx.x; d < D; d += 64) {
+        float total = 0.f;
+        for (int s = 0; s < num_splits; ++s) {
+            const float l = part_ml[(base + s) * 2 + 1];
+            if (l > 0.f) total += part_acc[(base + s) * D + d] * expf(part_ml[(base + s) * 2] - m_all);
+        }
+        out[((int64_t)t * nq + h) * D + d] = (bf16)(total / l_all);
+    }
+}
+
+template <int DT>
+static int launch_decode(const void* q, int64_t q_stride, const void* kc, const void* vc, const int* block_table,
+                         int max_blocks, const int* token_list, const int* token_entry, const int* positions,
+                         int n_list, int nq, int nkv, int page_size, int window, float scale, int split_len,
+                         int num_splits, void* out, float* part_acc, float* part_ml, hipStream_t stream) {
+    const int waves = DT <= 8 ? 4 : 2;
+    const int G = nq / nkv, HB = (G + 15) / 16;
+    const size_t smem = (size_t)(waves * DT * 256 + waves * 32) * sizeof(float);
+    hipLaunchKernelGGL((attention_decode_kernel<DT>), dim3(n_list, nkv * HB, num_splits), dim3(waves * 64), smem,
+                       stream, (const bf16*)q, q_stride, (const bf16*)kc, (const bf16*)vc, block_table, max_blocks,
+                       token_list, token_entry, positions, nq, nkv, page_size, window, scale, split_len, num_splits,
+                       (bf16*)out, part_acc, part_ml);
+    SOMI_LAUNCH_CHECK("attention_decode");
+    if (num_splits > 1) {
+        hipLaunchKernelGGL(attention_combine_kernel, dim3(n_list, nq), dim3(64), 0, stream, part_acc, part_ml,
+                           token_list, nq, DT * 16, num_splits, (bf16*)out);
+        SOMI_LAUNCH_CHECK("attention_combine");
+    }
+    return 0;
+}
+
+// Attention of the listed tokens (token_list: [n_list] indices into the step's tokens, or null for tokens
+// 0 .. n_list - 1) over their requests' pages.  bfloat16 only; head_dim a multiple of 16 up to 256;
+// page_size a multiple of 4.  k_cache [pages, nkv, page_size, D], v_cache [pages, nkv, D, page_size].
+// With num_splits > 1, part_acc holds n_list * nq * num_splits * D floats and part_ml
+// n_list * nq * num_splits * 2 floats; split_len is a multiple of 16 and split_len * num_splits covers every
+// listed token's position.
+extern "C" int somi_attention_decode(const void* q, int64_t q_stride, const void* k_cache, const void* v_cache,
+                                     const int* block_table, int max_blocks, const int* token_list,
+                                     const int* token_entry, const int* positions, int n_list, int nq, int nkv, int D,
+                                     int page_size, int window, float scale, int split_len, int num_splits, void* out,
+                                     float* part_acc, float* part_ml, hipStream_t stream) {
+    SOMI_REQUIRE(n_list >= 0 && nq > 0 && nkv > 0 && max_blocks > 0, "attention_decode: bad sizes");
+    SOMI_REQUIRE(nq % nkv == 0, "attention_decode: num_q_heads (%d) must be divisible by num_kv_heads (%d)", nq, nkv);
+    SOMI_REQUIRE(D % 16 == 0 && D >= 16 && D <= 256, "attention_decode: head_dim %d must be a multiple of 16 up to 256", D);
+    SOMI_REQUIRE(page_size > 0 && page_size % 4 == 0, "attention_decode: page size %d must be a multiple of 4", page_size);
+    SOMI_REQUIRE(window >= 0, "attention_decode: window must be >= 0");
+    SOMI_REQUIRE(num_splits >= 1 && num_splits <= 65535 && split_len > 0 && split_len % 16 == 0,
+                 "attention_decode: bad split (len %d, count %d)", split_len, num_splits);
+    SOMI_REQUIRE(num_splits == 1 || (part_acc && part_ml), "attention_decode: a workspace is needed for %d splits", num_splits);
+    SOMI_REQUIRE((uintptr_t)q % 16 == 0 && (q_stride * 2) % 16 == 0 && (uintptr_t)k_cache % 16 == 0 &&
+                 (uintptr_t)v_cache % 8 == 0, "attention_decode: q, k and v must be 16-byte aligned");
+    const int G = nq / nkv, HB = (G + 15) / 16;
+    SOMI_REQUIRE(nkv * HB <= 65535, "attention_decode: too many heads");
+    if (n_list == 0) return 0;
+#define SOMI_DECODE(DT)                                                                                              \
+    case DT:                                                                                                         \
+        return launch_decode<DT>(q, q_stride, k_cache, v_cache, block_table, max_blocks, token_list, token_entry,    \
+                                 positions, n_list, nq, nkv, page_size, window, scale, split_len, num_splits, out,   \
+                                 part_acc, part_ml, stream)
+    switch (D / 16) {
+        SOMI_DECODE(1); SOMI_DECODE(2); SOMI_DECODE(3); SOMI_DECODE(4); SOMI_DECODE(5); SOMI_DECODE(6);
+        SOMI_DECODE(7); SOMI_DECODE(8); SOMI_DECODE(9); SOMI_DECODE(10); SOMI_DECODE(11); SOMI_DECODE(12);
+        SOMI_DECODE(13); SOMI_DECODE(14); SOMI_DECODE(15); SOMI_DECODE(16);
+    }
+#undef SOMI_DECODE
+    return somi_fail("attention_decode: unsupported head_dim %d", D);
+}

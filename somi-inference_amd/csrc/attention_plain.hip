@@ -23,6 +23,7 @@ paged_attention_plain_kernel(const T* __restrict__ q, int64_t q_stride, const T*
     float* ps = qs + ((D + 1) & ~1);           // [NT] softmax weights of the tile
     float* red = ps + NT;                      // [16]
     int64_t* rowoff = (int64_t*)(red + 16);    // [NT] element offset of each key row of the tile
+    int64_t* coloff = rowoff + NT;             // [NT] element offset of each value column (V is [.., D, page_size])
 
     const int t = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
     const int e = token_entry[t];
@@ -45,6 +46,7 @@ paged_attention_plain_kernel(const T* __restrict__ q, int64_t q_stride, const T*
             const int64_t page = table[pos / page_size];
             const int64_t off = ((page * nkv + kvh) * page_size + pos % page_size) * (int64_t)D;
             rowoff[tid] = off;
+            coloff[tid] = (page * nkv + kvh) * (int64_t)D * page_size + pos % page_size;
             const T* kr = kc + off;
             float dot = 0.f;
             for (int d = 0; d < D; ++d) dot = fmaf(qs[d], to_float(kr[d]), dot);
@@ -66,7 +68,7 @@ paged_attention_plain_kernel(const T* __restrict__ q, int64_t q_stride, const T*
             const int d = tid + r * NT;
             if (d < D) {
                 float a = acc[r] * corr;
-                for (int j = j0; j <= j1; ++j) a = fmaf(ps[j], to_float(vc[rowoff[j] + d]), a);
+                for (int j = j0; j <= j1; ++j) a = fmaf(ps[j], to_float(vc[coloff[j] + (int64_t)d * page_size]), a);
                 acc[r] = a;
             }
         }
@@ -78,7 +80,8 @@ paged_attention_plain_kernel(const T* __restrict__ q, int64_t q_stride, const T*
     }
 }
 
-// q: token t's head h starts at q + t * q_stride + h * D.  k_cache / v_cache: [num_pages, nkv, page_size, D].
+// q: token t's head h starts at q + t * q_stride + h * D.  k_cache: [num_pages, nkv, page_size, D];
+// v_cache: [num_pages, nkv, D, page_size].
 // block_table: [n_entries, max_blocks] int32 page ids of each entry's request (pages a window has passed
 // may hold -1; they are never read).  token_entry, positions: [n_tokens] int32.  out: [n_tokens, nq * D].
 extern "C" int somi_paged_attention_plain(const void* q, int dtype, int64_t q_stride, const void* k_cache,
@@ -95,7 +98,7 @@ extern "C" int somi_paged_attention_plain(const void* q, int dtype, int64_t q_st
     SOMI_REQUIRE(nq <= 65535, "paged_attention: too many heads");
     if (n_tokens == 0) return 0;
     const dim3 grid(n_tokens, nq);
-    const size_t smem = (size_t)(((D + 1) & ~1) + NT + 16) * sizeof(float) + NT * sizeof(int64_t);
+    const size_t smem = (size_t)(((D + 1) & ~1) + NT + 16) * sizeof(float) + 2 * NT * sizeof(int64_t);
     if (dtype == SOMI_F32)
         hipLaunchKernelGGL((paged_attention_plain_kernel<float, NT>), grid, dim3(NT), smem, stream, (const float*)q,
                            q_stride, (const float*)k_cache, (const float*)v_cache, block_table, max_blocks,

@@ -7,7 +7,9 @@
 //
 // The angle p * inv_freq[j] and its cos/sin are float32 whatever the storage type; inv_freq comes
 // from the host as a float32 table so both engines and the plain implementation share it.
-// Cache layout per layer: [num_pages, n_kv_heads, page_size, head_dim] for K and for V.
+// Cache layout per layer: K [num_pages, n_kv_heads, page_size, head_dim]; V is kept transposed inside
+// a page, [num_pages, n_kv_heads, head_dim, page_size], so that the attention kernels read consecutive
+// positions of one channel with one load (the operand layout of the matrix cores for P.V).
 #include "common.h"
 
 template <typename T>
@@ -27,11 +29,12 @@ rope_kv_store_kernel(T* __restrict__ qkv, int64_t row_stride, const int* __restr
         const bool is_v = hh >= nq + nkv;
         const int kvh = hh - nq - (is_v ? nkv : 0);
         const int64_t page = slot / page_size, off = slot % page_size;
-        dst = (is_v ? vc : kc) + ((page * nkv + kvh) * page_size + off) * D;
         if (is_v) {
-            for (int d = threadIdx.x; d < D; d += 64) dst[d] = src[d];
+            T* col = vc + (page * nkv + kvh) * (int64_t)D * page_size + off;
+            for (int d = threadIdx.x; d < D; d += 64) col[(int64_t)d * page_size] = src[d];
             return;
         }
+        dst = kc + ((page * nkv + kvh) * page_size + off) * D;
     }
     T* q_or_k = dst ? dst : src;               // q is rotated in place, k goes to its page
     for (int j = threadIdx.x; j < rot_half; j += 64) {

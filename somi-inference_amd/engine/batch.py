@@ -66,12 +66,9 @@ class StepBatch:
     block_size: int
 
 
-def build_step(entries: list[StepEntry], cache: CacheManager, device: torch.device) -> StepBatch:
-    """Lay out the step on the host and copy it to the device in one transfer.
-
-    Pages for the new tokens must already be reserved: slot mappings and block
-    tables are read from the cache manager as they stand.
-    """
+def _layout(entries: list[StepEntry], cache: CacheManager, table_widths: list[int] | None):
+    """The step as host arrays: (sections, infos, widths).  ``table_widths`` fixes the block tables'
+    widths (a captured graph needs the same layout at every replay); None = as narrow as possible."""
     infos: list[EntryInfo] = []
     token_ids: list[int] = []
     positions: list[int] = []
@@ -86,11 +83,14 @@ def build_step(entries: list[StepEntry], cache: CacheManager, device: torch.devi
         positions.extend(range(first, first + len(entry.tokens)))
         token_entry.extend([index] * len(entry.tokens))
     n, e = len(token_ids), len(entries)
-    bs = cache.block_size
     tables, slot_maps, widths = [], [], []
     for g in range(len(cache.groups)):
         rows = [cache.page_list(g, info.request_id) for info in infos]
         width = max(1, max((len(r) for r in rows), default=1))
+        if table_widths is not None:
+            if width > table_widths[g]:
+                raise ValueError(f"block table of width {width} does not fit the fixed width {table_widths[g]}")
+            width = table_widths[g]
         table = np.zeros((e, width), dtype=np.int32)
         for r, pages in enumerate(rows):
             # released pages read as page 0: the kernels never look below a window
@@ -101,7 +101,6 @@ def build_step(entries: list[StepEntry], cache: CacheManager, device: torch.devi
         tables.append(table)
         slot_maps.append(np.asarray(slots, dtype=np.int32))
         widths.append(width)
-
     sections = [
         np.asarray(token_ids, dtype=np.int32), np.asarray(positions, dtype=np.int32),
         np.asarray(token_entry, dtype=np.int32),
@@ -113,22 +112,64 @@ def build_step(entries: list[StepEntry], cache: CacheManager, device: torch.devi
     ]
     for table, slots in zip(tables, slot_maps):
         sections += [slots, table.reshape(-1)]
-    offsets = np.cumsum([0] + [s.size for s in sections])
-    packed = torch.from_numpy(np.concatenate(sections) if sections else np.zeros(0, np.int32))
-    on_device = packed.to(device)
+    return sections, infos, widths
+
+
+def _views(on_device: torch.Tensor, sizes: list[int], infos: list[EntryInfo], widths: list[int],
+           num_groups: int, block_size: int, max_context: int | None = None) -> StepBatch:
+    offsets = np.cumsum([0] + sizes)
 
     def part(i: int) -> torch.Tensor:
         return on_device[int(offsets[i]):int(offsets[i + 1])]
 
-    paged = []
-    for g in range(len(cache.groups)):
-        paged.append(PagedView(part(8 + 2 * g), part(9 + 2 * g).view(e, widths[g])))
+    e = len(infos)
+    paged = [PagedView(part(8 + 2 * g), part(9 + 2 * g).view(e, widths[g])) for g in range(num_groups)]
     return StepBatch(
-        num_tokens=n, num_entries=e, num_logit_rows=len(logit_rows),
+        num_tokens=sizes[0], num_entries=e, num_logit_rows=sizes[7],
         token_ids=part(0), positions=part(1), token_entry=part(2), entry_start=part(3),
         entry_first_position=part(4), context_lens=part(5), state_slots=part(6), logit_rows=part(7),
         paged=paged, entries=infos,
         max_entry_len=max((i.length for i in infos), default=0),
-        max_context=max((i.first_position + i.length for i in infos), default=0),
-        block_size=bs,
+        max_context=max_context if max_context is not None else max((i.first_position + i.length for i in infos), default=0),
+        block_size=block_size,
     )
+
+
+def build_step(entries: list[StepEntry], cache: CacheManager, device: torch.device) -> StepBatch:
+    """Lay out the step on the host and copy it to the device in one transfer.
+
+    Pages for the new tokens must already be reserved: slot mappings and block
+    tables are read from the cache manager as they stand.
+    """
+    sections, infos, widths = _layout(entries, cache, None)
+    packed = torch.from_numpy(np.concatenate(sections))
+    return _views(packed.to(device), [s.size for s in sections], infos, widths, len(cache.groups), cache.block_size)
+
+
+class StaticStep:
+    """A step of fixed shape (one token and one wanted logit per entry, block tables of fixed width)
+    whose device arrays stay in place, so that a captured HIP graph can be replayed on new contents."""
+
+    def __init__(self, entries: list[StepEntry], cache: CacheManager, device: torch.device,
+                 table_widths: list[int]) -> None:
+        self.table_widths = list(table_widths)
+        sections, infos, widths = _layout(entries, cache, self.table_widths)
+        self.sizes = [s.size for s in sections]
+        self.host = torch.empty(sum(self.sizes), dtype=torch.int32).pin_memory()
+        self.device_buffer = torch.empty(sum(self.sizes), dtype=torch.int32, device=device)
+        # kernels that size their launch by the context use the widest the tables allow
+        self.batch = _views(self.device_buffer, self.sizes, infos, widths, len(cache.groups), cache.block_size,
+                            max_context=max(self.table_widths, default=1) * cache.block_size)
+        self._fill(sections, infos)
+
+    def _fill(self, sections, infos) -> None:
+        self.host.copy_(torch.from_numpy(np.concatenate(sections)))
+        self.device_buffer.copy_(self.host)      # blocking: the staging buffer is free again on return
+        self.batch.entries = infos
+
+    def update(self, entries: list[StepEntry], cache: CacheManager) -> StepBatch:
+        sections, infos, _ = _layout(entries, cache, self.table_widths)
+        if [s.size for s in sections] != self.sizes:
+            raise ValueError("the entries do not fit the shape this step was laid out for")
+        self._fill(sections, infos)
+        return self.batch

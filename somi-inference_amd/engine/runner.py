@@ -18,20 +18,33 @@ import torch
 from ..cache.manager import CacheManager
 from ..cache.pool import OutOfPages
 from ..models.decoder import DecoderModel
-from .batch import StepBatch, StepEntry, build_step
+from .batch import StaticStep, StepBatch, StepEntry, build_step
 
 
 class StepError(ValueError):
     """A step's entries break the step function's contract."""
 
 
+class _DecodeGraph:
+    """One captured decode step: its static arrays, the HIP graph and the logits it writes."""
+
+    def __init__(self, static: StaticStep, graph: torch.cuda.CUDAGraph, logits: torch.Tensor) -> None:
+        self.static, self.graph, self.logits = static, graph, logits
+
+
 class ModelRunner:
-    def __init__(self, model: DecoderModel, cache: CacheManager) -> None:
+    def __init__(self, model: DecoderModel, cache: CacheManager, *, decode_graphs: bool = True) -> None:
         self.model = model
         self.cache = cache
         self.device = model.runtime.device
         self.vocab_size = model.vocab_size
         self.steps_run = 0
+        # Steps of single decoded tokens are bound by kernel launches, so they are captured once per
+        # shape as a HIP graph and replayed.  Only for models whose parts all launch on the stream
+        # without looking at host-side values of the step.
+        self.decode_graphs = bool(decode_graphs) and model.graph_safe()
+        self._graphs: dict[tuple, _DecodeGraph] = {}
+        self.graph_replays = 0
 
     # ------------------------------------------------------------ request life
     def begin(self, request_id: Hashable) -> None:
@@ -74,9 +87,45 @@ class ModelRunner:
             raise OutOfPages(f"the step needs more pages than are free ({self.cache.free_pages()} free)")
         for request_id, count in portions:
             self.cache.reserve(request_id, count)
-        batch = build_step(entries, self.cache, self.device)
-        logits = self.model.forward(batch, self.cache.layer_caches)
+        if self.decode_graphs and all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries):
+            logits = self._decode_with_graph(entries)
+        else:
+            batch = build_step(entries, self.cache, self.device)
+            logits = self.model.forward(batch, self.cache.layer_caches)
         for request_id, count in portions:
             self.cache.commit(request_id, count)
         self.steps_run += 1
         return logits
+
+    # ------------------------------------------------------------- HIP graphs
+    def _decode_with_graph(self, entries: list[StepEntry]) -> torch.Tensor:
+        """Replay (or first capture) the graph for this many single-token entries.
+
+        The block tables of a captured step have a fixed width, the next power of two of pages that
+        holds the longest request, so a graph serves until a request outgrows it.  The returned logits
+        are the graph's own output tensor: they are overwritten by the next replay of the same graph.
+        """
+        widths = []
+        for g in range(len(self.cache.groups)):
+            longest = max(len(self.cache.page_list(g, e.request_id)) for e in entries)
+            width = 16
+            while width < longest:
+                width *= 2
+            widths.append(width)
+        key = (len(entries), tuple(widths))
+        held = self._graphs.get(key)
+        if held is None:
+            static = StaticStep(entries, self.cache, self.device, widths)
+            # once outside a capture: lazy initialisation (library handles, first allocations) must
+            # not happen while the stream is being recorded; the step's writes are simply redone
+            self.model.forward(static.batch, self.cache.layer_caches)
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                logits = self.model.forward(static.batch, self.cache.layer_caches)
+            held = self._graphs[key] = _DecodeGraph(static, graph, logits)
+        else:
+            held.static.update(entries, self.cache)
+        held.graph.replay()
+        self.graph_replays += 1
+        return held.logits

@@ -6,12 +6,43 @@ import torch
 
 from . import ops
 
+TARGET_WORKGROUPS = 1024        # about four per compute unit
+MIN_SPLIT = 64                  # keys per split at least (a multiple of the 16-key tile)
+
+
+def decode_splits(num_tokens: int, groups: int, max_context: int) -> tuple[int, int]:
+    """(split_len, num_splits): how the keys of a request are cut over workgroups so that
+    ``num_tokens * groups * num_splits`` is about TARGET_WORKGROUPS.  Boundaries are multiples of
+    MIN_SPLIT in absolute positions."""
+    max_context = max(1, max_context)
+    most = (max_context + MIN_SPLIT - 1) // MIN_SPLIT
+    splits = max(1, min(TARGET_WORKGROUPS // max(1, num_tokens * groups), most))
+    split_len = ((max_context + splits - 1) // splits + MIN_SPLIT - 1) // MIN_SPLIT * MIN_SPLIT
+    return split_len, (max_context + split_len - 1) // split_len
+
+
+def mfma_attention_supported(q: torch.Tensor, k_cache: torch.Tensor) -> bool:
+    head_dim, page_size = k_cache.shape[3], k_cache.shape[2]
+    return (q.dtype == torch.bfloat16 and head_dim % 16 == 0 and head_dim <= 256 and page_size % 4 == 0
+            and q.data_ptr() % 16 == 0 and (q.shape[1] * 2) % 16 == 0)
+
 
 def paged_attention(qkv: torch.Tensor, num_heads: int, k_cache: torch.Tensor, v_cache: torch.Tensor,
                     block_table: torch.Tensor, step, *, window: int, scale: float) -> torch.Tensor:
     """Attention of every token of the step over its request's cache pages -> [N, nq * D].
 
-    ``qkv`` holds each token's query heads first in its row (rotated already).
+    ``qkv`` holds each token's query heads first in its row (rotated already).  float32, and shapes the
+    MFMA kernels do not take (head sizes that are no multiple of 16, page sizes that are no multiple
+    of 4), run the plain kernel.
     """
-    return ops.paged_attention_plain(qkv, qkv.shape[1], k_cache, v_cache, block_table,
-                                     step.token_entry, step.positions, num_heads, window, scale)
+    if not mfma_attention_supported(qkv, k_cache):
+        return ops.paged_attention_plain(qkv, qkv.shape[1], k_cache, v_cache, block_table,
+                                         step.token_entry, step.positions, num_heads, window, scale)
+    nkv, head_dim = k_cache.shape[1], k_cache.shape[3]
+    groups = nkv * ((num_heads // nkv + 15) // 16)
+    out = torch.empty((qkv.shape[0], num_heads * head_dim), dtype=qkv.dtype, device=qkv.device)
+    reach = min(step.max_context, window + step.max_entry_len) if window else step.max_context
+    split_len, num_splits = decode_splits(step.num_tokens, groups, step.max_context)
+    ops.attention_decode(qkv, qkv.shape[1], k_cache, v_cache, block_table, step.token_entry, step.positions,
+                         num_heads, window, scale, split_len, num_splits, out)
+    return out

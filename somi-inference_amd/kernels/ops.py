@@ -60,6 +60,11 @@ def _need(t: torch.Tensor, name: str, dtype: torch.dtype | None = None, shape: t
         raise KernelError(f"{name}: expected shape {tuple(shape)}, got {tuple(t.shape)}")
 
 
+def _v_shape(k_cache: torch.Tensor) -> tuple:
+    pages, nkv, page_size, head_dim = k_cache.shape
+    return (pages, nkv, head_dim, page_size)
+
+
 def embedding(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
     """h[t] = table[ids[t]] as float32.  table: [V, H]; ids: [N] int32."""
     _need(table, "embedding table")
@@ -124,12 +129,31 @@ def linear_plain(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | Non
     return out
 
 
+def linear_skinny(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None,
+                  out_dtype: torch.dtype | None = None) -> torch.Tensor:
+    """x @ weight.T (+ bias) for at most 64 bfloat16 rows on the matrix cores (weight streamed once)."""
+    _need(x, "linear input", torch.bfloat16)
+    m, k = x.shape
+    _need(weight, "linear weight", torch.bfloat16)
+    n = weight.shape[0]
+    if weight.shape[1] != k:
+        raise KernelError(f"linear: input has {k} features, weight expects {weight.shape[1]}")
+    if bias is not None:
+        _need(bias, "linear bias", torch.float32, (n,))
+    out_dtype = out_dtype or x.dtype
+    out = torch.empty((m, n), dtype=out_dtype, device=x.device)
+    _check(library().somi_linear_skinny(_ptr(x), _ptr(weight), _ptr(bias), _ptr(out), dtype_code(out_dtype),
+                                        m, n, k, _stream()))
+    return out
+
+
 def rope_kv_store(qkv: torch.Tensor, positions: torch.Tensor, slots: torch.Tensor | None,
                   inv_freq: torch.Tensor | None, rotary_dim: int, nq: int, nkv: int, head_dim: int,
                   k_cache: torch.Tensor | None, v_cache: torch.Tensor | None) -> None:
     """Rotate q (in place) and k, and store k and v in their cache pages.
 
-    qkv: [N, (nq + 2 nkv) * D]; caches: [pages, nkv, page_size, D]; slots: [N] int32.
+    qkv: [N, (nq + 2 nkv) * D]; k cache: [pages, nkv, page_size, D]; v cache: [pages, nkv, D, page_size];
+    slots: [N] int32.
     """
     _need(qkv, "qkv")
     n = qkv.shape[0]
@@ -140,7 +164,9 @@ def rope_kv_store(qkv: torch.Tensor, positions: torch.Tensor, slots: torch.Tenso
     if nkv > 0:
         _need(slots, "slot mapping", torch.int32, (n,))
         _need(k_cache, "k cache", qkv.dtype)
-        _need(v_cache, "v cache", qkv.dtype, tuple(k_cache.shape))
+        if k_cache.dim() != 4:
+            raise KernelError("rope_kv_store: the k cache must be [pages, kv_heads, page_size, head_dim]")
+        _need(v_cache, "v cache", qkv.dtype, _v_shape(k_cache))
         if k_cache.dim() != 4 or k_cache.shape[1] != nkv or k_cache.shape[3] != head_dim:
             raise KernelError(f"rope_kv_store: cache shape {tuple(k_cache.shape)} != [pages, {nkv}, page, {head_dim}]")
         page_size = k_cache.shape[2]
@@ -161,7 +187,9 @@ def paged_attention_plain(q: torch.Tensor, q_stride: int, k_cache: torch.Tensor,
     _need(q, "q")
     n = q.shape[0]
     _need(k_cache, "k cache", q.dtype)
-    _need(v_cache, "v cache", q.dtype, tuple(k_cache.shape))
+    if k_cache.dim() != 4:
+        raise KernelError("paged_attention: the k cache must be [pages, kv_heads, page_size, head_dim]")
+    _need(v_cache, "v cache", q.dtype, _v_shape(k_cache))
     _, nkv, page_size, head_dim = k_cache.shape
     if q_stride < nq * head_dim or q.shape[1] < nq * head_dim:
         raise KernelError("paged_attention: q rows are narrower than nq * head_dim")
@@ -174,6 +202,40 @@ def paged_attention_plain(q: torch.Tensor, q_stride: int, k_cache: torch.Tensor,
         block_table.shape[1], _ptr(token_entry), _ptr(positions), n, nq, nkv, head_dim, page_size, window,
         ctypes.c_float(scale), _ptr(out), _stream()))
     return out
+
+
+def attention_decode(q: torch.Tensor, q_stride: int, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                     block_table: torch.Tensor, token_entry: torch.Tensor, positions: torch.Tensor,
+                     nq: int, window: int, scale: float, split_len: int, num_splits: int,
+                     out: torch.Tensor, token_list: torch.Tensor | None = None) -> None:
+    """MFMA attention of the listed tokens (all when ``token_list`` is None) over their pages, written
+    into ``out`` ([N, nq * D] bfloat16).  The keys of a request are cut into ``num_splits`` ranges of
+    ``split_len`` positions that run in parallel and are merged afterwards."""
+    _need(q, "q", torch.bfloat16)
+    n = q.shape[0]
+    _need(k_cache, "k cache", torch.bfloat16)
+    if k_cache.dim() != 4:
+        raise KernelError("attention_decode: the k cache must be [pages, kv_heads, page_size, head_dim]")
+    _need(v_cache, "v cache", torch.bfloat16, _v_shape(k_cache))
+    _, nkv, page_size, head_dim = k_cache.shape
+    if q_stride < nq * head_dim or q.shape[1] < nq * head_dim:
+        raise KernelError("attention_decode: q rows are narrower than nq * head_dim")
+    _need(block_table, "block table", torch.int32)
+    _need(token_entry, "token entries", torch.int32, (n,))
+    _need(positions, "positions", torch.int32, (n,))
+    _need(out, "attention out", torch.bfloat16, (n, nq * head_dim))
+    n_list = n
+    if token_list is not None:
+        _need(token_list, "token list", torch.int32)
+        n_list = token_list.numel()
+    part_acc = part_ml = None
+    if num_splits > 1:
+        part_acc = torch.empty((n_list * nq * num_splits, head_dim), dtype=torch.float32, device=q.device)
+        part_ml = torch.empty((n_list * nq * num_splits, 2), dtype=torch.float32, device=q.device)
+    _check(library().somi_attention_decode(
+        _ptr(q), ctypes.c_int64(q_stride), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), block_table.shape[1],
+        _ptr(token_list), _ptr(token_entry), _ptr(positions), n_list, nq, nkv, head_dim, page_size, window,
+        ctypes.c_float(scale), split_len, num_splits, _ptr(out), _ptr(part_acc), _ptr(part_ml), _stream()))
 
 
 def silu_mul(gate_up: torch.Tensor) -> torch.Tensor:

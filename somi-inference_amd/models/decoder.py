@@ -53,6 +53,15 @@ class DecoderModel:
             self.head.tie(self.embedding)
         self.loaded = True
 
+    def graph_safe(self) -> bool:
+        """True when every part says that its forward only launches work on the current stream from
+        device-side arrays of the step (so a step can be captured once and replayed)."""
+        parts = [self.embedding, self.final_norm, self.head]
+        for layer in self.layers:
+            parts.append(layer)
+            parts.extend(layer.parts())
+        return all(getattr(part, "graph_safe", False) for part in parts)
+
     # -------------------------------------------------------------------- cache
     def cache_needs(self) -> list[PagedKVSpec | FixedStateSpec | int | None]:
         """For each run of a layer: the cache its mixer needs, the index of the earlier

@@ -24,6 +24,8 @@ from .registry import build_part
 
 
 class GroupedQueryAttention(Mixer):
+    graph_safe = True
+
     def __init__(self, prefix: str, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  position: PartSpec, qkv_bias: bool = True, out_bias: bool = False,
                  window: int | None = None, scale: float | None = None, shares_cache: bool = False) -> None:

@@ -85,7 +85,7 @@ class LayerCache:
     spec: PagedKVSpec | FixedStateSpec
     group: int
     k: torch.Tensor | None = None        # [pages, kv_heads, page_size, head_dim]
-    v: torch.Tensor | None = None
+    v: torch.Tensor | None = None        # [pages, kv_heads, head_dim, page_size]
     state: torch.Tensor | None = None    # [slots, *shape]
     writes: bool = True
 
@@ -94,7 +94,14 @@ Fetch = Callable[[str], torch.Tensor]
 
 
 class Part:
-    """Base of all parts: weights in, nothing else assumed."""
+    """Base of all parts: weights in, nothing else assumed.
+
+    ``graph_safe``: the part's forward only launches work on the current stream and reads the step
+    through its device arrays, never through host-side values that change from step to step.  The
+    runner captures decode steps as HIP graphs only if every part of the model says so.
+    """
+
+    graph_safe = False
 
     def __init__(self, prefix: str = "") -> None:
         self.prefix = prefix

@@ -13,6 +13,7 @@ class PreNormBlock(Block):
     Reference: somi_inference/models/qwen2.py:325-339.  ``names`` gives the
     sub-prefixes of the four parts under the layer's prefix.
     """
+    graph_safe = True
 
     DEFAULT_NAMES = {"mixer_norm": "input_layernorm", "mixer": "self_attn",
                      "ffn_norm": "post_attention_layernorm", "feed_forward": "mlp"}

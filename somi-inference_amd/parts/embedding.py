@@ -17,6 +17,8 @@ from .base import Fetch, Part, Runtime
 
 
 class TokenEmbedding(Part):
+    graph_safe = True
+
     def __init__(self, prefix: str, vocab_size: int, hidden_size: int) -> None:
         super().__init__(prefix)
         self.vocab_size, self.hidden_size = int(vocab_size), int(hidden_size)
@@ -36,6 +38,7 @@ class TokenEmbedding(Part):
 
 class LMHead(Part):
     """logits = x . W^T in float32, for the rows that were asked for only."""
+    graph_safe = True
 
     def __init__(self, prefix: str, vocab_size: int, hidden_size: int, tied: bool = False) -> None:
         super().__init__(prefix)

@@ -14,6 +14,7 @@ class SwiGLU(FeedForward):
     """y = down(silu(gate(x)) * up(x)), no biases.  gate and up are stacked into one
     ``[2I, H]`` matrix, gate rows first, as the reference merges them at load
     (somi_inference/models/qwen2_adapter.py:183-190, 244-248; qwen2.py:228 chunks the result)."""
+    graph_safe = True
 
     def __init__(self, prefix: str, hidden_size: int, intermediate_size: int) -> None:
         super().__init__(prefix)

@@ -19,6 +19,9 @@ class Projection:
         self.weight = weight
         self.bias = bias
         self.out_features, self.in_features = weight.shape
+        # the library GEMM used for many rows wants the bias in the compute dtype (exact for a
+        # bias that came from a bfloat16 checkpoint)
+        self.bias_lowp = bias.to(weight.dtype) if bias is not None and weight.dtype != torch.float32 else None
 
     @classmethod
     def stacked(cls, weights: list[torch.Tensor], biases: list[torch.Tensor] | None = None) -> "Projection":
@@ -29,4 +32,4 @@ class Projection:
         return cls(weight, bias)
 
     def __call__(self, x: torch.Tensor, out_dtype: torch.dtype | None = None) -> torch.Tensor:
-        return linear_kernels.linear(x, self.weight, self.bias, out_dtype)
+        return linear_kernels.linear(x, self.weight, self.bias, out_dtype, self.bias_lowp)

@@ -12,6 +12,7 @@ from .base import Fetch, Norm, Runtime
 class RMSNorm(Norm):
     """y = w * x * rsqrt(mean(x^2) + eps), no mean subtraction, no bias
     (qwen2.py:55-62).  Square, mean, rsqrt and scale are float32."""
+    graph_safe = True
 
     def __init__(self, prefix: str, hidden_size: int, eps: float,
                  init: tuple[float, float] = (1.0, 0.1)) -> None:

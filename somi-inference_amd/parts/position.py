@@ -13,6 +13,7 @@ class RotaryPosition(PositionEncoding):
     (qwen2.py:76-79).  No table over positions is kept (the reference bounds the
     sequence length by its table, qwen2.py:72-81): the angle is computed from the
     position in float32 by the kernel that also writes k into its cache page."""
+    graph_safe = True
 
     def __init__(self, prefix: str, head_dim: int, theta: float, rotary_dim: int | None = None) -> None:
         super().__init__(prefix)
@@ -34,6 +35,7 @@ class RotaryPosition(PositionEncoding):
 
 class NoPosition(PositionEncoding):
     """No position information (attention is then invariant to a shift of all positions)."""
+    graph_safe = True
 
     def __init__(self, prefix: str = "") -> None:
         super().__init__(prefix)

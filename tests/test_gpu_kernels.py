@@ -81,7 +81,7 @@ def test_rope_and_cache_write(dtype, nq, nkv, d, page):
         pytest.skip("needs distinct slots")
     slots = i32(slot_list)
     kc = torch.zeros(pages, nkv, page, d, dtype=DT[dtype], device=DEV)
-    vc = torch.zeros_like(kc)
+    vc = torch.zeros(pages, nkv, d, page, dtype=DT[dtype], device=DEV)      # V is transposed inside a page
     inv_freq = plain.rope_inv_freq(d, theta).to(DEV)
     before = qkv.clone()
     ops.rope_kv_store(qkv, positions, slots, inv_freq, d, nq, nkv, d, kc, vc)
@@ -94,7 +94,7 @@ def test_rope_and_cache_write(dtype, nq, nkv, d, page):
     for t, slot in enumerate(slot_list):
         pg, off = divmod(slot, page)
         torch.testing.assert_close(kc[pg, :, off].float().cpu(), want_k[t], **tol)
-        assert torch.equal(vc[pg, :, off].cpu(), before.view(n, -1, d)[t, nq + nkv:].cpu())
+        assert torch.equal(vc[pg, :, :, off].cpu(), before.view(n, -1, d)[t, nq + nkv:].cpu())
     written = torch.zeros(pages * page, dtype=torch.bool)
     written[slot_list] = True
     untouched = kc.float().permute(0, 2, 1, 3).reshape(pages * page, -1).cpu()[~written]
@@ -140,11 +140,11 @@ def test_paged_attention_over_permuted_pages_for_portions_and_single_tokens(dtyp
     keys = [rnd(t, nkv, d, dtype=dtype, seed=10 + i) for i, t in enumerate(total)]
     values = [rnd(t, nkv, d, dtype=dtype, seed=20 + i) for i, t in enumerate(total)]
     kc = rnd(n_pages, nkv, page, d, dtype=dtype, seed=99)      # garbage everywhere else must be inert
-    vc = rnd(n_pages, nkv, page, d, dtype=dtype, seed=98)      # (reference tests/core/test_paged_attention.py:243-256)
+    vc = rnd(n_pages, nkv, d, page, dtype=dtype, seed=98)      # (reference tests/core/test_paged_attention.py:243-256)
     for r, t in enumerate(total):
         for pos in range(t):
             kc[tables[r][pos // page], :, pos % page] = keys[r][pos]
-            vc[tables[r][pos // page], :, pos % page] = values[r][pos]
+            vc[tables[r][pos // page], :, :, pos % page] = values[r][pos]
     n = sum(new)
     q = rnd(n, nq * d, dtype=dtype, seed=5, scale=2.0)
     positions = [cached[0] + i for i in range(new[0])] + [cached[1]]
@@ -163,11 +163,11 @@ def test_paged_attention_refuses_what_it_cannot_do():
     q = rnd(1, 5 * 16)
     kc = rnd(2, 2, 4, 16)
     with pytest.raises(KernelError, match="divisible"):      # reference: AssertionError on bad GQA (tests/core/test_paged_attention.py:340-350)
-        ops.paged_attention_plain(q, 80, kc, kc.clone(), i32([[0]]), i32([0]), i32([0]), 5, 0, 0.25)
+        ops.paged_attention_plain(q, 80, kc, rnd(2, 2, 16, 4), i32([[0]]), i32([0]), i32([0]), 5, 0, 0.25)
     big = rnd(1, 2 * 272)
     kc2 = rnd(2, 2, 4, 272)
     with pytest.raises(KernelError, match="head_dim"):
-        ops.paged_attention_plain(big, 544, kc2, kc2.clone(), i32([[0]]), i32([0]), i32([0]), 2, 0, 0.1)
+        ops.paged_attention_plain(big, 544, kc2, rnd(2, 2, 272, 4), i32([[0]]), i32([0]), i32([0]), 2, 0, 0.1)
     with pytest.raises(KernelError, match="GPU"):
         ops.silu_mul(torch.zeros(2, 4))
 
@@ -217,3 +217,97 @@ def test_repetition_penalty_rule():
     assert row.tolist() == [1.0, 1.5, -2.0, 0.5]
     with pytest.raises(KernelError, match="penalty"):
         ops.repetition_penalty(row, i32([0]), 0.0)
+
+
+@pytest.mark.parametrize("m, n, k", [(1, 503, 192), (7, 64, 72), (16, 130, 200), (17, 33, 1000), (48, 3584 + 16, 3584),
+                                     (64, 70, 18944), (8, 152064 // 16 + 3, 512)])
+def test_linear_skinny_mfma_against_float32(m, n, k):
+    x, w, b = rnd(m, k, dtype="bfloat16", seed=1), rnd(n, k, dtype="bfloat16", seed=2, scale=0.05), rnd(n, seed=3)
+    want = F.linear(x.float(), w.float(), b)
+    scale = float(want.abs().max())
+    got32 = ops.linear_skinny(x, w, b, torch.float32)
+    torch.testing.assert_close(got32, want, atol=2e-5 * scale * math.sqrt(k), rtol=1e-4)     # float32 sums of exact products
+    got = ops.linear_skinny(x, w, b)
+    assert got.dtype == torch.bfloat16
+    torch.testing.assert_close(got.float(), want, atol=scale * 2 ** -8, rtol=2 ** -7)         # one rounding to bfloat16
+    torch.testing.assert_close(ops.linear_skinny(x, w, None, torch.float32), F.linear(x.float(), w.float()),
+                               atol=2e-5 * scale * math.sqrt(k), rtol=1e-4)
+    # the same rows give the same bits whatever else is in the batch, as long as the number of 16-row
+    # tiles (which sets how K is split over wavefronts) is the same
+    first = (m - 1) // 16 * 16
+    assert torch.equal(ops.linear_skinny(x[first:first + 1].contiguous().repeat(first + 1, 1), w, b, torch.float32)[-1:],
+                       got32[first:first + 1])
+
+
+def test_linear_skinny_refuses_what_it_cannot_do():
+    with pytest.raises(KernelError, match="64 rows"):
+        ops.linear_skinny(rnd(65, 64, dtype="bfloat16"), rnd(8, 64, dtype="bfloat16"))
+    with pytest.raises(KernelError, match="multiple of 8"):
+        ops.linear_skinny(rnd(2, 12, dtype="bfloat16"), rnd(8, 12, dtype="bfloat16"))
+    with pytest.raises(KernelError, match="bfloat16"):
+        ops.linear_skinny(rnd(2, 16), rnd(8, 16))
+
+
+@pytest.mark.parametrize("nq, nkv, d, page, window, splits", [
+    (8, 4, 32, 4, 0, 1), (12, 2, 64, 16, 0, 3), (8, 1, 48, 8, 0, 2), (6, 3, 128, 16, 37, 4), (28, 4, 128, 16, 0, 5),
+    (40, 2, 16, 8, 0, 1), (14, 2, 256, 16, 0, 2), (5, 5, 80, 4, 5, 3), (7, 1, 112, 32, 100, 2)])
+def test_attention_decode_mfma_against_dense_softmax(nq, nkv, d, page, window, splits):
+    """The reference's own check of its decode kernel: dense softmax over the tokens gathered through a
+    permuted table (tests/core/test_paged_attention.py:292-338), here for portions and single tokens,
+    several splits of the keys, 1 to 20 query heads per key/value head and head sizes in steps of 16."""
+    cached, new = [30, 200, 0], [9, 1, 3]
+    total = [c + n for c, n in zip(cached, new)]
+    n_pages = sum((t + page - 1) // page for t in total) + 3
+    perm = torch.randperm(n_pages, generator=torch.Generator().manual_seed(3)).tolist()
+    tables, at = [], 0
+    for t in total:
+        count = (t + page - 1) // page
+        tables.append(perm[at:at + count])
+        at += count
+    width = max(len(t) for t in tables)
+    block_table = i32([t + [0] * (width - len(t)) for t in tables])
+    keys = [rnd(t, nkv, d, dtype="bfloat16", seed=10 + i) for i, t in enumerate(total)]
+    values = [rnd(t, nkv, d, dtype="bfloat16", seed=20 + i) for i, t in enumerate(total)]
+    kc = rnd(n_pages, nkv, page, d, dtype="bfloat16", seed=99)
+    vc = rnd(n_pages, nkv, d, page, dtype="bfloat16", seed=98)
+    for r, t in enumerate(total):
+        for pos in range(t):
+            kc[tables[r][pos // page], :, pos % page] = keys[r][pos]
+            vc[tables[r][pos // page], :, :, pos % page] = values[r][pos]
+    n = sum(new)
+    q = rnd(n, nq * d, dtype="bfloat16", seed=5, scale=2.0)
+    positions, entry = [], []
+    for e, (c, k) in enumerate(zip(cached, new)):
+        positions += [c + i for i in range(k)]
+        entry += [e] * k
+    scale = d ** -0.5
+    split_len = ((max(total) + splits - 1) // splits + 15) // 16 * 16
+    num_splits = (max(total) + split_len - 1) // split_len
+    out = torch.full((n, nq * d), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ops.attention_decode(q, nq * d, kc, vc, block_table, i32(entry), i32(positions), nq, window, scale,
+                         split_len, num_splits, out)
+    qh = q.float().view(n, nq, d).cpu()
+    want, at = [], 0
+    for e, k in enumerate(new):
+        want.append(dense_attention_reference(qh[at:at + k], keys[e].float().cpu(), values[e].float().cpu(),
+                                              positions[at:at + k], cached[e], window, scale))
+        at += k
+    torch.testing.assert_close(out.float().view(n, nq, d).cpu(), torch.cat(want), atol=2e-2, rtol=2e-2)
+    plain_out = ops.paged_attention_plain(q, nq * d, kc, vc, block_table, i32(entry), i32(positions), nq, window, scale)
+    torch.testing.assert_close(out.float(), plain_out.float(), atol=2e-2, rtol=2e-2)
+    # a list of tokens: only those rows are written
+    out2 = torch.zeros_like(out)
+    ops.attention_decode(q, nq * d, kc, vc, block_table, i32(entry), i32(positions), nq, window, scale,
+                         split_len, num_splits, out2, token_list=i32([9, 2]))
+    assert torch.equal(out2[[9, 2]], out[[9, 2]]) and float(out2[[0, 1, 3, 12]].abs().sum()) == 0.0
+
+
+def test_attention_decode_refuses_what_it_cannot_do():
+    q, kc, vc = rnd(1, 2 * 24, dtype="bfloat16"), rnd(2, 2, 4, 24, dtype="bfloat16"), rnd(2, 2, 24, 4, dtype="bfloat16")
+    out = torch.zeros(1, 48, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(KernelError, match="multiple of 16"):
+        ops.attention_decode(q, 48, kc, vc, i32([[0]]), i32([0]), i32([0]), 2, 0, 0.2, 16, 1, out)
+    q, kc, vc = rnd(1, 2 * 16, dtype="bfloat16"), rnd(2, 2, 6, 16, dtype="bfloat16"), rnd(2, 2, 16, 6, dtype="bfloat16")
+    out = torch.zeros(1, 32, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(KernelError, match="multiple of 4"):
+        ops.attention_decode(q, 32, kc, vc, i32([[0]]), i32([0]), i32([0]), 2, 0, 0.2, 16, 1, out)
