@@ -174,27 +174,35 @@ attention_decode_kernel(const bf16* __restrict__ q, int64_t q_stride, const bf16
     }
 }
 
-// Merge the splits of one (token, head) in split order.
-__global__ void __launch_bounds__(64)
+// Merge the splits of one (token, head) in split order.  The weights exp(m_s - m) of the splits are
+// computed once into LDS; then each thread sums one channel over the splits.
+#define COMBINE_MAX_SPLITS 1024
+__global__ void __launch_bounds__(128)
 attention_combine_kernel(const float* __restrict__ part_acc, const float* __restrict__ part_ml,
                          const int* __restrict__ token_list, int nq, int D, int num_splits,
                          bf16* __restrict__ out) {
-    const int ti = blockIdx.x, h = blockIdx.y;
+    __shared__ float factor[COMBINE_MAX_SPLITS];
+    __shared__ float red[16];
+    const int ti = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
     const int t = token_list ? token_list[ti] : ti;
     const int64_t base = ((int64_t)ti * nq + h) * num_splits;
-    float m_all = -INFINITY;
-    for (int s = 0; s < num_splits; ++s)
-        if (part_ml[(base + s) * 2 + 1] > 0.f) m_all = fmaxf(m_all, part_ml[(base + s) * 2]);
-    float l_all = 0.f;
-    for (int s = 0; s < num_splits; ++s) {
+    float mx = -INFINITY;
+    for (int s = tid; s < num_splits; s += 128)
+        if (part_ml[(base + s) * 2 + 1] > 0.f) mx = fmaxf(mx, part_ml[(base + s) * 2]);
+    const float m_all = block_max<128>(mx, red);
+    float lsum = 0.f;
+    for (int s = tid; s < num_splits; s += 128) {
         const float l = part_ml[(base + s) * 2 + 1];
-        if (l > 0.f) l_all += l * expf(part_ml[(base + s) * 2] - m_all);
+        const float f = l > 0.f ? expf(part_ml[(base + s) * 2] - m_all) : 0.f;
+        factor[s] = f;
+        lsum += l * f;
     }
-    for (int d = threadIdx.x; d < D; d += 64) {
+    const float l_all = block_sum<128>(lsum, red);      // also makes factor[] visible
+    for (int d = tid; d < D; d += 128) {
         float total = 0.f;
         for (int s = 0; s < num_splits; ++s) {
-            const float l = part_ml[(base + s) * 2 + 1];
-            if (l > 0.f) total += part_acc[(base + s) * D + d] * expf(part_ml[(base + s) * 2] - m_all);
+            const float f = factor[s];
+            if (f > 0.f) total += part_acc[(base + s) * D + d] * f;
         }
         out[((int64_t)t * nq + h) * D + d] = (bf16)(total / l_all);
     }
@@ -214,7 +222,7 @@ static int launch_decode(const void* q, int64_t q_stride, const void* kc, const 
                        (bf16*)out, part_acc, part_ml);
     SOMI_LAUNCH_CHECK("attention_decode");
     if (num_splits > 1) {
-        hipLaunchKernelGGL(attention_combine_kernel, dim3(n_list, nq), dim3(64), 0, stream, part_acc, part_ml,
+        hipLaunchKernelGGL(attention_combine_kernel, dim3(n_list, nq), dim3(128), 0, stream, part_acc, part_ml,
                            token_list, nq, DT * 16, num_splits, (bf16*)out);
         SOMI_LAUNCH_CHECK("attention_combine");
     }
@@ -237,7 +245,7 @@ extern "C" int somi_attention_decode(const void* q, int64_t q_stride, const void
     SOMI_REQUIRE(D % 16 == 0 && D >= 16 && D <= 256, "attention_decode: head_dim %d must be a multiple of 16 up to 256", D);
     SOMI_REQUIRE(page_size > 0 && page_size % 4 == 0, "attention_decode: page size %d must be a multiple of 4", page_size);
     SOMI_REQUIRE(window >= 0, "attention_decode: window must be >= 0");
-    SOMI_REQUIRE(num_splits >= 1 && num_splits <= 65535 && split_len > 0 && split_len % 16 == 0,
+    SOMI_REQUIRE(num_splits >= 1 && num_splits <= COMBINE_MAX_SPLITS && split_len > 0 && split_len % 16 == 0,
                  "attention_decode: bad split (len %d, count %d)", split_len, num_splits);
     SOMI_REQUIRE(num_splits == 1 || (part_acc && part_ml), "attention_decode: a workspace is needed for %d splits", num_splits);
     SOMI_REQUIRE((uintptr_t)q % 16 == 0 && (q_stride * 2) % 16 == 0 && (uintptr_t)k_cache % 16 == 0 &&

@@ -7,95 +7,159 @@
 // depend on what else is in the batch.
 #include "common.h"
 
-#define SAMPLE_NT 1024
+// The vocabulary is cut into chunks of SAMPLE_CHUNK entries; one workgroup per (row, chunk) finds the
+// chunk's maximum, its first index and (for a draw) the chunk's softmax mass relative to that maximum.  A
+// second kernel, one workgroup per row, merges the chunks in index order, locates the chunk that holds the
+// target mass u * total, and walks that chunk once more to pick the entry.  Chunk boundaries depend on the
+// vocabulary only, so a row's token does not depend on the batch.
+#define SAMPLE_NT 256
+#define SAMPLE_PER_THREAD 8
+#define SAMPLE_CHUNK (SAMPLE_NT * SAMPLE_PER_THREAD)
 
 __global__ void __launch_bounds__(SAMPLE_NT)
-sample_kernel(const float* __restrict__ logits, int vocab, const float* __restrict__ temperature,
-              const float* __restrict__ uniform, int* __restrict__ out) {
+sample_chunks_kernel(const float* __restrict__ logits, int vocab, int chunks, const float* __restrict__ temperature,
+                     float* __restrict__ part /*[rows, chunks, 3]: max, first index (as int bits), mass*/) {
     __shared__ float red[16];
-    __shared__ float part[SAMPLE_NT];
+    __shared__ float vals[SAMPLE_NT];
     __shared__ int idxs[SAMPLE_NT];
-    __shared__ float s_target;
-    __shared__ int s_owner;
-    const int row = blockIdx.x, tid = threadIdx.x;
+    const int row = blockIdx.y, chunk = blockIdx.x, tid = threadIdx.x;
     const float* z = logits + (int64_t)row * vocab;
     const float temp = temperature[row];
-    const int chunk = (vocab + SAMPLE_NT - 1) / SAMPLE_NT;
-    const int begin = tid * chunk < vocab ? tid * chunk : vocab;
-    const int end = begin + chunk < vocab ? begin + chunk : vocab;
-
-    if (temp == 0.f) {
-        // first index of the maximum (torch.argmax on ties is not specified; the first is the rule here)
-        float best = -INFINITY;
-        int best_i = vocab;
-        for (int i = begin; i < end; ++i) {
-            const float v = z[i];
-            if (v > best || best_i == vocab) { best = v; best_i = i; }
-        }
-        part[tid] = best;
-        idxs[tid] = best_i;
-        __syncthreads();
-        for (int step = SAMPLE_NT / 2; step > 0; step >>= 1) {
-            if (tid < step) {
-                const float ov = part[tid + step];
-                const int oi = idxs[tid + step];
-                const bool take = oi < vocab && (idxs[tid] == vocab || ov > part[tid] ||
-                                                 (ov == part[tid] && oi < idxs[tid]));
-                if (take) { part[tid] = ov; idxs[tid] = oi; }
-            }
-            __syncthreads();
-        }
-        if (tid == 0) out[row] = idxs[0];
-        return;
+    const float inv_unit = temp > 0.f ? temp : 1.f;        // greedy compares the logits themselves
+    const int begin = chunk * SAMPLE_CHUNK + tid * SAMPLE_PER_THREAD;
+    float v[SAMPLE_PER_THREAD];
+    float best = -INFINITY;
+    int best_i = vocab;
+#pragma unroll
+    for (int j = 0; j < SAMPLE_PER_THREAD; ++j) {
+        const int i = begin + j;
+        v[j] = i < vocab ? z[i] / inv_unit : -INFINITY;
+        if (i < vocab && (v[j] > best || best_i == vocab)) { best = v[j]; best_i = i; }
     }
+    vals[tid] = best;
+    idxs[tid] = best_i;
+    __syncthreads();
+    for (int step = SAMPLE_NT / 2; step > 0; step >>= 1) {
+        if (tid < step) {
+            const float ov = vals[tid + step];
+            const int oi = idxs[tid + step];
+            const bool take = oi < vocab && (idxs[tid] == vocab || ov > vals[tid] || (ov == vals[tid] && oi < idxs[tid]));
+            if (take) { vals[tid] = ov; idxs[tid] = oi; }
+        }
+        __syncthreads();
+    }
+    const float chunk_max = vals[0];
+    float mass = 0.f;
+    if (temp > 0.f) {
+#pragma unroll
+        for (int j = 0; j < SAMPLE_PER_THREAD; ++j)
+            if (begin + j < vocab) mass += expf(v[j] - chunk_max);
+        mass = block_sum<SAMPLE_NT>(mass, red);
+    }
+    if (tid == 0) {
+        float* p = part + ((int64_t)row * chunks + chunk) * 3;
+        p[0] = chunk_max;
+        p[1] = __int_as_float(idxs[0]);
+        p[2] = mass;
+    }
+}
 
-    float mx = -INFINITY;
-    for (int i = begin; i < end; ++i) mx = fmaxf(mx, z[i] / temp);
-    mx = block_max<SAMPLE_NT>(mx, red);
-    float sum = 0.f;
-    for (int i = begin; i < end; ++i) sum += expf(z[i] / temp - mx);
-    part[tid] = sum;
+__global__ void __launch_bounds__(SAMPLE_NT)
+sample_pick_kernel(const float* __restrict__ logits, int vocab, int chunks, const float* __restrict__ temperature,
+                   const float* __restrict__ uniform, const float* __restrict__ part, int* __restrict__ out) {
+    __shared__ float sums[SAMPLE_NT];
+    __shared__ float s_before, s_target, s_max;
+    __shared__ int s_chunk, s_owner;
+    const int row = blockIdx.x, tid = threadIdx.x;
+    const float* z = logits + (int64_t)row * vocab;
+    const float* p = part + (int64_t)row * chunks * 3;
+    const float temp = temperature[row];
+    if (tid == 0) {
+        float mx = -INFINITY;
+        int first = vocab;
+        for (int c = 0; c < chunks; ++c)                    // chunks in index order: the first maximum wins
+            if (p[c * 3] > mx || first == vocab) { mx = p[c * 3]; first = __float_as_int(p[c * 3 + 1]); }
+        s_max = mx;
+        if (temp == 0.f) {
+            out[row] = first;
+        } else {
+            float total = 0.f;
+            for (int c = 0; c < chunks; ++c) total += p[c * 3 + 2] * expf(p[c * 3] - mx);
+            const float target = uniform[row] * total;
+            float run = 0.f;
+            int owner = -1, last_nonzero = 0;
+            for (int c = 0; c < chunks; ++c) {
+                const float mass = p[c * 3 + 2] * expf(p[c * 3] - mx);
+                if (mass > 0.f) last_nonzero = c;
+                if (owner < 0 && target < run + mass) { owner = c; s_before = run; }
+                run += mass;
+            }
+            if (owner < 0) {                                // rounding pushed the target past the total
+                owner = last_nonzero;
+                s_before = -INFINITY;                       // take the chunk's last entry with mass
+            }
+            s_chunk = owner;
+            s_target = target;
+        }
+    }
+    __syncthreads();
+    if (temp == 0.f) return;
+    const int begin = s_chunk * SAMPLE_CHUNK + tid * SAMPLE_PER_THREAD;
+    float w[SAMPLE_PER_THREAD];
+    float mine = 0.f;
+#pragma unroll
+    for (int j = 0; j < SAMPLE_PER_THREAD; ++j) {
+        w[j] = begin + j < vocab ? expf(z[begin + j] / temp - s_max) : 0.f;
+        mine += w[j];
+    }
+    sums[tid] = mine;
     __syncthreads();
     if (tid == 0) {
-        // exclusive prefix of the per-thread masses, in index order
-        float run = 0.f;
+        const bool overshoot = s_before == -INFINITY;
+        float run = overshoot ? 0.f : s_before;
         int owner = -1, last_nonzero = 0;
         for (int k = 0; k < SAMPLE_NT; ++k) {
-            const float mass = part[k];
-            part[k] = run;
+            const float mass = sums[k];
+            sums[k] = run;
             if (mass > 0.f) last_nonzero = k;
+            if (!overshoot && owner < 0 && s_target < run + mass) owner = k;
             run += mass;
         }
-        const float target = uniform[row] * run;
-        for (int k = 0; k < SAMPLE_NT; ++k) {
-            const float hi = (k + 1 < SAMPLE_NT) ? part[k + 1] : run;
-            if (target >= part[k] && target < hi) { owner = k; break; }
-        }
         s_owner = owner < 0 ? last_nonzero : owner;
-        s_target = target;
     }
     __syncthreads();
     if (tid == s_owner) {
-        float run = part[tid];
+        float run = sums[tid];
         int pick = -1, last = begin;
-        for (int i = begin; i < end; ++i) {
-            const float w = expf(z[i] / temp - mx);
-            if (w > 0.f) last = i;
-            run += w;
-            if (run > s_target) { pick = i; break; }
+#pragma unroll
+        for (int j = 0; j < SAMPLE_PER_THREAD; ++j) {
+            if (w[j] > 0.f) last = begin + j;
+            run += w[j];
+            if (pick < 0 && s_before != -INFINITY && run > s_target) pick = begin + j;
         }
         out[row] = pick < 0 ? last : pick;
     }
 }
 
-// logits: [rows, vocab] float32; temperature, uniform: [rows] float32 (uniform in [0, 1)); out: [rows] int32.
+extern "C" int somi_sample_workspace_floats(int rows, int vocab) {
+    return rows * ceil_div(vocab, SAMPLE_CHUNK) * 3;
+}
+
+// logits: [rows, vocab] float32; temperature, uniform: [rows] float32 (uniform in [0, 1)); out: [rows] int32;
+// workspace: somi_sample_workspace_floats(rows, vocab) floats.
 extern "C" int somi_sample(const float* logits, int rows, int vocab, const float* temperature,
-                           const float* uniform, int* out, hipStream_t stream) {
+                           const float* uniform, int* out, float* workspace, hipStream_t stream) {
     SOMI_REQUIRE(rows >= 0 && vocab > 0, "sample: bad sizes rows=%d vocab=%d", rows, vocab);
+    SOMI_REQUIRE(rows <= 65535, "sample: too many rows");
+    SOMI_REQUIRE(workspace != nullptr || rows == 0, "sample: a workspace is needed");
     if (rows == 0) return 0;
-    hipLaunchKernelGGL(sample_kernel, dim3(rows), dim3(SAMPLE_NT), 0, stream, logits, vocab, temperature, uniform,
-                       out);
-    SOMI_LAUNCH_CHECK("sample");
+    const int chunks = ceil_div(vocab, SAMPLE_CHUNK);
+    hipLaunchKernelGGL(sample_chunks_kernel, dim3(chunks, rows), dim3(SAMPLE_NT), 0, stream, logits, vocab, chunks,
+                       temperature, workspace);
+    SOMI_LAUNCH_CHECK("sample_chunks");
+    hipLaunchKernelGGL(sample_pick_kernel, dim3(rows), dim3(SAMPLE_NT), 0, stream, logits, vocab, chunks, temperature,
+                       uniform, workspace, out);
+    SOMI_LAUNCH_CHECK("sample_pick");
     return 0;
 }
 

@@ -8,6 +8,7 @@ from . import ops
 
 TARGET_WORKGROUPS = 1024        # about four per compute unit
 MIN_SPLIT = 64                  # keys per split at least (a multiple of the 16-key tile)
+MAX_SPLITS = 1024               # what the merge kernel holds
 
 
 def decode_splits(num_tokens: int, groups: int, max_context: int) -> tuple[int, int]:
@@ -16,7 +17,7 @@ def decode_splits(num_tokens: int, groups: int, max_context: int) -> tuple[int, 
     MIN_SPLIT in absolute positions."""
     max_context = max(1, max_context)
     most = (max_context + MIN_SPLIT - 1) // MIN_SPLIT
-    splits = max(1, min(TARGET_WORKGROUPS // max(1, num_tokens * groups), most))
+    splits = max(1, min(TARGET_WORKGROUPS // max(1, num_tokens * groups), most, MAX_SPLITS))
     split_len = ((max_context + splits - 1) // splits + MIN_SPLIT - 1) // MIN_SPLIT * MIN_SPLIT
     return split_len, (max_context + split_len - 1) // split_len
 
@@ -41,7 +42,6 @@ def paged_attention(qkv: torch.Tensor, num_heads: int, k_cache: torch.Tensor, v_
     nkv, head_dim = k_cache.shape[1], k_cache.shape[3]
     groups = nkv * ((num_heads // nkv + 15) // 16)
     out = torch.empty((qkv.shape[0], num_heads * head_dim), dtype=qkv.dtype, device=qkv.device)
-    reach = min(step.max_context, window + step.max_entry_len) if window else step.max_context
     split_len, num_splits = decode_splits(step.num_tokens, groups, step.max_context)
     ops.attention_decode(qkv, qkv.shape[1], k_cache, v_cache, block_table, step.token_entry, step.positions,
                          num_heads, window, scale, split_len, num_splits, out)

@@ -256,7 +256,10 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, uniform: torch.Tenso
     _need(temperature, "temperature", torch.float32, (rows,))
     _need(uniform, "uniform", torch.float32, (rows,))
     out = torch.empty((rows,), dtype=torch.int32, device=logits.device)
-    _check(library().somi_sample(_ptr(logits), rows, vocab, _ptr(temperature), _ptr(uniform), _ptr(out), _stream()))
+    workspace = torch.empty((max(1, library().somi_sample_workspace_floats(rows, vocab)),), dtype=torch.float32,
+                            device=logits.device)
+    _check(library().somi_sample(_ptr(logits), rows, vocab, _ptr(temperature), _ptr(uniform), _ptr(out),
+                                 _ptr(workspace), _stream()))
     return out
 
 
