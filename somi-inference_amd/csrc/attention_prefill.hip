@@ -1,0 +1,231 @@
+// Causal attention of prompt portions over the paged cache, bfloat16, on the matrix cores.
+//
+// Reference: somi_inference/models/qwen2.py:158-186 (scores, causal mask, float32 softmax, weights . v;
+// query head h reads key/value head h // (nq / nkv)) and the flash-style Triton kernel
+// somi_inference/core/flash_attention_triton.py:31-194 (query tiles against key tiles with a running
+// maximum and sum, base-2 exponentials with the scale folded in, :26, 119-120, 286).  The reference's
+// kernel sees only the tokens of its own call on contiguous tensors; this one reads keys and values through
+// the block table, so a portion attends to everything cached before it and to itself: the step's keys
+// and values are written to their pages before the launch.
+//
+// A wavefront owns QB blocks of 16 consecutive query tokens of one (request portion, query head) and walks
+// the keys 32 at a time:
+//   S^T[key, query] = K[key, :] . Q^T        v_mfma_f32_16x16x32_bf16, K rows as the A operand (16 B loads)
+//   online softmax per query (= per lane column) in float32, base 2
+//   O^T[d, query] += V^T[d, key] . P^T       v_mfma_f32_16x16x32_bf16; the two 16-key halves of P^T leave the
+//                                            first product in the B-operand layout, and V is stored transposed
+//                                            inside a page, so a lane reads 2 x 4 consecutive keys of a channel
+// Every key tile is used for all QB query blocks from registers.  Key tiles are aligned to absolute
+// positions (multiples of 32), so a query's arithmetic does not depend on how the prompt was cut.
+#include "common.h"
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(4))) short short4_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+__device__ __forceinline__ bf16x8 pld8(const bf16* p) { return *reinterpret_cast<const bf16x8*>(p); }
+__device__ __forceinline__ short4_t pld4(const bf16* p) { return *reinterpret_cast<const short4_t*>(p); }
+__device__ __forceinline__ bf16x8 phalf(const bf16* p) {
+    union { bf16x8 wide; short4_t half[2]; } u;
+    u.half[0] = pld4(p);
+    u.half[1] = short4_t{0, 0, 0, 0};
+    return u.wide;
+}
+__device__ __forceinline__ bf16x8 pjoin(short4_t lo, short4_t hi) {
+    union { bf16x8 wide; short4_t half[2]; } u;
+    u.half[0] = lo;
+    u.half[1] = hi;
+    return u.wide;
+}
+
+template <int DT, int QB>
+__global__ void __launch_bounds__(256)
+attention_prefill_kernel(const bf16* __restrict__ q, int64_t q_stride, const bf16* __restrict__ kc,
+                         const bf16* __restrict__ vc, const int* __restrict__ block_table, int max_blocks,
+                         const int* __restrict__ entry_start, const int* __restrict__ entry_first_pos, int nq,
+                         int nkv, int page_size, int window, float scale_log2, bf16* __restrict__ out) {
+    constexpr int D = DT * 16;
+    constexpr int QK_STEPS = (DT + 1) / 2;
+    constexpr int QW = QB * 16;                         // queries per wavefront
+    const int e = blockIdx.y, h = blockIdx.z;
+    const int kvh = h / (nq / nkv);
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4;
+    const int start = entry_start[e];
+    const int len = entry_start[e + 1] - start;
+    const int q0 = (blockIdx.x * (blockDim.x >> 6) + wave) * QW;
+    if (q0 >= len) return;                              // no workgroup barrier is used below
+    const int pos0 = entry_first_pos[e];
+    const int nvalid = len - q0 < QW ? len - q0 : QW;
+    const int* table = block_table + (int64_t)e * max_blocks;
+
+    // queries: column r of block qb is token start + q0 + 16 qb + r (past the portion's end: its last token,
+    // computed again and not stored)
+    bf16x8 qf[QB][QK_STEPS];
+    int pcol[QB];
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb) {
+        int qi = q0 + qb * 16 + r;
+        qi = qi < len ? qi : len - 1;
+        pcol[qb] = pos0 + qi;
+        const bf16* qrow = q + (int64_t)(start + qi) * q_stride + (int64_t)h * D;
+#pragma unroll
+        for (int c = 0; c < DT / 2; ++c) qf[qb][c] = pld8(qrow + c * 32 + g * 8);
+        if (DT & 1) qf[qb][QK_STEPS - 1] = phalf(qrow + (DT - 1) * 16 + g * 4);
+    }
+    const int p_first = pos0 + q0, p_last = pos0 + q0 + nvalid - 1;
+    const int lo = (window > 0 && p_first - window + 1 > 0) ? p_first - window + 1 : 0;
+
+    float m_run[QB], l_run[QB];
+    f32x4 acc[QB][DT];
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb) {
+        m_run[qb] = -INFINITY;
+        l_run[qb] = 0.f;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) acc[qb][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+
+    const int vlo = lo & ~3, vhi = p_last & ~3;
+    for (int j0 = lo & ~31; j0 <= p_last; j0 += 32) {
+        // keys of the two 16-key halves: lane reads rows j0 + r and j0 + 16 + r (addresses kept inside the
+        // visible range; what lies outside is masked below)
+        bf16x8 kf[2][QK_STEPS];
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+            int pos = j0 + half * 16 + r;
+            pos = pos < lo ? lo : (pos > p_last ? p_last : pos);
+            const int64_t page = table[pos / page_size];
+            const bf16* krow = kc + ((page * nkv + kvh) * page_size + pos % page_size) * (int64_t)D;
+#pragma unroll
+            for (int c = 0; c < DT / 2; ++c) kf[half][c] = pld8(krow + c * 32 + g * 8);
+            if (DT & 1) kf[half][QK_STEPS - 1] = phalf(krow + (DT - 1) * 16 + g * 4);
+        }
+        // values: channel dt * 16 + r at keys j0 + 4 g .. + 3 and j0 + 16 + 4 g .. + 3
+        bf16x8 vf[DT];
+        {
+            int va = j0 + g * 4, vb = j0 + 16 + g * 4;
+            va = va < vlo ? vlo : (va > vhi ? vhi : va);
+            vb = vb < vlo ? vlo : (vb > vhi ? vhi : vb);
+            const int64_t pa = table[va / page_size], pb = table[vb / page_size];
+            const bf16* vbase_a = vc + (pa * nkv + kvh) * (int64_t)D * page_size + va % page_size;
+            const bf16* vbase_b = vc + (pb * nkv + kvh) * (int64_t)D * page_size + vb % page_size;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+                vf[dt] = pjoin(pld4(vbase_a + (int64_t)(dt * 16 + r) * page_size),
+                               pld4(vbase_b + (int64_t)(dt * 16 + r) * page_size));
+        }
+#pragma unroll
+        for (int qb = 0; qb < QB; ++qb) {
+            f32x4 s[2];
+#pragma unroll
+            for (int half = 0; half < 2; ++half) {
+                s[half] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int c = 0; c < QK_STEPS; ++c)
+                    s[half] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[half][c], qf[qb][c], s[half], 0, 0, 0);
+            }
+            // s[half][i] = S[key j0 + 16 half + 4 g + i][query column r of block qb]
+            const int p = pcol[qb];
+            const int first = window > 0 ? p - window + 1 : 0;
+            float mx = -INFINITY;
+#pragma unroll
+            for (int half = 0; half < 2; ++half)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int key = j0 + half * 16 + g * 4 + i;
+                    s[half][i] = (key <= p && key >= first) ? s[half][i] * scale_log2 : -INFINITY;
+                    mx = fmaxf(mx, s[half][i]);
+                }
+            mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            const float m_new = fmaxf(m_run[qb], mx);
+            const float m_use = m_new == -INFINITY ? 0.f : m_new;     // nothing visible yet: weights stay 0
+            const float corr = exp2f(m_run[qb] - m_use);
+            float pr[2][4], sum = 0.f;
+#pragma unroll
+            for (int half = 0; half < 2; ++half)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    pr[half][i] = exp2f(s[half][i] - m_use);
+                    sum += pr[half][i];
+                }
+            sum += __shfl_xor(sum, 16, 64);
+            sum += __shfl_xor(sum, 32, 64);
+            l_run[qb] = l_run[qb] * corr + sum;
+            m_run[qb] = m_new;
+            const bf16x8 pf = {(bf16)pr[0][0], (bf16)pr[0][1], (bf16)pr[0][2], (bf16)pr[0][3],
+                               (bf16)pr[1][0], (bf16)pr[1][1], (bf16)pr[1][2], (bf16)pr[1][3]};
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                acc[qb][dt] *= corr;
+                acc[qb][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt], pf, acc[qb][dt], 0, 0, 0);
+            }
+        }
+    }
+
+    // acc[qb][dt][i] = O^T[d = dt * 16 + 4 g + i][query column r]
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb) {
+        const int qi = q0 + qb * 16 + r;
+        if (qi >= len) continue;
+        const float inv = 1.0f / l_run[qb];
+        bf16* orow = out + ((int64_t)(start + qi) * nq + h) * D + g * 4;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+            const bf16x4 o = {(bf16)(acc[qb][dt][0] * inv), (bf16)(acc[qb][dt][1] * inv),
+                              (bf16)(acc[qb][dt][2] * inv), (bf16)(acc[qb][dt][3] * inv)};
+            *reinterpret_cast<bf16x4*>(orow + dt * 16) = o;
+        }
+    }
+}
+
+template <int DT, int QB>
+static int launch_prefill(const void* q, int64_t q_stride, const void* kc, const void* vc, const int* block_table,
+                          int max_blocks, const int* entry_start, const int* entry_first_pos, int n_entries,
+                          int max_entry_len, int nq, int nkv, int page_size, int window, float scale, void* out,
+                          hipStream_t stream) {
+    constexpr int WAVES = 4;
+    const int per_group = WAVES * QB * 16;
+    const dim3 grid(ceil_div(max_entry_len, per_group), n_entries, nq);
+    hipLaunchKernelGGL((attention_prefill_kernel<DT, QB>), grid, dim3(WAVES * 64), 0, stream, (const bf16*)q, q_stride,
+                       (const bf16*)kc, (const bf16*)vc, block_table, max_blocks, entry_start, entry_first_pos, nq, nkv,
+                       page_size, window, scale * 1.44269504088896341f, (bf16*)out);
+    SOMI_LAUNCH_CHECK("attention_prefill");
+    return 0;
+}
+
+// Attention of every token of every entry (portion) over its request's pages.  entry_start: [n_entries + 1]
+// offsets of the portions in the flat token batch; entry_first_pos: [n_entries] position of each portion's
+// first token; max_entry_len: the longest portion (sizes the grid).  bfloat16 only; head_dim a multiple of 16
+// up to 256; page_size a multiple of 4.  k_cache [pages, nkv, page_size, D], v_cache [pages, nkv, D, page_size];
+// out: [n_tokens, nq * D].
+extern "C" int somi_attention_prefill(const void* q, int64_t q_stride, const void* k_cache, const void* v_cache,
+                                      const int* block_table, int max_blocks, const int* entry_start,
+                                      const int* entry_first_pos, int n_entries, int max_entry_len, int nq, int nkv,
+                                      int D, int page_size, int window, float scale, void* out, hipStream_t stream) {
+    SOMI_REQUIRE(n_entries >= 0 && max_entry_len >= 0 && nq > 0 && nkv > 0 && max_blocks > 0,
+                 "attention_prefill: bad sizes");
+    SOMI_REQUIRE(nq % nkv == 0, "attention_prefill: num_q_heads (%d) must be divisible by num_kv_heads (%d)", nq, nkv);
+    SOMI_REQUIRE(D % 16 == 0 && D >= 16 && D <= 256, "attention_prefill: head_dim %d must be a multiple of 16 up to 256", D);
+    SOMI_REQUIRE(page_size > 0 && page_size % 4 == 0, "attention_prefill: page size %d must be a multiple of 4", page_size);
+    SOMI_REQUIRE(window >= 0, "attention_prefill: window must be >= 0");
+    SOMI_REQUIRE(n_entries <= 65535 && nq <= 65535, "attention_prefill: too many entries or heads");
+    SOMI_REQUIRE((uintptr_t)q % 16 == 0 && (q_stride * 2) % 16 == 0 && (uintptr_t)k_cache % 16 == 0 &&
+                 (uintptr_t)v_cache % 8 == 0 && (uintptr_t)out % 8 == 0,
+                 "attention_prefill: q, k, v and out must be 16-byte aligned");
+    if (n_entries == 0 || max_entry_len == 0) return 0;
+#define SOMI_PREFILL(DT, QB)                                                                                       \
+    case DT:                                                                                                       \
+        return launch_prefill<DT, QB>(q, q_stride, k_cache, v_cache, block_table, max_blocks, entry_start,         \
+                                      entry_first_pos, n_entries, max_entry_len, nq, nkv, page_size, window, scale, \
+                                      out, stream)
+    switch (D / 16) {
+        SOMI_PREFILL(1, 4); SOMI_PREFILL(2, 4); SOMI_PREFILL(3, 4); SOMI_PREFILL(4, 4); SOMI_PREFILL(5, 4);
+        SOMI_PREFILL(6, 4); SOMI_PREFILL(7, 4); SOMI_PREFILL(8, 4); SOMI_PREFILL(9, 2); SOMI_PREFILL(10, 2);
+        SOMI_PREFILL(11, 2); SOMI_PREFILL(12, 2); SOMI_PREFILL(13, 2); SOMI_PREFILL(14, 2); SOMI_PREFILL(15, 2);
+        SOMI_PREFILL(16, 2);
+    }
+#undef SOMI_PREFILL
+    return somi_fail("attention_prefill: unsupported head_dim %d", D);
+}

@@ -9,6 +9,7 @@ from . import ops
 TARGET_WORKGROUPS = 1024        # about four per compute unit
 MIN_SPLIT = 64                  # keys per split at least (a multiple of the 16-key tile)
 MAX_SPLITS = 1024               # what the merge kernel holds
+DECODE_PORTION = 8              # batches whose longest portion is at most this take the decode kernel
 
 
 def decode_splits(num_tokens: int, groups: int, max_context: int) -> tuple[int, int]:
@@ -42,6 +43,12 @@ def paged_attention(qkv: torch.Tensor, num_heads: int, k_cache: torch.Tensor, v_
     nkv, head_dim = k_cache.shape[1], k_cache.shape[3]
     groups = nkv * ((num_heads // nkv + 15) // 16)
     out = torch.empty((qkv.shape[0], num_heads * head_dim), dtype=qkv.dtype, device=qkv.device)
+    if step.max_entry_len > DECODE_PORTION:
+        # portions of prompts: query tiles against key tiles (single tokens in the same batch ride along
+        # as portions of one)
+        ops.attention_prefill(qkv, qkv.shape[1], k_cache, v_cache, block_table, step.entry_start,
+                              step.entry_first_position, step.max_entry_len, num_heads, window, scale, out)
+        return out
     split_len, num_splits = decode_splits(step.num_tokens, groups, step.max_context)
     ops.attention_decode(qkv, qkv.shape[1], k_cache, v_cache, block_table, step.token_entry, step.positions,
                          num_heads, window, scale, split_len, num_splits, out)

@@ -238,6 +238,34 @@ def attention_decode(q: torch.Tensor, q_stride: int, k_cache: torch.Tensor, v_ca
         ctypes.c_float(scale), split_len, num_splits, _ptr(out), _ptr(part_acc), _ptr(part_ml), _stream()))
 
 
+def attention_prefill(q: torch.Tensor, q_stride: int, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                      block_table: torch.Tensor, entry_start: torch.Tensor, entry_first_position: torch.Tensor,
+                      max_entry_len: int, nq: int, window: int, scale: float, out: torch.Tensor) -> None:
+    """MFMA causal attention of every token of every portion over its request's pages, into ``out``
+    ([N, nq * D] bfloat16).  entry_start: [E + 1] int32 offsets of the portions in the flat batch;
+    entry_first_position: [E] int32."""
+    _need(q, "q", torch.bfloat16)
+    n = q.shape[0]
+    _need(k_cache, "k cache", torch.bfloat16)
+    if k_cache.dim() != 4:
+        raise KernelError("attention_prefill: the k cache must be [pages, kv_heads, page_size, head_dim]")
+    _need(v_cache, "v cache", torch.bfloat16, _v_shape(k_cache))
+    _, nkv, page_size, head_dim = k_cache.shape
+    if q_stride < nq * head_dim or q.shape[1] < nq * head_dim:
+        raise KernelError("attention_prefill: q rows are narrower than nq * head_dim")
+    _need(block_table, "block table", torch.int32)
+    entries = block_table.shape[0]
+    _need(entry_start, "entry offsets", torch.int32, (entries + 1,))
+    _need(entry_first_position, "entry first positions", torch.int32, (entries,))
+    _need(out, "attention out", torch.bfloat16, (n, nq * head_dim))
+    if not 0 <= max_entry_len <= n:
+        raise KernelError(f"attention_prefill: longest portion {max_entry_len} does not fit {n} tokens")
+    _check(library().somi_attention_prefill(
+        _ptr(q), ctypes.c_int64(q_stride), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), block_table.shape[1],
+        _ptr(entry_start), _ptr(entry_first_position), entries, max_entry_len, nq, nkv, head_dim, page_size, window,
+        ctypes.c_float(scale), _ptr(out), _stream()))
+
+
 def silu_mul(gate_up: torch.Tensor) -> torch.Tensor:
     """silu(gate_up[:, :I]) * gate_up[:, I:]."""
     _need(gate_up, "gate_up")

@@ -311,3 +311,49 @@ def test_attention_decode_refuses_what_it_cannot_do():
     out = torch.zeros(1, 32, dtype=torch.bfloat16, device=DEV)
     with pytest.raises(KernelError, match="multiple of 4"):
         ops.attention_decode(q, 32, kc, vc, i32([[0]]), i32([0]), i32([0]), 2, 0, 0.2, 16, 1, out)
+
+
+@pytest.mark.parametrize("nq, nkv, d, page, window", [
+    (8, 4, 32, 4, 0), (12, 2, 64, 16, 0), (8, 1, 48, 8, 0), (6, 3, 128, 16, 37), (28, 4, 128, 16, 0),
+    (4, 2, 16, 8, 0), (14, 2, 256, 16, 0), (5, 5, 80, 4, 5), (7, 1, 112, 32, 100), (3, 1, 208, 16, 0)])
+def test_attention_prefill_mfma_against_dense_softmax(nq, nkv, d, page, window):
+    """Portions of several requests in one launch: a long one that starts at position 0, one that continues
+    after 150 cached tokens, a portion of two tokens, single tokens after 77 and after 0 cached ones."""
+    cached, new = [0, 150, 30, 77, 0], [203, 130, 2, 1, 1]
+    total = [c + n for c, n in zip(cached, new)]
+    n_pages = sum((t + page - 1) // page for t in total) + 3
+    perm = torch.randperm(n_pages, generator=torch.Generator().manual_seed(4)).tolist()
+    tables, at = [], 0
+    for t in total:
+        count = (t + page - 1) // page
+        tables.append(perm[at:at + count])
+        at += count
+    width = max(len(t) for t in tables)
+    block_table = i32([t + [0] * (width - len(t)) for t in tables])
+    keys = [rnd(t, nkv, d, dtype="bfloat16", seed=10 + i) for i, t in enumerate(total)]
+    values = [rnd(t, nkv, d, dtype="bfloat16", seed=20 + i) for i, t in enumerate(total)]
+    kc = rnd(n_pages, nkv, page, d, dtype="bfloat16", seed=99)
+    vc = rnd(n_pages, nkv, d, page, dtype="bfloat16", seed=98)
+    for r, t in enumerate(total):
+        for pos in range(t):
+            kc[tables[r][pos // page], :, pos % page] = keys[r][pos]
+            vc[tables[r][pos // page], :, :, pos % page] = values[r][pos]
+    n = sum(new)
+    q = rnd(n, nq * d, dtype="bfloat16", seed=5, scale=2.0)
+    positions, entry, starts = [], [], [0]
+    for e, (c, k) in enumerate(zip(cached, new)):
+        positions += [c + i for i in range(k)]
+        entry += [e] * k
+        starts.append(starts[-1] + k)
+    scale = d ** -0.5
+    out = torch.full((n, nq * d), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ops.attention_prefill(q, nq * d, kc, vc, block_table, i32(starts), i32(cached), max(new), nq, window, scale, out)
+    qh = q.float().view(n, nq, d).cpu()
+    want, at = [], 0
+    for e, k in enumerate(new):
+        want.append(dense_attention_reference(qh[at:at + k], keys[e].float().cpu(), values[e].float().cpu(),
+                                              positions[at:at + k], cached[e], window, scale))
+        at += k
+    torch.testing.assert_close(out.float().view(n, nq, d).cpu(), torch.cat(want), atol=2e-2, rtol=2e-2)
+    plain_out = ops.paged_attention_plain(q, nq * d, kc, vc, block_table, i32(entry), i32(positions), nq, window, scale)
+    torch.testing.assert_close(out.float(), plain_out.float(), atol=2e-2, rtol=2e-2)
