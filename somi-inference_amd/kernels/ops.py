@@ -266,14 +266,31 @@ def attention_prefill(q: torch.Tensor, q_stride: int, k_cache: torch.Tensor, v_c
         ctypes.c_float(scale), _ptr(out), _stream()))
 
 
-def silu_mul(gate_up: torch.Tensor) -> torch.Tensor:
-    """silu(gate_up[:, :I]) * gate_up[:, I:]."""
+def silu_mul(gate_up: torch.Tensor, block: int = 0) -> torch.Tensor:
+    """silu(gate) * up.  block == 0: gate_up = [gate | up]; block == b: gate and up columns interleaved
+    in blocks of b columns (gate 0..b-1, up 0..b-1, gate b..2b-1, ...)."""
     _need(gate_up, "gate_up")
     n, two_i = gate_up.shape
     if two_i % 2:
         raise KernelError(f"silu_mul: width {two_i} is odd")
     out = torch.empty((n, two_i // 2), dtype=gate_up.dtype, device=gate_up.device)
-    _check(library().somi_silu_mul(_ptr(gate_up), _ptr(out), dtype_code(gate_up.dtype), n, two_i // 2, _stream()))
+    _check(library().somi_silu_mul(_ptr(gate_up), _ptr(out), dtype_code(gate_up.dtype), n, two_i // 2, block,
+                                   _stream()))
+    return out
+
+
+def linear_skinny_swiglu(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+    """silu(x @ gate.T) * (x @ up.T) in one kernel for at most 64 bfloat16 rows.  weight: [2 I, K] with
+    gate and up rows interleaved in blocks of 16."""
+    _need(x, "linear input", torch.bfloat16)
+    m, k = x.shape
+    _need(weight, "gate_up weight", torch.bfloat16)
+    if weight.shape[1] != k or weight.shape[0] % 32:
+        raise KernelError(f"linear_skinny_swiglu: weight {tuple(weight.shape)} does not fit input width {k}")
+    inter = weight.shape[0] // 2
+    out = torch.empty((m, inter), dtype=x.dtype, device=x.device)
+    _check(library().somi_linear_skinny_swiglu(_ptr(x), _ptr(weight), _ptr(out), dtype_code(x.dtype), m, inter, k,
+                                               _stream()))
     return out
 
 

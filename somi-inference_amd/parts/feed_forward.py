@@ -4,6 +4,7 @@ from __future__ import annotations
 
 import torch
 
+from ..kernels import linear as linear_kernels
 from ..kernels import ops
 from ..weights.spec import MATRIX, WeightSpec
 from .base import FeedForward, Fetch, Runtime
@@ -26,10 +27,27 @@ class SwiGLU(FeedForward):
                 WeightSpec(self.name("up_proj.weight"), (i, h), MATRIX),
                 WeightSpec(self.name("down_proj.weight"), (h, i), MATRIX)]
 
+    INTERLEAVE = 16       # rows per block when gate and up are interleaved for the fused kernel
+
     def load(self, fetch: Fetch, runtime: Runtime) -> None:
         super().load(fetch, runtime)
-        self.gate_up = Projection.stacked([fetch(self.name("gate_proj.weight")), fetch(self.name("up_proj.weight"))])
+        gate, up = fetch(self.name("gate_proj.weight")), fetch(self.name("up_proj.weight"))
+        # The layout of the merged matrix is private.  In bfloat16 the rows are interleaved in blocks of 16
+        # (gate 0..15, up 0..15, gate 16..31, ...), so that the decode kernel has gate and up of the same
+        # columns in one workgroup and applies the gate in its epilogue.
+        self.interleaved = (runtime.dtype == torch.bfloat16 and self.intermediate_size % self.INTERLEAVE == 0
+                            and self.hidden_size % 8 == 0)
+        if self.interleaved:
+            b, h = self.INTERLEAVE, self.hidden_size
+            merged = torch.stack([gate.view(-1, b, h), up.view(-1, b, h)], dim=1).reshape(-1, h).contiguous()
+            self.gate_up = Projection(merged)
+        else:
+            self.gate_up = Projection.stacked([gate, up])
         self.down = Projection(fetch(self.name("down_proj.weight")))
 
     def forward(self, x: torch.Tensor, step=None) -> torch.Tensor:
-        return self.down(ops.silu_mul(self.gate_up(x)))
+        if not self.interleaved:
+            return self.down(ops.silu_mul(self.gate_up(x)))
+        if x.shape[0] <= linear_kernels.SKINNY_ROWS and x.data_ptr() % 16 == 0:
+            return self.down(ops.linear_skinny_swiglu(x, self.gate_up.weight))
+        return self.down(ops.silu_mul(self.gate_up(x), block=self.INTERLEAVE))

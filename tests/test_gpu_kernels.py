@@ -357,3 +357,19 @@ def test_attention_prefill_mfma_against_dense_softmax(nq, nkv, d, page, window):
     torch.testing.assert_close(out.float().view(n, nq, d).cpu(), torch.cat(want), atol=2e-2, rtol=2e-2)
     plain_out = ops.paged_attention_plain(q, nq * d, kc, vc, block_table, i32(entry), i32(positions), nq, window, scale)
     torch.testing.assert_close(out.float(), plain_out.float(), atol=2e-2, rtol=2e-2)
+
+
+@pytest.mark.parametrize("m, inter, k", [(1, 48, 72), (8, 18944 // 8, 512), (17, 160, 200), (40, 4096 + 32, 64), (64, 32, 3584)])
+def test_linear_skinny_with_the_gate_fused_in(m, inter, k):
+    x = rnd(m, k, dtype="bfloat16", seed=1)
+    gate, up = rnd(inter, k, dtype="bfloat16", seed=2, scale=0.1), rnd(inter, k, dtype="bfloat16", seed=3, scale=0.1)
+    merged = torch.stack([gate.view(-1, 16, k), up.view(-1, 16, k)], dim=1).reshape(-1, k).contiguous()
+    want = F.silu(x.float() @ gate.float().t()) * (x.float() @ up.float().t())
+    got = ops.linear_skinny_swiglu(x, merged)
+    scale = float(want.abs().max())
+    torch.testing.assert_close(got.float(), want, atol=scale * 2 ** -7, rtol=2 ** -6)
+    # the unfused way over the same interleaved matrix
+    unfused = ops.silu_mul(ops.linear_skinny(x, merged), block=16)
+    torch.testing.assert_close(unfused.float(), want, atol=scale * 2 ** -6, rtol=2 ** -5)
+    with pytest.raises(KernelError, match="does not fit"):
+        ops.linear_skinny_swiglu(x, merged[:-16].contiguous())
