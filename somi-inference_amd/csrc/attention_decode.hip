@@ -174,6 +174,215 @@ attention_decode_kernel(const bf16* __restrict__ q, int64_t q_stride, const bf16
     }
 }
 
+// The same with the keys and values of a split staged through LDS, 32 keys at a time: all 256 threads
+// fetch the next 32 keys and values into registers while the current ones are used from LDS (many bytes
+// in flight per workgroup, which is what a bandwidth-bound kernel needs).  Every wavefront computes the
+// scores and the softmax of the 32 keys (a few products), then applies the weights to its own quarter of
+// the head's channels, so the output needs no merge across wavefronts.
+typedef __attribute__((ext_vector_type(2))) unsigned u32x2;
+__device__ __forceinline__ float lanes4_max(float v) {       // over lanes l, l ^ 16, l ^ 32, l ^ 48
+    u32x2 a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    v = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+    u32x2 b = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+__device__ __forceinline__ float lanes4_sum(float v) {
+    u32x2 a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    v = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+    u32x2 b = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return __uint_as_float(b[0]) + __uint_as_float(b[1]);
+}
+
+#define DECODE_LDS_PAGES 512
+template <int DT>
+__global__ void __launch_bounds__(256)
+attention_decode_lds_kernel(const bf16* __restrict__ q, int64_t q_stride, const bf16* __restrict__ kc,
+                            const bf16* __restrict__ vc, const int* __restrict__ block_table, int max_blocks,
+                            const int* __restrict__ token_list, const int* __restrict__ token_entry,
+                            const int* __restrict__ positions, int nq, int nkv, int page_size, int window,
+                            float scale, int split_len, int num_splits, bf16* __restrict__ out,
+                            float* __restrict__ part_acc, float* __restrict__ part_ml) {
+    constexpr int D = DT * 16;
+    constexpr int QK_STEPS = (DT + 1) / 2;
+    constexpr int KROW = D + 8, VROW = 32 + 4;               // padded LDS rows, in elements
+    constexpr int K_CHUNKS = 32 * D / 8;                     // 16-byte pieces of a 32-key tile
+    constexpr int K_PER_THREAD = (K_CHUNKS + 255) / 256;
+    constexpr int V_PER_THREAD = (D + 31) / 32;              // 8-byte pieces: key group tid % 8 of channels tid / 8 + 32 i
+    constexpr int MY_TILES = (DT + 3) / 4;                   // channel tiles of one wavefront: dt = wave + 4 i
+    __shared__ __attribute__((aligned(16))) bf16 ks[2][32 * KROW];
+    __shared__ __attribute__((aligned(16))) bf16 vs[2][D * VROW];
+    __shared__ int pages[DECODE_LDS_PAGES];
+
+    const int ti = blockIdx.x;
+    const int t = token_list ? token_list[ti] : ti;
+    const int G = nq / nkv, HB = (G + 15) / 16;
+    const int kvh = blockIdx.y / HB, hb = blockIdx.y % HB;
+    const int split = blockIdx.z;
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, r = lane & 15, g = lane >> 4;
+
+    const int p = positions[t];
+    const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+    const int* table = block_table + (int64_t)token_entry[t] * max_blocks;
+    const int begin = lo > split * split_len ? lo : split * split_len;
+    const int end = p < (split + 1) * split_len - 1 ? p : (split + 1) * split_len - 1;      // inclusive
+    const int hloc = hb * 16 + r;
+    const int head = kvh * G + (hloc < G ? hloc : G - 1);
+
+    float m_run = -INFINITY, l_run = 0.f;
+    f32x4 acc[MY_TILES];
+#pragma unroll
+    for (int i = 0; i < MY_TILES; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    if (begin <= end) {                                      // the whole workgroup takes the same branch
+        const bf16* qrow = q + (int64_t)t * q_stride + (int64_t)head * D;
+        bf16x8 qf[QK_STEPS];
+#pragma unroll
+        for (int c = 0; c < DT / 2; ++c) qf[c] = ld8(qrow + c * 32 + g * 8);
+        if (DT & 1) qf[QK_STEPS - 1] = half_step(qrow + (DT - 1) * 16 + g * 4);
+
+        const int vlo = begin & ~3, vhi = end & ~3;
+        const int page_lo = begin / page_size, page_count = end / page_size - page_lo + 1;
+        const bool table_in_lds = page_count <= DECODE_LDS_PAGES;
+        if (table_in_lds)
+            for (int i = tid; i < page_count; i += 256) pages[i] = table[page_lo + i];
+        __syncthreads();
+        auto page_of = [&](int pos) -> int64_t {
+            return table_in_lds ? pages[pos / page_size - page_lo] : table[pos / page_size];
+        };
+        bf16x8 kreg[K_PER_THREAD];
+        short4_t vreg[V_PER_THREAD];
+        auto fetch = [&](int j0) {
+#pragma unroll
+            for (int i = 0; i < K_PER_THREAD; ++i) {
+                const int c = tid + i * 256;
+                if (K_CHUNKS % 256 == 0 || c < K_CHUNKS) {
+                    const int row = c / (D / 8), col = c % (D / 8);
+                    int pos = j0 + row;
+                    pos = pos < begin ? begin : (pos > end ? end : pos);
+                    kreg[i] = ld8(kc + ((page_of(pos) * nkv + kvh) * page_size + pos % page_size) * (int64_t)D + col * 8);
+                }
+            }
+            const int kg = tid & 7;
+            int vpos = j0 + kg * 4;
+            vpos = vpos < vlo ? vlo : (vpos > vhi ? vhi : vpos);
+            const bf16* vbase = vc + (page_of(vpos) * nkv + kvh) * (int64_t)D * page_size + vpos % page_size;
+#pragma unroll
+            for (int i = 0; i < V_PER_THREAD; ++i) {
+                const int d = (tid >> 3) + 32 * i;
+                if (D % 32 == 0 || d < D) vreg[i] = ld4(vbase + (int64_t)d * page_size);
+            }
+        };
+        auto stash = [&](int buf) {
+#pragma unroll
+            for (int i = 0; i < K_PER_THREAD; ++i) {
+                const int c = tid + i * 256;
+                if (K_CHUNKS % 256 == 0 || c < K_CHUNKS) {
+                    const int row = c / (D / 8), col = c % (D / 8);
+                    *reinterpret_cast<bf16x8*>(&ks[buf][row * KROW + col * 8]) = kreg[i];
+                }
+            }
+            const int kg = tid & 7;
+#pragma unroll
+            for (int i = 0; i < V_PER_THREAD; ++i) {
+                const int d = (tid >> 3) + 32 * i;
+                if (D % 32 == 0 || d < D) *reinterpret_cast<short4_t*>(&vs[buf][d * VROW + kg * 4]) = vreg[i];
+            }
+        };
+
+        const int j_begin = begin & ~31;
+        fetch(j_begin);
+        stash(0);
+        __syncthreads();
+        int buf = 0;
+        for (int j0 = j_begin; j0 <= end; j0 += 32, buf ^= 1) {
+            const bool more = j0 + 32 <= end;
+            if (more) fetch(j0 + 32);
+            f32x4 s[2];
+#pragma unroll
+            for (int half = 0; half < 2; ++half) {
+                const bf16* krow = &ks[buf][(half * 16 + r) * KROW];
+                s[half] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int c = 0; c < DT / 2; ++c)
+                    s[half] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<const bf16x8*>(krow + c * 32 + g * 8),
+                                                                      qf[c], s[half], 0, 0, 0);
+                if (DT & 1) {
+                    union { bf16x8 wide; short4_t half4[2]; } u;
+                    u.half4[0] = *reinterpret_cast<const short4_t*>(krow + (DT - 1) * 16 + g * 4);
+                    u.half4[1] = short4_t{0, 0, 0, 0};
+                    s[half] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(u.wide, qf[QK_STEPS - 1], s[half], 0, 0, 0);
+                }
+            }
+            // s[half][i] = S[key j0 + 16 half + 4 g + i][head r]
+            float mx = -INFINITY;
+#pragma unroll
+            for (int half = 0; half < 2; ++half)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int key = j0 + half * 16 + g * 4 + i;
+                    s[half][i] = (key >= begin && key <= end) ? s[half][i] * scale : -INFINITY;
+                    mx = fmaxf(mx, s[half][i]);
+                }
+            mx = lanes4_max(mx);
+            const float m_new = fmaxf(m_run, mx);            // finite: every 32-key step holds a visible key
+            const float corr = expf(m_run - m_new);
+            float pr[2][4], sum = 0.f;
+#pragma unroll
+            for (int half = 0; half < 2; ++half)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    pr[half][i] = expf(s[half][i] - m_new);
+                    sum += pr[half][i];
+                }
+            sum = lanes4_sum(sum);
+            l_run = l_run * corr + sum;
+            m_run = m_new;
+            const bf16x8 pf = {(bf16)pr[0][0], (bf16)pr[0][1], (bf16)pr[0][2], (bf16)pr[0][3],
+                               (bf16)pr[1][0], (bf16)pr[1][1], (bf16)pr[1][2], (bf16)pr[1][3]};
+#pragma unroll
+            for (int i = 0; i < MY_TILES; ++i) {
+                const int dt = wave + 4 * i;
+                if (DT % 4 == 0 || dt < DT) {
+                    const bf16* vrow = &vs[buf][(dt * 16 + r) * VROW];
+                    union { bf16x8 wide; short4_t half4[2]; } v;
+                    v.half4[0] = *reinterpret_cast<const short4_t*>(vrow + g * 4);
+                    v.half4[1] = *reinterpret_cast<const short4_t*>(vrow + 16 + g * 4);
+                    acc[i] *= corr;
+                    acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v.wide, pf, acc[i], 0, 0, 0);
+                }
+            }
+            if (more) stash(buf ^ 1);
+            __syncthreads();
+        }
+    }
+
+    // acc[i][j] = O^T[d = (wave + 4 i) * 16 + 4 g + j][head r]; every wavefront holds the same m_run, l_run
+    const int hq = kvh * G + hloc;
+    if (hloc < G) {
+#pragma unroll
+        for (int i = 0; i < MY_TILES; ++i) {
+            const int dt = wave + 4 * i;
+            if (DT % 4 == 0 || dt < DT) {
+                const int d = dt * 16 + g * 4;
+                if (num_splits == 1) {
+                    const float inv = 1.0f / l_run;
+                    bf16x4 o = {(bf16)(acc[i][0] * inv), (bf16)(acc[i][1] * inv), (bf16)(acc[i][2] * inv),
+                                (bf16)(acc[i][3] * inv)};
+                    *reinterpret_cast<bf16x4*>(out + ((int64_t)t * nq + hq) * D + d) = o;
+                } else {
+                    const int64_t slot = ((int64_t)ti * nq + hq) * num_splits + split;
+                    *reinterpret_cast<f32x4*>(part_acc + slot * D + d) = acc[i];
+                }
+            }
+        }
+        if (num_splits > 1 && wave == 0 && g == 0) {
+            const int64_t slot = ((int64_t)ti * nq + hq) * num_splits + split;
+            part_ml[slot * 2] = m_run;
+            part_ml[slot * 2 + 1] = l_run;
+        }
+    }
+}
+
 // Merge the splits of one (token, head) in split order.  The weights exp(m_s - m) of the splits are
 // computed once into LDS; then each thread sums one channel over the splits.
 #define COMBINE_MAX_SPLITS 1024
@@ -216,10 +425,17 @@ static int launch_decode(const void* q, int64_t q_stride, const void* kc, const 
     const int waves = DT <= 8 ? 4 : 2;
     const int G = nq / nkv, HB = (G + 15) / 16;
     const size_t smem = (size_t)(waves * DT * 256 + waves * 32) * sizeof(float);
-    hipLaunchKernelGGL((attention_decode_kernel<DT>), dim3(n_list, nkv * HB, num_splits), dim3(waves * 64), smem,
-                       stream, (const bf16*)q, q_stride, (const bf16*)kc, (const bf16*)vc, block_table, max_blocks,
-                       token_list, token_entry, positions, nq, nkv, page_size, window, scale, split_len, num_splits,
-                       (bf16*)out, part_acc, part_ml);
+    if (DT >= 2 && DT <= 8 && split_len % 32 == 0)
+        // head sizes 32..128: keys and values staged through LDS (two tiles fit)
+        hipLaunchKernelGGL((attention_decode_lds_kernel<(DT >= 2 && DT <= 8 ? DT : 2)>), dim3(n_list, nkv * HB, num_splits),
+                           dim3(256), 0, stream, (const bf16*)q, q_stride, (const bf16*)kc, (const bf16*)vc, block_table,
+                           max_blocks, token_list, token_entry, positions, nq, nkv, page_size, window, scale, split_len,
+                           num_splits, (bf16*)out, part_acc, part_ml);
+    else
+        hipLaunchKernelGGL((attention_decode_kernel<DT>), dim3(n_list, nkv * HB, num_splits), dim3(waves * 64), smem,
+                           stream, (const bf16*)q, q_stride, (const bf16*)kc, (const bf16*)vc, block_table, max_blocks,
+                           token_list, token_entry, positions, nq, nkv, page_size, window, scale, split_len, num_splits,
+                           (bf16*)out, part_acc, part_ml);
     SOMI_LAUNCH_CHECK("attention_decode");
     if (num_splits > 1) {
         hipLaunchKernelGGL(attention_combine_kernel, dim3(n_list, nq), dim3(128), 0, stream, part_acc, part_ml,

@@ -39,6 +39,23 @@ __device__ __forceinline__ bf16x8 pjoin(short4_t lo, short4_t hi) {
     return u.wide;
 }
 
+// Maximum / sum over the four lane groups (lanes l, l ^ 16, l ^ 32, l ^ 48) with the row-swap instructions
+// of gfx950: v_permlane16_swap exchanges odd 16-lane rows of one operand with even rows of the other,
+// v_permlane32_swap the upper and lower halves; no LDS round trip.
+typedef __attribute__((ext_vector_type(2))) unsigned u32x2;
+__device__ __forceinline__ float group_max(float v) {
+    u32x2 a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    v = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+    u32x2 b = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+__device__ __forceinline__ float group_sum(float v) {
+    u32x2 a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    v = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+    u32x2 b = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return __uint_as_float(b[0]) + __uint_as_float(b[1]);
+}
+
 template <int DT, int QB>
 __global__ void __launch_bounds__(256)
 attention_prefill_kernel(const bf16* __restrict__ q, int64_t q_stride, const bf16* __restrict__ kc,
@@ -180,6 +197,253 @@ attention_prefill_kernel(const bf16* __restrict__ q, int64_t q_stride, const bf1
     }
 }
 
+// The same computation with the key and value tiles staged through LDS: the four wavefronts of a
+// workgroup own 4 x 32 consecutive queries of one (portion, head) and walk the keys together, 32 at a time.
+// All 256 threads fetch the next tile from the pages into registers while the current one is being used
+// from LDS, then store it into the other LDS buffer; one barrier per step.  Every key and value is read
+// from L2/HBM once per 128 queries instead of once per wavefront.
+//   K tile in LDS: [32 keys][D + 8] (rows padded by 16 bytes: the 16 rows a 16-byte read touches fall into
+//   different banks); V tile: [D channels][32 + 4 keys].
+#define PREFILL_LDS_PAGES 2048     // block-table entries of the visible range kept in LDS (else read from memory)
+template <int DT>
+__global__ void __launch_bounds__(256, 2)
+attention_prefill_lds_kernel(const bf16* __restrict__ q, int64_t q_stride, const bf16* __restrict__ kc,
+                             const bf16* __restrict__ vc, const int* __restrict__ block_table, int max_blocks,
+                             const int* __restrict__ entry_start, const int* __restrict__ entry_first_pos, int nq,
+                             int nkv, int page_size, int window, float scale_log2, bf16* __restrict__ out) {
+    constexpr int D = DT * 16;
+    constexpr int QK_STEPS = (DT + 1) / 2;
+    constexpr int QB = 2, QW = QB * 16, WAVES = 4, QG = WAVES * QW;     // 128 queries per workgroup
+    constexpr int KROW = D + 8, VROW = 32 + 4;                          // padded LDS rows, in elements
+    constexpr int K_CHUNKS = 32 * D / 8;                                // 16-byte pieces of a key tile
+    constexpr int K_PER_THREAD = (K_CHUNKS + 255) / 256;
+    constexpr int V_PER_THREAD = (D + 31) / 32;                         // 8-byte pieces (4 keys of a channel): a
+                                                                        // thread takes key group tid % 8 of
+                                                                        // channels tid / 8 + 32 i
+    __shared__ __attribute__((aligned(16))) bf16 ks[2][32 * KROW];
+    __shared__ __attribute__((aligned(16))) bf16 vs[2][D * VROW];
+    __shared__ int pages[PREFILL_LDS_PAGES];
+
+    const int e = blockIdx.y, h = blockIdx.z;
+    const int kvh = h / (nq / nkv);
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, r = lane & 15, g = lane >> 4;
+    const int start = entry_start[e];
+    const int len = entry_start[e + 1] - start;
+    const int group = gridDim.x - 1 - blockIdx.x;           // the longest (latest) query groups start first
+    const int g0 = group * QG;
+    if (g0 >= len) return;                                  // the whole workgroup leaves together
+    const int pos0 = entry_first_pos[e];
+    const int* table = block_table + (int64_t)e * max_blocks;
+    const int wg_valid = len - g0 < QG ? len - g0 : QG;
+    const int wg_first = pos0 + g0, wg_last = pos0 + g0 + wg_valid - 1;
+    const int lo = (window > 0 && wg_first - window + 1 > 0) ? wg_first - window + 1 : 0;
+    const int vlo = lo & ~3, vhi = wg_last & ~3;
+
+    // The pages of the visible range go to LDS once, so that a tile's addresses do not wait for a
+    // table read from memory before its own loads can start.
+    const int page_lo = lo / page_size, page_count = wg_last / page_size - page_lo + 1;
+    const bool table_in_lds = page_count <= PREFILL_LDS_PAGES;
+    if (table_in_lds)
+        for (int i = tid; i < page_count; i += 256) pages[i] = table[page_lo + i];
+    __syncthreads();
+    auto page_of = [&](int pos) -> int64_t {
+        return table_in_lds ? pages[pos / page_size - page_lo] : table[pos / page_size];
+    };
+
+    // this wavefront's queries
+    const int q0 = g0 + wave * QW;
+    const bool active = q0 < len;
+    const int nvalid = active ? (len - q0 < QW ? len - q0 : QW) : 0;
+    const int w_last = pos0 + q0 + nvalid - 1;
+    bf16x8 qf[QB][QK_STEPS];
+    int pcol[QB];
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb) {
+        int qi = q0 + qb * 16 + r;
+        qi = qi < len ? qi : len - 1;
+        pcol[qb] = pos0 + qi;
+        const bf16* qrow = q + (int64_t)(start + qi) * q_stride + (int64_t)h * D;
+#pragma unroll
+        for (int c = 0; c < DT / 2; ++c) qf[qb][c] = pld8(qrow + c * 32 + g * 8);
+        if (DT & 1) qf[qb][QK_STEPS - 1] = phalf(qrow + (DT - 1) * 16 + g * 4);
+    }
+    float m_run[QB], l_run[QB];
+    f32x4 acc[QB][DT];
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb) {
+        m_run[qb] = -INFINITY;
+        l_run[qb] = 0.f;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) acc[qb][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+
+    // staging registers of the next tile
+    bf16x8 kreg[K_PER_THREAD];
+    short4_t vreg[V_PER_THREAD];
+    auto fetch = [&](int j0) {
+#pragma unroll
+        for (int i = 0; i < K_PER_THREAD; ++i) {
+            const int c = tid + i * 256;
+            if (K_CHUNKS % 256 == 0 || c < K_CHUNKS) {
+                const int row = c / (D / 8), col = c % (D / 8);
+                int pos = j0 + row;
+                pos = pos < lo ? lo : (pos > wg_last ? wg_last : pos);
+                const int64_t page = page_of(pos);
+                kreg[i] = pld8(kc + ((page * nkv + kvh) * page_size + pos % page_size) * (int64_t)D + col * 8);
+            }
+        }
+        {
+            const int kg = tid & 7;
+            int vpos = j0 + kg * 4;
+            vpos = vpos < vlo ? vlo : (vpos > vhi ? vhi : vpos);
+            const int64_t page = page_of(vpos);
+            const bf16* vbase = vc + (page * nkv + kvh) * (int64_t)D * page_size + vpos % page_size;
+#pragma unroll
+            for (int i = 0; i < V_PER_THREAD; ++i) {
+                const int d = (tid >> 3) + 32 * i;
+                if (D % 32 == 0 || d < D) vreg[i] = pld4(vbase + (int64_t)d * page_size);
+            }
+        }
+    };
+    auto stash = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < K_PER_THREAD; ++i) {
+            const int c = tid + i * 256;
+            if (K_CHUNKS % 256 == 0 || c < K_CHUNKS) {
+                const int row = c / (D / 8), col = c % (D / 8);
+                *reinterpret_cast<bf16x8*>(&ks[buf][row * KROW + col * 8]) = kreg[i];
+            }
+        }
+        {
+            const int kg = tid & 7;
+#pragma unroll
+            for (int i = 0; i < V_PER_THREAD; ++i) {
+                const int d = (tid >> 3) + 32 * i;
+                if (D % 32 == 0 || d < D) *reinterpret_cast<short4_t*>(&vs[buf][d * VROW + kg * 4]) = vreg[i];
+            }
+        }
+    };
+
+    const int j_begin = lo & ~31;
+    fetch(j_begin);
+    stash(0);
+    __syncthreads();
+    int buf = 0;
+    for (int j0 = j_begin; j0 <= wg_last; j0 += 32, buf ^= 1) {
+        const bool more = j0 + 32 <= wg_last;
+        if (more) fetch(j0 + 32);
+        if (active && j0 <= w_last) {
+            bf16x8 kf[2][QK_STEPS];
+#pragma unroll
+            for (int half = 0; half < 2; ++half) {
+                const bf16* krow = &ks[buf][(half * 16 + r) * KROW];
+#pragma unroll
+                for (int c = 0; c < DT / 2; ++c) kf[half][c] = *reinterpret_cast<const bf16x8*>(krow + c * 32 + g * 8);
+                if (DT & 1) {
+                    union { bf16x8 wide; short4_t half4[2]; } u;
+                    u.half4[0] = *reinterpret_cast<const short4_t*>(krow + (DT - 1) * 16 + g * 4);
+                    u.half4[1] = short4_t{0, 0, 0, 0};
+                    kf[half][QK_STEPS - 1] = u.wide;
+                }
+            }
+            // all query blocks stage by stage, so that their dependent chains overlap
+            f32x4 s[QB][2];
+#pragma unroll
+            for (int qb = 0; qb < QB; ++qb)
+#pragma unroll
+                for (int half = 0; half < 2; ++half) {
+                    s[qb][half] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int c = 0; c < QK_STEPS; ++c)
+                        s[qb][half] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[half][c], qf[qb][c], s[qb][half], 0, 0, 0);
+                }
+            float mx[QB];
+#pragma unroll
+            for (int qb = 0; qb < QB; ++qb) {
+                const int p = pcol[qb];
+                const int first = window > 0 ? p - window + 1 : 0;
+                mx[qb] = -INFINITY;
+#pragma unroll
+                for (int half = 0; half < 2; ++half)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const int key = j0 + half * 16 + g * 4 + i;
+                        s[qb][half][i] = (key <= p && key >= first) ? s[qb][half][i] * scale_log2 : -INFINITY;
+                        mx[qb] = fmaxf(mx[qb], s[qb][half][i]);
+                    }
+            }
+#pragma unroll
+            for (int qb = 0; qb < QB; ++qb) mx[qb] = group_max(mx[qb]);
+            float corr[QB], sum[QB];
+            bf16x8 pf[QB];
+#pragma unroll
+            for (int qb = 0; qb < QB; ++qb) {
+                const float m_new = fmaxf(m_run[qb], mx[qb]);
+                const float m_use = m_new == -INFINITY ? 0.f : m_new;     // nothing visible yet: weights stay 0
+                corr[qb] = exp2f(m_run[qb] - m_use);
+                m_run[qb] = m_new;
+                float pr[2][4];
+                sum[qb] = 0.f;
+#pragma unroll
+                for (int half = 0; half < 2; ++half)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        pr[half][i] = exp2f(s[qb][half][i] - m_use);
+                        sum[qb] += pr[half][i];
+                    }
+                pf[qb] = bf16x8{(bf16)pr[0][0], (bf16)pr[0][1], (bf16)pr[0][2], (bf16)pr[0][3],
+                                (bf16)pr[1][0], (bf16)pr[1][1], (bf16)pr[1][2], (bf16)pr[1][3]};
+            }
+#pragma unroll
+            for (int qb = 0; qb < QB; ++qb) {
+                sum[qb] = group_sum(sum[qb]);
+                l_run[qb] = l_run[qb] * corr[qb] + sum[qb];
+            }
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                const bf16* vrow = &vs[buf][(dt * 16 + r) * VROW];
+                const bf16x8 vf = pjoin(*reinterpret_cast<const short4_t*>(vrow + g * 4),
+                                        *reinterpret_cast<const short4_t*>(vrow + 16 + g * 4));
+#pragma unroll
+                for (int qb = 0; qb < QB; ++qb) {
+                    acc[qb][dt] *= corr[qb];
+                    acc[qb][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[qb], acc[qb][dt], 0, 0, 0);
+                }
+            }
+        }
+        if (more) stash(buf ^ 1);
+        __syncthreads();
+    }
+
+    if (!active) return;
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb) {
+        const int qi = q0 + qb * 16 + r;
+        if (qi >= len) continue;
+        const float inv = 1.0f / l_run[qb];
+        bf16* orow = out + ((int64_t)(start + qi) * nq + h) * D + g * 4;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+            const bf16x4 o = {(bf16)(acc[qb][dt][0] * inv), (bf16)(acc[qb][dt][1] * inv),
+                              (bf16)(acc[qb][dt][2] * inv), (bf16)(acc[qb][dt][3] * inv)};
+            *reinterpret_cast<bf16x4*>(orow + dt * 16) = o;
+        }
+    }
+}
+
+template <int DT>
+static int launch_prefill_lds(const void* q, int64_t q_stride, const void* kc, const void* vc, const int* block_table,
+                              int max_blocks, const int* entry_start, const int* entry_first_pos, int n_entries,
+                              int max_entry_len, int nq, int nkv, int page_size, int window, float scale, void* out,
+                              hipStream_t stream) {
+    const dim3 grid(ceil_div(max_entry_len, 128), n_entries, nq);
+    hipLaunchKernelGGL((attention_prefill_lds_kernel<DT>), grid, dim3(256), 0, stream, (const bf16*)q, q_stride,
+                       (const bf16*)kc, (const bf16*)vc, block_table, max_blocks, entry_start, entry_first_pos, nq, nkv,
+                       page_size, window, scale * 1.44269504088896341f, (bf16*)out);
+    SOMI_LAUNCH_CHECK("attention_prefill_lds");
+    return 0;
+}
+
 template <int DT, int QB>
 static int launch_prefill(const void* q, int64_t q_stride, const void* kc, const void* vc, const int* block_table,
                           int max_blocks, const int* entry_start, const int* entry_first_pos, int n_entries,
@@ -220,12 +484,20 @@ extern "C" int somi_attention_prefill(const void* q, int64_t q_stride, const voi
         return launch_prefill<DT, QB>(q, q_stride, k_cache, v_cache, block_table, max_blocks, entry_start,         \
                                       entry_first_pos, n_entries, max_entry_len, nq, nkv, page_size, window, scale, \
                                       out, stream)
+#define SOMI_PREFILL_LDS(DT)                                                                                       \
+    case DT:                                                                                                       \
+        return launch_prefill_lds<DT>(q, q_stride, k_cache, v_cache, block_table, max_blocks, entry_start,         \
+                                      entry_first_pos, n_entries, max_entry_len, nq, nkv, page_size, window, scale, \
+                                      out, stream)
+    // head sizes 32..128 stage keys and values through LDS; the others (LDS would not hold two tiles, or a
+    // tile is smaller than the workgroup's loads) keep them in registers per wavefront
     switch (D / 16) {
-        SOMI_PREFILL(1, 4); SOMI_PREFILL(2, 4); SOMI_PREFILL(3, 4); SOMI_PREFILL(4, 4); SOMI_PREFILL(5, 4);
-        SOMI_PREFILL(6, 4); SOMI_PREFILL(7, 4); SOMI_PREFILL(8, 4); SOMI_PREFILL(9, 2); SOMI_PREFILL(10, 2);
+        SOMI_PREFILL(1, 4); SOMI_PREFILL_LDS(2); SOMI_PREFILL_LDS(3); SOMI_PREFILL_LDS(4); SOMI_PREFILL_LDS(5);
+        SOMI_PREFILL_LDS(6); SOMI_PREFILL_LDS(7); SOMI_PREFILL_LDS(8); SOMI_PREFILL(9, 2); SOMI_PREFILL(10, 2);
         SOMI_PREFILL(11, 2); SOMI_PREFILL(12, 2); SOMI_PREFILL(13, 2); SOMI_PREFILL(14, 2); SOMI_PREFILL(15, 2);
         SOMI_PREFILL(16, 2);
     }
 #undef SOMI_PREFILL
+#undef SOMI_PREFILL_LDS
     return somi_fail("attention_prefill: unsupported head_dim %d", D);
 }
