@@ -171,3 +171,45 @@ def test_step_contract_errors(model_folders):
         runner.step([StepEntry("q", [1] * 33, [0])])       # 3 pages, the pool has 2
     assert runner.cache.free_pages() == before and runner.cache.num_tokens("q") == 0
     assert runner.step([StepEntry("q", [1] * 32, [31])]).shape == (1, config.vocab_size)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_captured_decode_steps_replay_like_eager_steps(dtype, model_folders):
+    """Decode steps are captured as HIP graphs per batch size.  Batches of 3 and of 40 requests (the larger
+    one takes the library matrix product inside the graph) are replayed several times, with eager work and
+    synchronisations in between, and every replay is compared with the same step run without graphs."""
+    from somi_inference_amd.models import load_model, make_runner
+    from somi_inference_amd.engine import ModelRunner
+    from somi_inference_amd.cache import CacheManager
+    vocab, bs = TINY["B"]["config"].vocab_size, TINY["B"]["block_size"]
+    model, _ = load_model(model_folders["B"], dtype=dtype)
+    graphed = make_runner(model, block_size=bs, num_blocks=256, max_requests=48)
+    eager_cache = CacheManager(model.cache_needs(), block_size=bs, num_blocks=256, max_requests=48,
+                               dtype=model.runtime.dtype, device=model.runtime.device)
+    eager = ModelRunner(model, eager_cache, decode_graphs=False)
+    assert graphed.decode_graphs and not eager.decode_graphs
+    for batch in (3, 40):
+        ids = [f"g{batch}_{i}" for i in range(batch)]
+        prompts = [token_ids(vocab, 5 + (i * 7) % 23, 300 + i) for i in range(batch)]
+        for runner in (graphed, eager):
+            for rid, prompt in zip(ids, prompts):
+                runner.begin(rid)
+                runner.step([StepEntry(rid, prompt, [])])
+        last = [p[-1] for p in prompts]
+        for step in range(12):
+            entries = [StepEntry(rid, [tok], [0]) for rid, tok in zip(ids, last)]
+            want = eager.step(entries).clone()
+            got = graphed.step(entries).clone()
+            torch.cuda.synchronize()
+            if dtype == "float32":
+                assert torch.equal(got, want), f"batch {batch}, replay {step}: graph and eager logits differ"
+            else:
+                # a captured step sizes its key splits for the widest context its block tables allow, an eager
+                # step for the actual one: the bfloat16 weights of P.V are rounded relative to another maximum
+                assert (got - want).abs().max() < 2e-2, f"batch {batch}, replay {step}"
+            last = want.argmax(dim=-1).tolist()
+            _ = torch.randn(64, 64, device="cuda:0") @ torch.randn(64, 64, device="cuda:0")   # eager work in between
+        for runner in (graphed, eager):
+            for rid in ids:
+                runner.end(rid)
+    assert graphed.graph_replays >= 24
