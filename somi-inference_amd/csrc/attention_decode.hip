@@ -228,7 +228,8 @@ attention_decode_lds_kernel(const bf16* __restrict__ q, int64_t q_stride, const 
     const int hloc = hb * 16 + r;
     const int head = kvh * G + (hloc < G ? hloc : G - 1);
 
-    float m_run = -INFINITY, l_run = 0.f;
+    const float scale_log2 = scale * 1.44269504088896341f;
+    float m_run = -INFINITY, l_run = 0.f;            // running maximum (in base-2 units) and sum
     f32x4 acc[MY_TILES];
 #pragma unroll
     for (int i = 0; i < MY_TILES; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -241,17 +242,20 @@ attention_decode_lds_kernel(const bf16* __restrict__ q, int64_t q_stride, const 
         if (DT & 1) qf[QK_STEPS - 1] = half_step(qrow + (DT - 1) * 16 + g * 4);
 
         const int vlo = begin & ~3, vhi = end & ~3;
-        const int page_lo = begin / page_size, page_count = end / page_size - page_lo + 1;
-        const bool table_in_lds = page_count <= DECODE_LDS_PAGES;
-        if (table_in_lds)
-            for (int i = tid; i < page_count; i += 256) pages[i] = table[page_lo + i];
+        // The page size is a power of two here (the launcher sees to it): page arithmetic is shift and mask.
+        // The split's pages (at most DECODE_LDS_PAGES, also the launcher's duty) are copied to LDS once, so
+        // that a tile's addresses never wait for a read of the table from memory: such a wait would also wait
+        // for every tile load issued before it.
+        const int shift = __builtin_ctz(page_size);
+        auto page_offset = [&](int pos) { return pos & (page_size - 1); };
+        const int page_lo = begin >> shift, page_count = (end >> shift) - page_lo + 1;
+        for (int i = tid; i < page_count; i += 256) pages[i] = table[page_lo + i];
         __syncthreads();
-        auto page_of = [&](int pos) -> int64_t {
-            return table_in_lds ? pages[pos / page_size - page_lo] : table[pos / page_size];
-        };
-        bf16x8 kreg[K_PER_THREAD];
-        short4_t vreg[V_PER_THREAD];
-        auto fetch = [&](int j0) {
+        auto page_of = [&](int pos) -> int64_t { return pages[(pos >> shift) - page_lo]; };
+        // two register sets: the tiles two and three steps ahead are in flight while one is computed
+        bf16x8 kreg_a[K_PER_THREAD], kreg_b[K_PER_THREAD];
+        short4_t vreg_a[V_PER_THREAD], vreg_b[V_PER_THREAD];
+        auto fetch = [&](bf16x8 (&kreg)[K_PER_THREAD], short4_t (&vreg)[V_PER_THREAD], int j0) {
 #pragma unroll
             for (int i = 0; i < K_PER_THREAD; ++i) {
                 const int c = tid + i * 256;
@@ -259,20 +263,20 @@ attention_decode_lds_kernel(const bf16* __restrict__ q, int64_t q_stride, const 
                     const int row = c / (D / 8), col = c % (D / 8);
                     int pos = j0 + row;
                     pos = pos < begin ? begin : (pos > end ? end : pos);
-                    kreg[i] = ld8(kc + ((page_of(pos) * nkv + kvh) * page_size + pos % page_size) * (int64_t)D + col * 8);
+                    kreg[i] = ld8(kc + ((page_of(pos) * nkv + kvh) * page_size + page_offset(pos)) * (int64_t)D + col * 8);
                 }
             }
             const int kg = tid & 7;
             int vpos = j0 + kg * 4;
             vpos = vpos < vlo ? vlo : (vpos > vhi ? vhi : vpos);
-            const bf16* vbase = vc + (page_of(vpos) * nkv + kvh) * (int64_t)D * page_size + vpos % page_size;
+            const bf16* vbase = vc + (page_of(vpos) * nkv + kvh) * (int64_t)D * page_size + page_offset(vpos);
 #pragma unroll
             for (int i = 0; i < V_PER_THREAD; ++i) {
                 const int d = (tid >> 3) + 32 * i;
                 if (D % 32 == 0 || d < D) vreg[i] = ld4(vbase + (int64_t)d * page_size);
             }
         };
-        auto stash = [&](int buf) {
+        auto stash = [&](const bf16x8 (&kreg)[K_PER_THREAD], const short4_t (&vreg)[V_PER_THREAD], int buf) {
 #pragma unroll
             for (int i = 0; i < K_PER_THREAD; ++i) {
                 const int c = tid + i * 256;
@@ -288,15 +292,7 @@ attention_decode_lds_kernel(const bf16* __restrict__ q, int64_t q_stride, const 
                 if (D % 32 == 0 || d < D) *reinterpret_cast<short4_t*>(&vs[buf][d * VROW + kg * 4]) = vreg[i];
             }
         };
-
-        const int j_begin = begin & ~31;
-        fetch(j_begin);
-        stash(0);
-        __syncthreads();
-        int buf = 0;
-        for (int j0 = j_begin; j0 <= end; j0 += 32, buf ^= 1) {
-            const bool more = j0 + 32 <= end;
-            if (more) fetch(j0 + 32);
+        auto compute = [&](int buf, int j0) {
             f32x4 s[2];
 #pragma unroll
             for (int half = 0; half < 2; ++half) {
@@ -313,25 +309,29 @@ attention_decode_lds_kernel(const bf16* __restrict__ q, int64_t q_stride, const 
                     s[half] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(u.wide, qf[QK_STEPS - 1], s[half], 0, 0, 0);
                 }
             }
-            // s[half][i] = S[key j0 + 16 half + 4 g + i][head r]
-            float mx = -INFINITY;
+            // s[half][i] = S[key j0 + 16 half + 4 g + i][head r], still unscaled; keys outside the split are
+            // masked (only the first and last step of a split can hold any)
+            if (j0 < begin || j0 + 31 > end) {
 #pragma unroll
-            for (int half = 0; half < 2; ++half)
+                for (int half = 0; half < 2; ++half)
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const int key = j0 + half * 16 + g * 4 + i;
-                    s[half][i] = (key >= begin && key <= end) ? s[half][i] * scale : -INFINITY;
-                    mx = fmaxf(mx, s[half][i]);
-                }
-            mx = lanes4_max(mx);
+                    for (int i = 0; i < 4; ++i) {
+                        const int key = j0 + half * 16 + g * 4 + i;
+                        if (key < begin || key > end) s[half][i] = -INFINITY;
+                    }
+            }
+            float mx = fmaxf(fmaxf(fmaxf(s[0][0], s[0][1]), fmaxf(s[0][2], s[0][3])),
+                             fmaxf(fmaxf(s[1][0], s[1][1]), fmaxf(s[1][2], s[1][3])));
+            mx = lanes4_max(mx) * scale_log2;                // scale > 0: the maximum commutes with it
+            // running maximum and weights in base 2: weight = 2^(s * scale * log2(e) - m)
             const float m_new = fmaxf(m_run, mx);            // finite: every 32-key step holds a visible key
-            const float corr = expf(m_run - m_new);
+            const float corr = __builtin_amdgcn_exp2f(m_run - m_new);
             float pr[2][4], sum = 0.f;
 #pragma unroll
             for (int half = 0; half < 2; ++half)
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    pr[half][i] = expf(s[half][i] - m_new);
+                    pr[half][i] = __builtin_amdgcn_exp2f(fmaf(s[half][i], scale_log2, -m_new));
                     sum += pr[half][i];
                 }
             sum = lanes4_sum(sum);
@@ -351,7 +351,28 @@ attention_decode_lds_kernel(const bf16* __restrict__ q, int64_t q_stride, const 
                     acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v.wide, pf, acc[i], 0, 0, 0);
                 }
             }
-            if (more) stash(buf ^ 1);
+        };
+
+        const int j_begin = begin & ~31;
+        const int n = (end - j_begin) / 32 + 1;              // 32-key steps of this split
+        // Every step stashes and fetches unconditionally (past the end: the last step once more, into a buffer
+        // nobody reads), so the number of loads in flight at each wait is known when the kernel is compiled
+        // and a wait for one register set does not also wait for the other.
+        auto step_at = [&](int c) { return j_begin + 32 * (c < n ? c : n - 1); };
+        fetch(kreg_a, vreg_a, j_begin);
+        stash(kreg_a, vreg_a, 0);
+        fetch(kreg_a, vreg_a, step_at(1));                   // odd steps travel in set a, even ones in set b
+        fetch(kreg_b, vreg_b, step_at(2));
+        __syncthreads();
+        for (int c = 0; c < n; c += 2) {
+            compute(0, j_begin + 32 * c);
+            stash(kreg_a, vreg_a, 1);
+            fetch(kreg_a, vreg_a, step_at(c + 3));
+            __syncthreads();
+            if (c + 1 >= n) break;
+            compute(1, j_begin + 32 * (c + 1));
+            stash(kreg_b, vreg_b, 0);
+            fetch(kreg_b, vreg_b, step_at(c + 4));
             __syncthreads();
         }
     }
@@ -377,7 +398,7 @@ attention_decode_lds_kernel(const bf16* __restrict__ q, int64_t q_stride, const 
         }
         if (num_splits > 1 && wave == 0 && g == 0) {
             const int64_t slot = ((int64_t)ti * nq + hq) * num_splits + split;
-            part_ml[slot * 2] = m_run;
+            part_ml[slot * 2] = m_run * 0.693147180559945309f;      // the merge works in natural units
             part_ml[slot * 2 + 1] = l_run;
         }
     }
@@ -407,12 +428,20 @@ attention_combine_kernel(const float* __restrict__ part_acc, const float* __rest
         lsum += l * f;
     }
     const float l_all = block_sum<128>(lsum, red);      // also makes factor[] visible
+    // every split wrote its partial output (zeros where it saw no key), so the loads need no condition and
+    // are issued eight at a time
     for (int d = tid; d < D; d += 128) {
+        const float* src = part_acc + base * D + d;
         float total = 0.f;
-        for (int s = 0; s < num_splits; ++s) {
-            const float f = factor[s];
-            if (f > 0.f) total += part_acc[(base + s) * D + d] * f;
+        int s = 0;
+        for (; s + 8 <= num_splits; s += 8) {
+            float v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = src[(int64_t)(s + u) * D];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) total += v[u] * factor[s + u];
         }
+        for (; s < num_splits; ++s) total += src[(int64_t)s * D] * factor[s];
         out[((int64_t)t * nq + h) * D + d] = (bf16)(total / l_all);
     }
 }
@@ -425,7 +454,8 @@ static int launch_decode(const void* q, int64_t q_stride, const void* kc, const 
     const int waves = DT <= 8 ? 4 : 2;
     const int G = nq / nkv, HB = (G + 15) / 16;
     const size_t smem = (size_t)(waves * DT * 256 + waves * 32) * sizeof(float);
-    if (DT >= 2 && DT <= 8 && split_len % 32 == 0)
+    const bool pow2_pages = (page_size & (page_size - 1)) == 0;
+    if (DT >= 2 && DT <= 8 && pow2_pages && split_len / page_size + 2 <= DECODE_LDS_PAGES)
         // head sizes 32..128: keys and values staged through LDS (two tiles fit)
         hipLaunchKernelGGL((attention_decode_lds_kernel<(DT >= 2 && DT <= 8 ? DT : 2)>), dim3(n_list, nkv * HB, num_splits),
                            dim3(256), 0, stream, (const bf16*)q, q_stride, (const bf16*)kc, (const bf16*)vc, block_table,

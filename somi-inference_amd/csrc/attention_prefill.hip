@@ -241,14 +241,14 @@ attention_prefill_lds_kernel(const bf16* __restrict__ q, int64_t q_stride, const
 
     // The pages of the visible range go to LDS once, so that a tile's addresses do not wait for a
     // table read from memory before its own loads can start.
-    const int page_lo = lo / page_size, page_count = wg_last / page_size - page_lo + 1;
-    const bool table_in_lds = page_count <= PREFILL_LDS_PAGES;
-    if (table_in_lds)
-        for (int i = tid; i < page_count; i += 256) pages[i] = table[page_lo + i];
+    // (power-of-two page size and at most PREFILL_LDS_PAGES pages in reach: the launcher's duty.  A read of
+    // the table from memory inside the loop would make every tile wait for all loads issued before it.)
+    const int shift = __builtin_ctz(page_size);
+    const int page_lo = lo >> shift, page_count = (wg_last >> shift) - page_lo + 1;
+    for (int i = tid; i < page_count; i += 256) pages[i] = table[page_lo + i];
     __syncthreads();
-    auto page_of = [&](int pos) -> int64_t {
-        return table_in_lds ? pages[pos / page_size - page_lo] : table[pos / page_size];
-    };
+    auto page_of = [&](int pos) -> int64_t { return pages[(pos >> shift) - page_lo]; };
+    auto page_offset = [&](int pos) { return pos & (page_size - 1); };
 
     // this wavefront's queries
     const int q0 = g0 + wave * QW;
@@ -289,7 +289,7 @@ attention_prefill_lds_kernel(const bf16* __restrict__ q, int64_t q_stride, const
                 int pos = j0 + row;
                 pos = pos < lo ? lo : (pos > wg_last ? wg_last : pos);
                 const int64_t page = page_of(pos);
-                kreg[i] = pld8(kc + ((page * nkv + kvh) * page_size + pos % page_size) * (int64_t)D + col * 8);
+                kreg[i] = pld8(kc + ((page * nkv + kvh) * page_size + page_offset(pos)) * (int64_t)D + col * 8);
             }
         }
         {
@@ -297,7 +297,7 @@ attention_prefill_lds_kernel(const bf16* __restrict__ q, int64_t q_stride, const
             int vpos = j0 + kg * 4;
             vpos = vpos < vlo ? vlo : (vpos > vhi ? vhi : vpos);
             const int64_t page = page_of(vpos);
-            const bf16* vbase = vc + (page * nkv + kvh) * (int64_t)D * page_size + vpos % page_size;
+            const bf16* vbase = vc + (page * nkv + kvh) * (int64_t)D * page_size + page_offset(vpos);
 #pragma unroll
             for (int i = 0; i < V_PER_THREAD; ++i) {
                 const int d = (tid >> 3) + 32 * i;
@@ -357,30 +357,38 @@ attention_prefill_lds_kernel(const bf16* __restrict__ q, int64_t q_stride, const
                     for (int c = 0; c < QK_STEPS; ++c)
                         s[qb][half] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[half][c], qf[qb][c], s[qb][half], 0, 0, 0);
                 }
+            // scores stay unscaled; keys a query must not see are masked, which only steps that reach past the
+            // wavefront's first query (or a window's lower edge) can hold
+            if (window > 0 || j0 + 31 > pos0 + q0) {
+#pragma unroll
+                for (int qb = 0; qb < QB; ++qb) {
+                    const int p = pcol[qb];
+                    const int first = window > 0 ? p - window + 1 : 0;
+#pragma unroll
+                    for (int half = 0; half < 2; ++half)
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            const int key = j0 + half * 16 + g * 4 + i;
+                            if (key > p || key < first) s[qb][half][i] = -INFINITY;
+                        }
+                }
+            }
             float mx[QB];
 #pragma unroll
-            for (int qb = 0; qb < QB; ++qb) {
-                const int p = pcol[qb];
-                const int first = window > 0 ? p - window + 1 : 0;
-                mx[qb] = -INFINITY;
+            for (int qb = 0; qb < QB; ++qb)
+                mx[qb] = fmaxf(fmaxf(fmaxf(s[qb][0][0], s[qb][0][1]), fmaxf(s[qb][0][2], s[qb][0][3])),
+                               fmaxf(fmaxf(s[qb][1][0], s[qb][1][1]), fmaxf(s[qb][1][2], s[qb][1][3])));
 #pragma unroll
-                for (int half = 0; half < 2; ++half)
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        const int key = j0 + half * 16 + g * 4 + i;
-                        s[qb][half][i] = (key <= p && key >= first) ? s[qb][half][i] * scale_log2 : -INFINITY;
-                        mx[qb] = fmaxf(mx[qb], s[qb][half][i]);
-                    }
-            }
-#pragma unroll
-            for (int qb = 0; qb < QB; ++qb) mx[qb] = group_max(mx[qb]);
+            for (int qb = 0; qb < QB; ++qb) mx[qb] = group_max(mx[qb]) * scale_log2;   // scale > 0 commutes with max
             float corr[QB], sum[QB];
             bf16x8 pf[QB];
+            bool rescale = false;
 #pragma unroll
             for (int qb = 0; qb < QB; ++qb) {
                 const float m_new = fmaxf(m_run[qb], mx[qb]);
                 const float m_use = m_new == -INFINITY ? 0.f : m_new;     // nothing visible yet: weights stay 0
-                corr[qb] = exp2f(m_run[qb] - m_use);
+                corr[qb] = __builtin_amdgcn_exp2f(m_run[qb] - m_use);
+                rescale = rescale || m_new != m_run[qb];
                 m_run[qb] = m_new;
                 float pr[2][4];
                 sum[qb] = 0.f;
@@ -388,7 +396,7 @@ attention_prefill_lds_kernel(const bf16* __restrict__ q, int64_t q_stride, const
                 for (int half = 0; half < 2; ++half)
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
-                        pr[half][i] = exp2f(s[qb][half][i] - m_use);
+                        pr[half][i] = __builtin_amdgcn_exp2f(fmaf(s[qb][half][i], scale_log2, -m_use));
                         sum[qb] += pr[half][i];
                     }
                 pf[qb] = bf16x8{(bf16)pr[0][0], (bf16)pr[0][1], (bf16)pr[0][2], (bf16)pr[0][3],
@@ -399,16 +407,21 @@ attention_prefill_lds_kernel(const bf16* __restrict__ q, int64_t q_stride, const
                 sum[qb] = group_sum(sum[qb]);
                 l_run[qb] = l_run[qb] * corr[qb] + sum[qb];
             }
+            // the outputs are rescaled only when some query's maximum moved (rare after the first steps)
+            if (__builtin_amdgcn_ballot_w64(rescale) != 0) {
+#pragma unroll
+                for (int qb = 0; qb < QB; ++qb)
+#pragma unroll
+                    for (int dt = 0; dt < DT; ++dt) acc[qb][dt] *= corr[qb];
+            }
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) {
                 const bf16* vrow = &vs[buf][(dt * 16 + r) * VROW];
                 const bf16x8 vf = pjoin(*reinterpret_cast<const short4_t*>(vrow + g * 4),
                                         *reinterpret_cast<const short4_t*>(vrow + 16 + g * 4));
 #pragma unroll
-                for (int qb = 0; qb < QB; ++qb) {
-                    acc[qb][dt] *= corr[qb];
+                for (int qb = 0; qb < QB; ++qb)
                     acc[qb][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[qb], acc[qb][dt], 0, 0, 0);
-                }
             }
         }
         if (more) stash(buf ^ 1);
@@ -486,11 +499,17 @@ extern "C" int somi_attention_prefill(const void* q, int64_t q_stride, const voi
                                       out, stream)
 #define SOMI_PREFILL_LDS(DT)                                                                                       \
     case DT:                                                                                                       \
+        if (!lds_ok)                                                                                               \
+            return launch_prefill<DT, 4>(q, q_stride, k_cache, v_cache, block_table, max_blocks, entry_start,      \
+                                         entry_first_pos, n_entries, max_entry_len, nq, nkv, page_size, window,    \
+                                         scale, out, stream);                                                      \
         return launch_prefill_lds<DT>(q, q_stride, k_cache, v_cache, block_table, max_blocks, entry_start,         \
                                       entry_first_pos, n_entries, max_entry_len, nq, nkv, page_size, window, scale, \
                                       out, stream)
     // head sizes 32..128 stage keys and values through LDS; the others (LDS would not hold two tiles, or a
-    // tile is smaller than the workgroup's loads) keep them in registers per wavefront
+    // tile is smaller than the workgroup's loads) keep them in registers per wavefront, and so do page sizes
+    // that are no power of two and block tables too wide for the LDS copy of a request's pages
+    const bool lds_ok = (page_size & (page_size - 1)) == 0 && max_blocks <= PREFILL_LDS_PAGES;
     switch (D / 16) {
         SOMI_PREFILL(1, 4); SOMI_PREFILL_LDS(2); SOMI_PREFILL_LDS(3); SOMI_PREFILL_LDS(4); SOMI_PREFILL_LDS(5);
         SOMI_PREFILL_LDS(6); SOMI_PREFILL_LDS(7); SOMI_PREFILL_LDS(8); SOMI_PREFILL(9, 2); SOMI_PREFILL(10, 2);

@@ -6,7 +6,7 @@ import torch
 
 from . import ops
 
-TARGET_WORKGROUPS = 1024        # about four per compute unit
+TARGET_WORKGROUPS = 512         # about two per compute unit (measured best at 8 requests x 4,096 keys)
 MIN_SPLIT = 64                  # keys per split at least (a multiple of the 16-key tile)
 MAX_SPLITS = 1024               # what the merge kernel holds
 DECODE_PORTION = 8              # batches whose longest portion is at most this take the decode kernel
