@@ -213,3 +213,67 @@ def test_captured_decode_steps_replay_like_eager_steps(dtype, model_folders):
             for rid in ids:
                 runner.end(rid)
     assert graphed.graph_replays >= 24
+
+
+@pytest.fixture(scope="module")
+def real_size_folder(tmp_path_factory):
+    """One layer of the 7B layer sizes (hidden 3584, 28 query heads over 4 key/value heads of 128, intermediate
+    18944) with a small vocabulary, so that the kernels run at the shapes they are tuned for."""
+    from somi_inference_amd.config import Qwen2Config
+    from somi_inference_amd.weights import write_random_model
+    config = Qwen2Config(vocab_size=1031, hidden_size=3584, intermediate_size=18944, num_hidden_layers=1,
+                         num_attention_heads=28, num_key_value_heads=4, head_dim=128, rope_theta=1e6,
+                         rms_norm_eps=1e-6, tie_word_embeddings=False)
+    folder = str(tmp_path_factory.mktemp("real") / "one_layer_7b")
+    write_random_model(folder, config, seed=5)
+    return {"float32": peaky_folder(folder, folder + "_peaky", factor=3.0), "bfloat16": folder}, config
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_one_layer_of_the_7b_sizes_under_all_cuttings(dtype, real_size_folder):
+    """With sums over up to 18,944 terms the order of float32 additions shows: the float32 engine is held to
+    the accuracy of the plain float32 implementation itself, both measured against the plain implementation
+    in float64 (its error may be a few times the plain one's, not more).  The float32 run uses sharpened
+    attention (single keys decide); in bfloat16 that sharpening amplifies the rounding of q and k into
+    per-cent changes of the weights, so the bfloat16 run uses the weights as drawn."""
+    folders, config = real_size_folder
+    folder = folders[dtype]
+    cfg, weights = plain.read_model(folder)
+    tokens = token_ids(config.vocab_size, 333, 8)
+    want = plain.model_logits(cfg, weights, tokens)
+    cfg64, weights64 = plain.read_model(folder, dtype=torch.float64)
+    want64 = plain.model_logits(cfg64, weights64, tokens)
+    plain_error = float((want.double() - want64).abs().max())
+
+    def check(got, rows, what):
+        if dtype == "float32":
+            error = float((got.double().cpu() - want64[rows]).abs().max())
+            assert error <= 4 * plain_error + 1e-6, f"{what}: error {error:.3e}, the plain float32 implementation's {plain_error:.3e}"
+        else:
+            # bfloat16 rounds to 2^-9 relative at about six places per layer (normed input, projections, gate,
+            # attention weights, sub-layer outputs); independent roundings add up to roughly half a per cent of
+            # the logits' size.  The bounds sit at four times that (rms) and at 3 % for a single element; a
+            # fault (wrong key, page or row) changes logits by their own size.
+            ref = want[rows]
+            error = (got.float().cpu() - ref).abs()
+            assert float(error.max()) <= 0.03 * float(ref.abs().max()), f"{what}: max error {float(error.max()):.3e}"
+            assert float(error.pow(2).mean().sqrt()) <= 0.02 * float(ref.pow(2).mean().sqrt()), \
+                f"{what}: rms error {float(error.pow(2).mean().sqrt()):.3e} of rms {float(ref.pow(2).mean().sqrt()):.3e}"
+
+    runner, _ = make_engine(folder, dtype, 16, 64, max_requests=4)
+    everything = list(range(len(tokens)))
+    whole = run_portions(runner, "w", tokens, [333])
+    check(whole, everything, f"7B layer sizes {dtype}: whole prompt")
+    cut = run_portions(runner, "c", tokens, [150, 2, 37, 1, 1, 64, 9, 33] + [1] * 36)
+    check(cut, everything, f"7B layer sizes {dtype}: portions and decoded tokens")
+    if dtype == "float32":
+        assert torch.equal(cut, whole)
+    # three requests decoding together after prompts of different lengths
+    prompts = {"a": tokens[:40], "b": tokens[:111], "c": tokens[:290]}
+    for rid, prompt in prompts.items():
+        runner.begin(rid)
+        runner.step([StepEntry(rid, prompt, [])])
+    for step in range(20):
+        entries = [StepEntry(rid, [tokens[len(p) + step]], [0]) for rid, p in prompts.items()]
+        got = runner.step(entries).cpu()
+        check(got, [len(p) + step for p in prompts.values()], f"7B layer sizes {dtype}: batched decode step {step}")
