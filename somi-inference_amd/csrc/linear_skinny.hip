@@ -3,100 +3,162 @@
 //
 // Reference: the same nn.Linear products as linear_plain.hip (somi_inference/models/qwen2.py:221-222,
 // 268-271; qwen2_adapter.py:60-62); the reference leaves them to a library.  With few rows the product
-// is bound by reading w once from HBM, so the kernel is built around that stream:
-//   * a workgroup owns 16, 32 or 64 output columns (rows of w) and all rows of x; its wavefronts take
-//     64-wide blocks of K in turn, so that at any time the workgroup reads (wavefronts * 128) contiguous
-//     bytes of each of its weight rows;
-//   * a lane loads 2 x 16 bytes of one weight row and of one x row per block and issues two
-//     v_mfma_f32_16x16x32_bf16 per 16 rows of x (w is the A operand, so a lane ends up with four
-//     consecutive output columns of one row of x);
-//   * the partial sums of the wavefronts are added through LDS in wavefront order, which fixes the
-//     order of the additions whatever else runs.
-// x is small and stays in L2; it is read directly.
+// is bound by reading w once from HBM, so the kernel is built around that stream.  The matrix core
+// wants lane l to hold 8 k-values of row (l % 16); a load straight into that layout makes every
+// group of four lanes touch four different rows (16 bytes from each of 64 places per instruction),
+// which costs a fifth of the bandwidth.  Here a wavefront reads whole pieces of rows instead (8
+// consecutive lanes read 128 consecutive bytes of one row, or 16 lanes 256 bytes), keeps DEPTH such
+// chunks in flight in registers, and turns them through a private piece of LDS into the operand layout:
+//   * a workgroup owns NS blocks of 16 output columns and all rows of x; its wavefronts take chunks
+//     of CK values of K in turn; a chunk is the workgroup's 16 * NS rows of w and the rows of x;
+//   * loads are buffer loads whose range ends at the last valid row, so rows past N or M read as zero
+//     without a branch; a chunk that crosses K is masked per lane the same way;
+//   * LDS rows are XOR-swizzled in 16-byte units so that neither the row-wise writes nor the
+//     column-wise operand reads collide;
+//   * w is the A operand, so a lane ends up with four consecutive output columns of one row of x;
+//   * partial sums of the wavefronts are added through LDS in wavefront order, which fixes the order
+//     of the additions whatever else runs.
 #include "common.h"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
 
-__device__ __forceinline__ bf16x8 load8(const bf16* p) { return *reinterpret_cast<const bf16x8*>(p); }
+#define SOMI_BUFFER_WORD3 0x00020000u            // raw buffer, 32-bit elements, no swizzle
+#define SOMI_OUT_OF_RANGE 0x80000000u
+#define SKINNY_MAX_WAVES 8
 
-template <int MT, int NS, int U, typename TO, bool SWIGLU>
-__global__ void __launch_bounds__(1024)
+template <int MT, int NS, int CK, int DEPTH, typename TO, bool SWIGLU, bool TAIL>
+__global__ void __launch_bounds__(SKINNY_MAX_WAVES * 64)
 linear_skinny_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, const float* __restrict__ bias,
                      TO* __restrict__ out, int M, int N, int K) {
-    extern __shared__ float red[];                   // [waves][NS][MT][64 lanes][4]
+    extern __shared__ __attribute__((aligned(16))) char lds[];
+    constexpr int ROW_BYTES = CK * 2;              // bytes of one row in a chunk: 256 or 128
+    constexpr int LPR = ROW_BYTES / 16;            // lanes that read one row: 16 or 8
+    constexpr int RPI = 64 / LPR;                  // rows per load instruction: 4 or 8
+    constexpr int WL = 16 / RPI;                   // load instructions per 16 rows: 4 or 2
+    constexpr int ROWS = 16 * (NS + MT);
+    constexpr int WAVE_BYTES = ROWS * ROW_BYTES;
+    constexpr int NL = (NS + MT) * WL;             // loads per lane and chunk
+    constexpr int TILES = NS * MT;
+
     const int waves = blockDim.x >> 6;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int r = lane & 15, g = lane >> 4;
     const int n0 = blockIdx.x * (16 * NS);
-    const bf16* wp[NS];
+    char* mine = lds + wave * WAVE_BYTES;
+
+    const int rows_here = min(16 * NS, N - n0);
+    const __amdgpu_buffer_rsrc_t wres = __builtin_amdgcn_make_buffer_rsrc(
+        (void*)(w + (int64_t)n0 * K), 0, (int)((int64_t)rows_here * K * 2), SOMI_BUFFER_WORD3);
+    const __amdgpu_buffer_rsrc_t xres = __builtin_amdgcn_make_buffer_rsrc(
+        (void*)x, 0, (int)((int64_t)M * K * 2), SOMI_BUFFER_WORD3);
+
+    // where this lane reads (bytes from the start of the workgroup's rows) and writes (bytes in LDS)
+    const int lrow = lane / LPR, lchunk = lane % LPR;
+    unsigned goff[NL];
+    int soff[NL];
 #pragma unroll
-    for (int s = 0; s < NS; ++s) {
-        const int row = n0 + s * 16 + r;
-        wp[s] = w + (int64_t)(row < N ? row : N - 1) * K + g * 16;
+    for (int i = 0; i < NL; ++i) {
+        const int tile = i / WL, j = i % WL;       // tiles 0..NS-1 are w, the others are x
+        const int row16 = j * RPI + lrow;          // row inside the tile
+        const int row = tile < NS ? tile * 16 + row16 : (tile - NS) * 16 + row16;
+        goff[i] = ((unsigned)row * (unsigned)K + lchunk * 8) * 2u;
+        const int swz = CK == 128 ? (row16 & 15) : ((row16 >> 1) & 7);
+        soff[i] = (tile * 16 + row16) * ROW_BYTES + ((lchunk ^ swz) << 4);
     }
-    const bf16* xp[MT];
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-        const int m = mt * 16 + r;
-        xp[mt] = x + (int64_t)(m < M ? m : M - 1) * K + g * 16;
-    }
+    const int rswz = CK == 128 ? r : ((r >> 1) & 7);
+
     f32x4 acc[NS][MT];
 #pragma unroll
     for (int s = 0; s < NS; ++s)
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) acc[s][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    const int stride = waves * 64;
-    int k0 = wave * 64;
-    // U whole blocks per trip: all their loads are issued before the first product
-    for (; k0 + (U - 1) * stride + 64 <= K; k0 += U * stride) {
-        bf16x8 wa[U][NS], wb[U][NS], xa[U][MT], xb[U][MT];
+    const int chunks = (K + CK - 1) / CK;
+    const int mine_n = wave < chunks ? (chunks - wave + waves - 1) / waves : 0;
+
+    auto issue = [&](u32x4 (&st)[NL], int at) {
+        const int k0 = (wave + at * waves) * CK;
+        const bool inside = !TAIL || k0 + lchunk * 8 < K;
 #pragma unroll
-        for (int u = 0; u < U; ++u)
+        for (int i = 0; i < NL; ++i) {
+            const unsigned off = inside ? goff[i] + (unsigned)k0 * 2u : SOMI_OUT_OF_RANGE;
+            st[i] = __builtin_amdgcn_raw_buffer_load_b128(i < NS * WL ? wres : xres, off, 0, 0);
+        }
+    };
+    auto stash = [&](const u32x4 (&st)[NL]) {
+#pragma unroll
+        for (int i = 0; i < NL; ++i) *reinterpret_cast<u32x4*>(mine + soff[i]) = st[i];
+    };
+    auto operand = [&](int tile, int c) -> bf16x8 {
+        return *reinterpret_cast<const bf16x8*>(mine + (tile * 16 + r) * ROW_BYTES + ((c ^ rswz) << 4));
+    };
+    // the k-values of a 64-wide block are dealt to the two products as 16-byte pieces 2g and 2g + 1 of
+    // lane group g: any order serves as long as w and x use the same
+    auto compute = [&]() {
+#pragma unroll
+        for (int cb = 0; cb < CK / 64; ++cb) {
+            bf16x8 xa[MT], xb[MT];
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                xa[mt] = operand(NS + mt, cb * 8 + 2 * g);
+                xb[mt] = operand(NS + mt, cb * 8 + 2 * g + 1);
+            }
 #pragma unroll
             for (int s = 0; s < NS; ++s) {
-                wa[u][s] = load8(wp[s] + k0 + u * stride);
-                wb[u][s] = load8(wp[s] + k0 + u * stride + 8);
-            }
-#pragma unroll
-        for (int u = 0; u < U; ++u)
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt) {
-                xa[u][mt] = load8(xp[mt] + k0 + u * stride);
-                xb[u][mt] = load8(xp[mt] + k0 + u * stride + 8);
-            }
-#pragma unroll
-        for (int u = 0; u < U; ++u)
-#pragma unroll
-            for (int s = 0; s < NS; ++s)
+                const bf16x8 wa = operand(s, cb * 8 + 2 * g), wb = operand(s, cb * 8 + 2 * g + 1);
 #pragma unroll
                 for (int mt = 0; mt < MT; ++mt) {
-                    acc[s][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[u][s], xa[u][mt], acc[s][mt], 0, 0, 0);
-                    acc[s][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wb[u][s], xb[u][mt], acc[s][mt], 0, 0, 0);
+                    acc[s][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa, xa[mt], acc[s][mt], 0, 0, 0);
+                    acc[s][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wb, xb[mt], acc[s][mt], 0, 0, 0);
                 }
-    }
-    for (; k0 < K; k0 += stride) {                   // remaining blocks; the last may be partial (K % 8 == 0)
-        const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
-        const bool ha = k0 + g * 16 < K, hb = k0 + g * 16 + 8 < K;
-        bf16x8 xa[MT], xb[MT];
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-            xa[mt] = ha ? load8(xp[mt] + k0) : zero;
-            xb[mt] = hb ? load8(xp[mt] + k0 + 8) : zero;
-        }
-#pragma unroll
-        for (int s = 0; s < NS; ++s) {
-            const bf16x8 wa = ha ? load8(wp[s] + k0) : zero, wb = hb ? load8(wp[s] + k0 + 8) : zero;
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt) {
-                acc[s][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa, xa[mt], acc[s][mt], 0, 0, 0);
-                acc[s][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wb, xb[mt], acc[s][mt], 0, 0, 0);
             }
         }
+    };
+
+    // DEPTH chunks in flight: set d holds chunk `at + d`.  The loop is entered on one path only, with
+    // every set issued, so that the waits inside it count loads exactly.
+    u32x4 st[DEPTH][NL];
+    if (mine_n >= DEPTH) {
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d) issue(st[d], d);
+        int at = 0;
+        for (; at + 2 * DEPTH - 1 < mine_n; at += DEPTH) {
+#pragma unroll
+            for (int d = 0; d < DEPTH; ++d) {
+                stash(st[d]);
+                issue(st[d], at + DEPTH + d);
+                compute();
+            }
+        }
+        // DEPTH to 2 * DEPTH - 1 chunks are left
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d) {
+            stash(st[d]);
+            if (d < DEPTH - 1 && at + DEPTH + d < mine_n) issue(st[d], at + DEPTH + d);
+            compute();
+        }
+#pragma unroll
+        for (int d = 0; d < DEPTH - 1; ++d)
+            if (at + DEPTH + d < mine_n) {
+                stash(st[d]);
+                compute();
+            }
+    } else {
+#pragma unroll
+        for (int d = 0; d < DEPTH - 1; ++d)
+            if (d < mine_n) issue(st[d], d);
+#pragma unroll
+        for (int d = 0; d < DEPTH - 1; ++d)
+            if (d < mine_n) {
+                stash(st[d]);
+                compute();
+            }
     }
 
-    constexpr int TILES = NS * MT;
+    __syncthreads();                                 // every wavefront is done with its staging space
+    float* red = reinterpret_cast<float*>(lds);      // [waves][TILES][64 lanes][4]
 #pragma unroll
     for (int s = 0; s < NS; ++s)
 #pragma unroll
@@ -137,43 +199,60 @@ linear_skinny_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, con
     }
 }
 
-template <int MT, int NS, int U, typename TO>
-static int launch_skinny(const void* x, const void* w, const float* bias, void* out, int M, int N, int K, int waves,
-                         bool swiglu, hipStream_t stream) {
-    const size_t smem = (size_t)waves * NS * MT * 256 * sizeof(float);
+// LDS of a launch: the staging space of every wavefront, or the partial sums, whichever is larger.
+static size_t skinny_lds(int mt, int strips, int chunk, int waves) {
+    const size_t staging = (size_t)16 * (strips + mt) * chunk * 2, sums = (size_t)strips * mt * 1024;
+    return waves * (staging > sums ? staging : sums);
+}
+
+template <int MT, int NS, int CK, int DEPTH, typename TO, bool SW, bool TL>
+static void skinny_launch_kernel(const void* x, const void* w, const float* bias, void* out, int M, int N, int K,
+                                 int waves, hipStream_t stream) {
+    const size_t smem = skinny_lds(MT, NS, CK, waves);
     const dim3 grid(ceil_div(N, 16 * NS)), block(waves * 64);
-    if (swiglu && NS >= 2)
-        hipLaunchKernelGGL((linear_skinny_kernel<MT, (NS >= 2 ? NS : 2), U, TO, true>), grid, block, smem, stream,
-                           (const bf16*)x, (const bf16*)w, bias, (TO*)out, M, N, K);
-    else
-        hipLaunchKernelGGL((linear_skinny_kernel<MT, NS, U, TO, false>), grid, block, smem, stream,
-                           (const bf16*)x, (const bf16*)w, bias, (TO*)out, M, N, K);
+    if (smem > 64 * 1024)                            // beyond the default limit of dynamic LDS
+        (void)hipFuncSetAttribute((const void*)linear_skinny_kernel<MT, NS, CK, DEPTH, TO, SW, TL>,
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    hipLaunchKernelGGL((linear_skinny_kernel<MT, NS, CK, DEPTH, TO, SW, TL>), grid, block, smem, stream,
+                       (const bf16*)x, (const bf16*)w, bias, (TO*)out, M, N, K);
+}
+
+template <int MT, int NS, int CK, int DEPTH, typename TO>
+static int skinny_launch(const void* x, const void* w, const float* bias, void* out, int M, int N, int K, int waves,
+                         bool swiglu, hipStream_t stream) {
+    const bool tail = K % CK != 0;
+    if constexpr (NS >= 2) {
+        if (swiglu) {
+            if (tail) skinny_launch_kernel<MT, NS, CK, DEPTH, TO, true, true>(x, w, bias, out, M, N, K, waves, stream);
+            else skinny_launch_kernel<MT, NS, CK, DEPTH, TO, true, false>(x, w, bias, out, M, N, K, waves, stream);
+            SOMI_LAUNCH_CHECK("linear_skinny");
+            return 0;
+        }
+    }
+    if (tail) skinny_launch_kernel<MT, NS, CK, DEPTH, TO, false, true>(x, w, bias, out, M, N, K, waves, stream);
+    else skinny_launch_kernel<MT, NS, CK, DEPTH, TO, false, false>(x, w, bias, out, M, N, K, waves, stream);
     SOMI_LAUNCH_CHECK("linear_skinny");
     return 0;
 }
 
-template <int MT, int NS, typename TO>
-static int launch_skinny_u(const void* x, const void* w, const float* bias, void* out, int M, int N, int K,
-                           int waves, int unroll, bool swiglu, hipStream_t stream) {
-    if (NS * MT <= 4 && unroll >= 2)
-        return launch_skinny<MT, NS, 2, TO>(x, w, bias, out, M, N, K, waves, swiglu, stream);
-    return launch_skinny<MT, NS, 1, TO>(x, w, bias, out, M, N, K, waves, swiglu, stream);
-}
-
+#ifndef SOMI_SKINNY_NO_ENTRY_POINTS
+// The shapes that are built: 1, 2 or 4 strips with chunks of 64, two chunks in flight.
 template <int MT, typename TO>
-static int launch_skinny_ns(const void* x, const void* w, const float* bias, void* out, int M, int N, int K,
-                            int waves, int strips, int unroll, bool swiglu, hipStream_t stream) {
-    if (strips >= 4) return launch_skinny_u<MT, 4, TO>(x, w, bias, out, M, N, K, waves, unroll, swiglu, stream);
-    if (strips >= 2) return launch_skinny_u<MT, 2, TO>(x, w, bias, out, M, N, K, waves, unroll, swiglu, stream);
-    return launch_skinny_u<MT, 1, TO>(x, w, bias, out, M, N, K, waves, unroll, swiglu, stream);
+static int skinny_strips(const void* x, const void* w, const float* bias, void* out, int M, int N, int K, int waves,
+                         int strips, bool swiglu, hipStream_t stream) {
+    if (strips >= 4) return skinny_launch<MT, 4, 64, 2, TO>(x, w, bias, out, M, N, K, waves, swiglu, stream);
+    if (strips >= 2) return skinny_launch<MT, 2, 64, 2, TO>(x, w, bias, out, M, N, K, waves, swiglu, stream);
+    return skinny_launch<MT, 1, 64, 2, TO>(x, w, bias, out, M, N, K, waves, swiglu, stream);
 }
 
 static int skinny_dispatch(const void* x, const void* w, const float* bias, void* out, int out_dtype, int M, int N,
-                           int K, int waves, int strips, int unroll, bool swiglu, hipStream_t stream) {
+                           int K, int waves, int strips, bool swiglu, hipStream_t stream) {
     const int mt = ceil_div(M, 16);
-#define SOMI_SKINNY(MT)                                                                                                  \
-    return out_dtype == SOMI_BF16 ? launch_skinny_ns<MT, bf16>(x, w, bias, out, M, N, K, waves, strips, unroll, swiglu, stream)   \
-                                  : launch_skinny_ns<MT, float>(x, w, bias, out, M, N, K, waves, strips, unroll, swiglu, stream)
+    SOMI_REQUIRE(skinny_lds(mt, strips, 64, waves) <= 160 * 1024,
+                 "linear_skinny: %d wavefronts with %d strips need more than 160 KB of LDS", waves, strips);
+#define SOMI_SKINNY(MT)                                                                                              \
+    return out_dtype == SOMI_BF16 ? skinny_strips<MT, bf16>(x, w, bias, out, M, N, K, waves, strips, swiglu, stream)  \
+                                  : skinny_strips<MT, float>(x, w, bias, out, M, N, K, waves, strips, swiglu, stream)
     switch (mt) {
         case 1: SOMI_SKINNY(1);
         case 2: SOMI_SKINNY(2);
@@ -187,6 +266,7 @@ static int skinny_check(const void* x, const void* w, int out_dtype, int M, int 
     SOMI_REQUIRE(M >= 0 && N > 0 && K > 0, "linear_skinny: bad sizes M=%d N=%d K=%d", M, N, K);
     SOMI_REQUIRE(M <= 64, "linear_skinny: at most 64 rows, got %d", M);
     SOMI_REQUIRE(K % 8 == 0, "linear_skinny: K (%d) must be a multiple of 8", K);
+    SOMI_REQUIRE((int64_t)K * 2 * 64 < (int64_t)1 << 31, "linear_skinny: K (%d) is too large", K);
     SOMI_REQUIRE(((uintptr_t)x % 16 == 0) && ((uintptr_t)w % 16 == 0), "linear_skinny: x and w must be 16-byte aligned");
     SOMI_REQUIRE(out_dtype == SOMI_BF16 || out_dtype == SOMI_F32, "linear_skinny: unknown out dtype %d", out_dtype);
     return 0;
@@ -194,26 +274,19 @@ static int skinny_check(const void* x, const void* w, int out_dtype, int M, int 
 
 static int skinny_auto(const void* x, const void* w, const float* bias, void* out, int out_dtype, int M, int N, int K,
                        bool swiglu, hipStream_t stream) {
+    // Launch shape, from measurements at 7B layer sizes on MI355X.  8 wavefronts split K.  A workgroup
+    // takes 2 (or 4) strips, reading x once for all of them, where that still leaves a workgroup for
+    // most compute units and x is more than a few rows; one strip otherwise.
     const int mt = ceil_div(M, 16);
-    // Launch shape, from measurements at 7B layer sizes on MI355X.  x comes from L2 and its traffic, not
-    // the weight stream, limits the kernel once there are several rows: then a wavefront computes 4
-    // blocks of 16 columns from one read of x wherever that still leaves two workgroups per compute
-    // unit.  One row is fastest with the widest split of K (16 wavefronts on one block of columns).
     const int blocks16 = ceil_div(N, 16);
-    int strips = swiglu ? 2 : 1, waves = 16, unroll = 1;
-    if (M > 1) {
-        if (blocks16 >= 2048) {
-            strips = 4;
-            waves = blocks16 / 4 >= 1024 ? 8 : 4;
-            unroll = 2;
-        } else {
-            waves = 8;
-        }
-    }
-    while (waves > 1 && waves * mt * strips > 32) waves /= 2;      // 32 KB of LDS for the partial sums
-    while (waves > 1 && waves * 64 > K + 63) waves /= 2;           // no more wavefronts than blocks of K
-    if (K / (waves * 64) < 2) unroll = 1;
-    return skinny_dispatch(x, w, bias, out, out_dtype, M, N, K, waves, strips, unroll, swiglu, stream);
+    int strips = 1;
+    if (blocks16 >= 256) strips = 2;
+    if (blocks16 >= 2048 && M <= 4) strips = 1;
+    if (blocks16 >= 4096 && mt >= 2) strips = 4;
+    if (swiglu && strips < 2) strips = 2;
+    int waves = SKINNY_MAX_WAVES;
+    while (waves > 1 && waves * 64 > K + 63) waves /= 2;           // no more wavefronts than chunks of K
+    return skinny_dispatch(x, w, bias, out, out_dtype, M, N, K, waves, strips, swiglu, stream);
 }
 
 // x: [M, K] bfloat16, w: [N, K] bfloat16, bias: [N] float32 or null, out: [M, N] bfloat16 or float32.
@@ -236,14 +309,14 @@ extern "C" int somi_linear_skinny_swiglu(const void* x, const void* w, void* out
     return skinny_auto(x, w, nullptr, out, out_dtype, M, 2 * I, K, true, stream);
 }
 
-// The same product with the launch shape given by the caller (wavefronts per workgroup, 16-column
-// strips per wavefront: 1, 2 or 4, unroll depth: 1 or 2): for measuring how the shape should be chosen.
+// The same product with the launch shape given by the caller (wavefronts per workgroup: 1 to 8; 16-column
+// strips per workgroup: 1, 2 or 4): for measuring how the shape should be chosen.
 extern "C" int somi_linear_skinny_shaped(const void* x, const void* w, const float* bias, void* out, int out_dtype,
-                                         int M, int N, int K, int waves, int strips, int unroll, hipStream_t stream) {
+                                         int M, int N, int K, int waves, int strips, hipStream_t stream) {
     if (skinny_check(x, w, out_dtype, M, N, K)) return 1;
     SOMI_REQUIRE(strips == 1 || strips == 2 || strips == 4, "linear_skinny: strips must be 1, 2 or 4");
-    SOMI_REQUIRE(waves >= 1 && waves <= 16 && waves * ceil_div(M, 16) * strips <= 32,
-                 "linear_skinny: bad wavefront count %d", waves);
+    SOMI_REQUIRE(waves >= 1 && waves <= SKINNY_MAX_WAVES, "linear_skinny: bad wavefront count %d", waves);
     if (M == 0) return 0;
-    return skinny_dispatch(x, w, bias, out, out_dtype, M, N, K, waves, strips, unroll, false, stream);
+    return skinny_dispatch(x, w, bias, out, out_dtype, M, N, K, waves, strips, false, stream);
 }
+#endif

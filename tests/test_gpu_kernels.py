@@ -220,7 +220,7 @@ def test_repetition_penalty_rule():
 
 
 @pytest.mark.parametrize("m, n, k", [(1, 503, 192), (7, 64, 72), (16, 130, 200), (17, 33, 1000), (48, 3584 + 16, 3584),
-                                     (64, 70, 18944), (8, 152064 // 16 + 3, 512)])
+                                     (64, 70, 18944), (8, 152064 // 16 + 3, 512), (2, 32768 + 16, 128), (20, 65536 + 48, 64)])
 def test_linear_skinny_mfma_against_float32(m, n, k):
     x, w, b = rnd(m, k, dtype="bfloat16", seed=1), rnd(n, k, dtype="bfloat16", seed=2, scale=0.05), rnd(n, seed=3)
     want = F.linear(x.float(), w.float(), b)
