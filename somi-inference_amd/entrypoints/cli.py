@@ -46,6 +46,8 @@ def parse_args(argv: list[str] | None = None) -> argparse.Namespace:
     parser.add_argument("--repetition-penalty", type=float, default=1.0,
                         help="Repetition penalty applied by the sampler.")
     parser.add_argument("--output-file", type=str, default=None, help="Append results to a JSONL file.")
+    parser.add_argument("--warm-up", action="store_true",
+                        help="Let the library time its matrix products for full prompt portions first.")
     return parser.parse_args(argv)
 
 
@@ -71,6 +73,8 @@ def main(argv: list[str] | None = None) -> int:
     llm = LLM(model_dir, num_blocks=args.num_blocks, block_size=args.block_size,
               max_concurrent=args.max_concurrent, device=args.device, dtype=args.dtype,
               max_num_batched_tokens=args.max_num_batched_tokens, max_chunk=args.max_chunk, seed=args.seed)
+    if args.warm_up:
+        llm.warm_up()
     outputs = llm.generate(prompts, max_new_tokens=args.max_new_tokens, temperature=args.temperature,
                            top_k=args.top_k, top_p=args.top_p, repetition_penalty=args.repetition_penalty,
                            seed=args.seed)

@@ -80,6 +80,17 @@ class LLM:
         self.engine = Engine(self.runner, self.scheduler, self.sampler, eos_token_id)
         self._next_seq_id = 0
 
+    # ----------------------------------------------------------------- warm-up
+    def warm_up(self) -> int:
+        """Optional: lets the library time its solutions for the matrix products of a full prompt portion.
+
+        Not in the reference.  Worth a few seconds before long prompts are served in bfloat16 (the
+        float32 engine has no library products); returns the portion length that was tuned.
+        """
+        if self.dtype != "bfloat16":
+            return 0
+        return self.runner.tune_library_products(min(self.options.chunk, self.options.max_num_batched_tokens))
+
     # ---------------------------------------------------------------- generate
     def _encode(self, prompt) -> tuple[list[int], bool]:
         if isinstance(prompt, str):

@@ -149,3 +149,23 @@ def test_command_line_generates_and_appends_jsonl(model_folders, tmp_path):
     want = plain.greedy_generate(cfg, weights, prompt, 5, eos=cfg.get("eos_token_id"))
     assert record["prompt"] == prompt and record["output"] == want
     assert json.loads(out_file.read_text().strip()) == record
+
+
+def test_warm_up_tunes_library_products_without_changing_results(model_folders, tmp_path, monkeypatch):
+    """The optional warm-up lets the library pick its matrix-product solutions for full prompt portions: the
+    tokens stay what the plain implementation gives, the pages are all given back, and no file appears in
+    the working directory."""
+    monkeypatch.chdir(tmp_path)
+    folder = model_folders["B"]
+    llm = LLM(folder, dtype="bfloat16", num_blocks=64, block_size=8, max_num_batched_tokens=96, max_concurrent=4,
+              eos_token_id=-1)
+    free_before = llm.kv_manager.free_pages()
+    assert llm.warm_up() == 96
+    assert llm.kv_manager.free_pages() == free_before
+    llm.kv_manager.check_invariants()
+    prompts = [token_ids(TINY["B"]["config"].vocab_size, 96, 3)]
+    want, cfg, weights = plain_greedy(folder, prompts, 6)
+    got = llm.generate(prompts, max_new_tokens=6, temperature=0.0)
+    assert_greedy_matches(got, want, prompts, cfg, weights, exact=False)
+    assert list(tmp_path.iterdir()) == []
+    assert LLM(folder, dtype="float32", num_blocks=64, block_size=8).warm_up() == 0
