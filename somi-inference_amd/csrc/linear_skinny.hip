@@ -14,7 +14,7 @@
 //   * loads are buffer loads whose range ends at the last valid row, so rows past N or M read as zero
 //     without a branch; a chunk that crosses K is masked per lane the same way;
 //   * LDS rows are XOR-swizzled in 16-byte units so that neither the row-wise writes nor the
-//     column-wise operand reads collide;
+//     column-wise operand reads collide, whether 8 or 16 lanes are served per cycle;
 //   * w is the A operand, so a lane ends up with four consecutive output columns of one row of x;
 //   * partial sums of the wavefronts are added through LDS in wavefront order, which fixes the order
 //     of the additions whatever else runs.
@@ -64,10 +64,10 @@ linear_skinny_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, con
         const int row16 = j * RPI + lrow;          // row inside the tile
         const int row = tile < NS ? tile * 16 + row16 : (tile - NS) * 16 + row16;
         goff[i] = ((unsigned)row * (unsigned)K + lchunk * 8) * 2u;
-        const int swz = CK == 128 ? (row16 & 15) : ((row16 >> 1) & 7);
+        const int swz = CK == 128 ? (row16 & 15) : ((row16 & 7) ^ (row16 >> 3));
         soff[i] = (tile * 16 + row16) * ROW_BYTES + ((lchunk ^ swz) << 4);
     }
-    const int rswz = CK == 128 ? r : ((r >> 1) & 7);
+    const int rswz = CK == 128 ? r : ((r & 7) ^ (r >> 3));
 
     f32x4 acc[NS][MT];
 #pragma unroll

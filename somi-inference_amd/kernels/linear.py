@@ -11,6 +11,24 @@ SKINNY_ROWS = 64       # up to here it beats the library product at 7B layer siz
                        # of 64 requests: gate_up with the gate fused in 80 us against 90 + 5, down 55 against 60)
 
 
+def _mid_is_faster(m: int, n: int, k: int) -> bool:
+    """Measured at 7B layer sizes: the kernel that shares x inside a workgroup and splits K over workgroups
+    wins from 17 rows on where K is long and the columns are few (down: 31 us against 38 at 32 rows, 38
+    against 53 at 64), and above 32 rows where there are very many columns (gate_up: 71 us against 79)."""
+    if m <= 16:
+        return False
+    return (k >= 8192 and n <= 8192) or (m > 32 and n >= 16384)
+
+
+def linear_swiglu(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+    """silu(x @ gate.T) * (x @ up.T) for at most SKINNY_ROWS bfloat16 rows; weight: [2 I, K], gate and up rows
+    interleaved in blocks of 16."""
+    m, k = x.shape
+    if _mid_is_faster(m, weight.shape[0], k):
+        return ops.linear_mid(x, weight, swiglu=True)
+    return ops.linear_skinny_swiglu(x, weight)
+
+
 def linear(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None,
            out_dtype: torch.dtype | None = None, bias_lowp: torch.Tensor | None = None) -> torch.Tensor:
     """x @ weight.T (+ bias).
@@ -28,6 +46,8 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = No
     if k % 8 != 0 or x.data_ptr() % 16 or weight.data_ptr() % 16:
         return ops.linear_plain(x, weight, bias, out_dtype)
     if m <= SKINNY_ROWS:
+        if _mid_is_faster(m, weight.shape[0], k):
+            return ops.linear_mid(x, weight, bias, out_dtype)
         return ops.linear_skinny(x, weight, bias, out_dtype)
     if out_dtype == torch.float32:
         return torch.cat([ops.linear_skinny(x[at:at + SKINNY_MAX_ROWS], weight, bias, out_dtype)

@@ -294,6 +294,39 @@ def linear_skinny_swiglu(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
     return out
 
 
+MID_WORKSPACE_FLOATS = 8 << 20        # 32 MB per device: partial sums of a split K (the kernel splits less if it is short)
+_mid_workspaces: dict[torch.device, torch.Tensor] = {}
+
+
+def _mid_workspace(device: torch.device) -> torch.Tensor:
+    """One workspace per device, shared by every launch: the launches of a device run on one stream."""
+    held = _mid_workspaces.get(device)
+    if held is None:
+        held = _mid_workspaces[device] = torch.empty((MID_WORKSPACE_FLOATS,), dtype=torch.float32, device=device)
+    return held
+
+
+def linear_mid(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None,
+               out_dtype: torch.dtype | None = None, swiglu: bool = False) -> torch.Tensor:
+    """x @ weight.T (+ bias) for at most 64 bfloat16 rows, x shared by the wavefronts of a workgroup, K split
+    over workgroups where the columns do not fill the device.  With ``swiglu`` weight is [2 I, K] with gate and
+    up rows interleaved in blocks of 16 and the result is silu(x @ gate.T) * (x @ up.T)."""
+    _need(x, "linear input", torch.bfloat16)
+    m, k = x.shape
+    _need(weight, "linear weight", torch.bfloat16)
+    n = weight.shape[0]
+    if weight.shape[1] != k or (swiglu and n % 32):
+        raise KernelError(f"linear_mid: weight {tuple(weight.shape)} does not fit input width {k}")
+    if bias is not None:
+        _need(bias, "linear bias", torch.float32, (n,))
+    out_dtype = out_dtype or x.dtype
+    out = torch.empty((m, n // 2 if swiglu else n), dtype=out_dtype, device=x.device)
+    workspace = _mid_workspace(x.device)
+    _check(library().somi_linear_mid(_ptr(x), _ptr(weight), _ptr(bias), _ptr(out), dtype_code(out_dtype), m, n, k,
+                                     1 if swiglu else 0, _ptr(workspace), ctypes.c_int64(workspace.numel()), _stream()))
+    return out
+
+
 def sample(logits: torch.Tensor, temperature: torch.Tensor, uniform: torch.Tensor) -> torch.Tensor:
     """One token per row: argmax where temperature is 0, else an inverse-CDF draw from softmax(logits / T)."""
     _need(logits, "logits", torch.float32)

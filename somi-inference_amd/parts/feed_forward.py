@@ -49,5 +49,5 @@ class SwiGLU(FeedForward):
         if not self.interleaved:
             return self.down(ops.silu_mul(self.gate_up(x)))
         if x.shape[0] <= linear_kernels.SKINNY_ROWS and x.data_ptr() % 16 == 0:
-            return self.down(ops.linear_skinny_swiglu(x, self.gate_up.weight))
+            return self.down(linear_kernels.linear_swiglu(x, self.gate_up.weight))
         return self.down(ops.silu_mul(self.gate_up(x), block=self.INTERLEAVE))

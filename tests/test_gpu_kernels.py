@@ -373,3 +373,36 @@ def test_linear_skinny_with_the_gate_fused_in(m, inter, k):
     torch.testing.assert_close(unfused.float(), want, atol=scale * 2 ** -6, rtol=2 ** -5)
     with pytest.raises(KernelError, match="does not fit"):
         ops.linear_skinny_swiglu(x, merged[:-16].contiguous())
+
+
+@pytest.mark.parametrize("m, n, k", [(1, 70, 72), (17, 130, 200), (40, 200, 2048), (64, 70, 18944), (33, 3584 + 16, 1000),
+                                     (48, 16384 + 80, 256), (64, 640, 8192)])
+def test_linear_mid_shared_rows_and_split_k_against_float32(m, n, k):
+    """The product for some tens of rows: x shared inside a workgroup, K split over workgroups with the partial
+    sums added by a second kernel.  Shapes with one and several splits, a K that ends inside a chunk, columns
+    that do not fill a tile."""
+    x, w, b = rnd(m, k, dtype="bfloat16", seed=1), rnd(n, k, dtype="bfloat16", seed=2, scale=0.05), rnd(n, seed=3)
+    want = F.linear(x.float(), w.float(), b)
+    scale = float(want.abs().max())
+    got32 = ops.linear_mid(x, w, b, torch.float32)
+    torch.testing.assert_close(got32, want, atol=2e-5 * scale * math.sqrt(k), rtol=1e-4)     # float32 sums of exact products
+    got = ops.linear_mid(x, w, b)
+    assert got.dtype == torch.bfloat16
+    torch.testing.assert_close(got.float(), want, atol=scale * 2 ** -8, rtol=2 ** -7)         # one rounding to bfloat16
+    torch.testing.assert_close(ops.linear_mid(x, w, None, torch.float32), F.linear(x.float(), w.float()),
+                               atol=2e-5 * scale * math.sqrt(k), rtol=1e-4)
+    assert torch.equal(ops.linear_mid(x, w, b, torch.float32), got32)                         # a fixed order of additions
+    with pytest.raises(KernelError, match="64 rows"):
+        ops.linear_mid(rnd(65, k, dtype="bfloat16"), w)
+
+
+@pytest.mark.parametrize("m, inter, k", [(8, 48, 72), (33, 160, 1536), (64, 4096 + 32, 64), (50, 96, 8192)])
+def test_linear_mid_with_the_gate_fused_in(m, inter, k):
+    x = rnd(m, k, dtype="bfloat16", seed=1)
+    gate, up = rnd(inter, k, dtype="bfloat16", seed=2, scale=0.1), rnd(inter, k, dtype="bfloat16", seed=3, scale=0.1)
+    merged = torch.stack([gate.view(-1, 16, k), up.view(-1, 16, k)], dim=1).reshape(-1, k).contiguous()
+    want = F.silu(x.float() @ gate.float().t()) * (x.float() @ up.float().t())
+    got = ops.linear_mid(x, merged, swiglu=True)
+    scale = float(want.abs().max())
+    torch.testing.assert_close(got.float(), want, atol=scale * 2 ** -7, rtol=2 ** -6)
+    torch.testing.assert_close(got.float(), ops.linear_skinny_swiglu(x, merged).float(), atol=scale * 2 ** -7, rtol=2 ** -6)
