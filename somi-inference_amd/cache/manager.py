@@ -21,6 +21,7 @@ from __future__ import annotations
 from dataclasses import dataclass, field
 from typing import Hashable
 
+import numpy as np
 import torch
 
 from ..parts.base import FixedStateSpec, LayerCache, PagedKVSpec
@@ -41,6 +42,18 @@ class RequestCache:
     num_tokens: int = 0
     pages: list[list[int]] = field(default_factory=list)   # per group: logical page -> physical page or RELEASED
     state_slot: int = -1
+    # per group: the same as ``pages`` as an int32 array for the kernels' block tables (released pages read
+    # as page 0: the kernels never look below a window); kept beside the lists so that laying out a step
+    # copies a slice instead of walking every page of every request
+    rows: list[np.ndarray] = field(default_factory=list)
+
+    def note_page(self, group: int, logical: int, page: int) -> None:
+        row = self.rows[group]
+        if logical >= row.size:
+            grown = np.zeros(max(16, 2 * row.size, logical + 1), dtype=np.int32)
+            grown[:row.size] = row
+            self.rows[group] = row = grown
+        row[logical] = page
 
 
 class CacheManager:
@@ -97,7 +110,8 @@ class CacheManager:
         if not self._free_slots:
             raise CacheError(f"all {self.max_requests} request slots are in use")
         slot = self._free_slots.pop()
-        self._requests[request_id] = RequestCache(0, [[] for _ in self.groups], slot)
+        self._requests[request_id] = RequestCache(0, [[] for _ in self.groups], slot,
+                                                  [np.zeros(16, dtype=np.int32) for _ in self.groups])
         for cache in self.layer_caches:
             if cache is not None and cache.state is not None and cache.writes:
                 cache.state[slot].zero_()
@@ -155,15 +169,16 @@ class CacheManager:
         for group, n in zip(self.groups, needed):
             if n > group.pool.num_free:
                 raise OutOfPages(f"request {request_id!r} needs {n} more pages, {group.pool.num_free} are free")
-        for group, pages, n in zip(self.groups, record.pages, needed):
+        for g, (group, pages, n) in enumerate(zip(self.groups, record.pages, needed)):
             for _ in range(n):
                 pages.append(group.pool.allocate())
+                record.note_page(g, len(pages) - 1, pages[-1])
 
     def commit(self, request_id: Hashable, new_tokens: int) -> None:
         """Count the tokens a step wrote, and give back pages a window has passed."""
         record = self._get(request_id)
         record.num_tokens += new_tokens
-        for group, pages in zip(self.groups, record.pages):
+        for g, (group, pages) in enumerate(zip(self.groups, record.pages)):
             if self._pages_for(record.num_tokens) > len(pages):
                 raise CacheError(f"request {request_id!r}: tokens committed beyond the reserved pages")
             if group.window is None:
@@ -175,10 +190,16 @@ class CacheManager:
                 if pages[logical] != RELEASED:
                     group.pool.release(pages[logical])
                     pages[logical] = RELEASED
+                    record.note_page(g, logical, 0)
 
     # ------------------------------------------------------- tables for a step
     def page_list(self, group: int, request_id: Hashable) -> list[int]:
         return self._get(request_id).pages[group]
+
+    def table_row(self, group: int, request_id: Hashable) -> np.ndarray:
+        """The request's block-table row for the kernels: int32, one entry per logical page, released pages as 0."""
+        record = self._get(request_id)
+        return record.rows[group][:len(record.pages[group])]
 
     def slots(self, group: int, request_id: Hashable, start: int, count: int) -> list[int]:
         """Physical slot (page * block_size + offset) of positions start .. start + count - 1."""
@@ -203,6 +224,10 @@ class CacheManager:
                     if page in held:
                         raise CacheError(f"group {g}: page {page} held by {held[page]!r} and {request_id!r}")
                     held[page] = request_id
+            for request_id, record in self._requests.items():
+                mirror = [0 if page == RELEASED else page for page in record.pages[g]]
+                if record.rows[g][:len(mirror)].tolist() != mirror:
+                    raise CacheError(f"group {g}: the block-table row of {request_id!r} differs from its pages")
             free = group.pool.free_pages()
             if len(set(free)) != len(free):
                 raise CacheError(f"group {g}: a page is on the free list twice")

@@ -17,7 +17,7 @@ from typing import Hashable
 import numpy as np
 import torch
 
-from ..cache.manager import RELEASED, CacheManager
+from ..cache.manager import CacheManager
 
 
 @dataclass
@@ -85,16 +85,15 @@ def _layout(entries: list[StepEntry], cache: CacheManager, table_widths: list[in
     n, e = len(token_ids), len(entries)
     tables, slot_maps, widths = [], [], []
     for g in range(len(cache.groups)):
-        rows = [cache.page_list(g, info.request_id) for info in infos]
-        width = max(1, max((len(r) for r in rows), default=1))
+        rows = [cache.table_row(g, info.request_id) for info in infos]
+        width = max(1, max((r.size for r in rows), default=1))
         if table_widths is not None:
             if width > table_widths[g]:
                 raise ValueError(f"block table of width {width} does not fit the fixed width {table_widths[g]}")
             width = table_widths[g]
         table = np.zeros((e, width), dtype=np.int32)
         for r, pages in enumerate(rows):
-            # released pages read as page 0: the kernels never look below a window
-            table[r, :len(pages)] = [0 if p == RELEASED else p for p in pages]
+            table[r, :pages.size] = pages                # released pages read as page 0 there
         slots: list[int] = []
         for info in infos:
             slots.extend(cache.slots(g, info.request_id, info.first_position, info.length))

@@ -20,6 +20,22 @@ from .rng import uniform
 
 
 class Sampler:
+    def __init__(self) -> None:
+        self._greedy_inputs: dict[tuple[int, torch.device], torch.Tensor] = {}
+
+    def _pick_inputs(self, plist: list[SamplingParams], seeds: list[int], counters: list[int],
+                     device: torch.device) -> tuple[torch.Tensor, torch.Tensor]:
+        """Temperatures and uniform draws of the rows on the device, in one transfer (none for all-greedy rows)."""
+        rows = len(plist)
+        if all(p.temperature == 0.0 for p in plist):
+            held = self._greedy_inputs.get((rows, device))
+            if held is None:
+                held = self._greedy_inputs[(rows, device)] = torch.zeros(2 * rows, dtype=torch.float32, device=device)
+        else:
+            held = torch.tensor([p.temperature for p in plist] + [uniform(s, c) for s, c in zip(seeds, counters)],
+                                dtype=torch.float32).to(device)
+        return held[:rows], held[rows:]
+
     def sample(self, logits: torch.Tensor, params: SamplingParams | list[SamplingParams],
                token_histories: list[list[int]] | None = None,
                seeds: list[int] | None = None, counters: list[int] | None = None) -> list[int]:
@@ -69,7 +85,5 @@ class Sampler:
                 remove[0] = False
                 work[row, order[remove]] = float("-inf")
 
-        temperature = torch.tensor([p.temperature for p in plist], dtype=torch.float32, device=work.device)
-        draws = torch.tensor([uniform(s, c) for s, c in zip(seeds, counters)], dtype=torch.float32,
-                             device=work.device)
+        temperature, draws = self._pick_inputs(plist, seeds, counters, work.device)
         return ops.sample(work, temperature, draws).tolist()
