@@ -24,6 +24,10 @@ class DecoderModel:
         self.plan = plan
         self.runtime = runtime
         self.embedding = build_part("embedding", plan.embedding, prefix=plan.embedding_prefix)
+        self.embedding_position = None
+        if plan.embedding_position is not None:
+            self.embedding_position = build_part("position", plan.embedding_position,
+                                                 prefix=plan.embedding_position_prefix)
         self.layers = [build_part("block", layer.block, prefix=layer.prefix) for layer in plan.layers]
         self.final_norm = build_part("norm", plan.final_norm, prefix=plan.final_norm_prefix)
         self.head = build_part("head", plan.head, prefix=plan.head_prefix)
@@ -34,10 +38,16 @@ class DecoderModel:
     # ------------------------------------------------------------------ weights
     def weight_specs(self) -> list[WeightSpec]:
         specs: dict[str, WeightSpec] = {}
-        for part in [self.embedding, *self.layers, self.final_norm, self.head]:
+        for part in self._top_level_parts():
             for spec in part.weight_specs():
                 specs[spec.name] = spec
         return list(specs.values())
+
+    def _top_level_parts(self) -> list:
+        parts = [self.embedding, *self.layers, self.final_norm, self.head]
+        if self.embedding_position is not None:
+            parts.insert(1, self.embedding_position)
+        return parts
 
     def load(self, source: WeightSource) -> None:
         """Check the source against the declared tensors (one error for everything), then place them."""
@@ -45,6 +55,8 @@ class DecoderModel:
         check_weights(specs, source, self.plan.ignore_weights)
         fetch = WeightFetcher(specs, source, self.runtime.dtype, self.runtime.device)
         self.embedding.load(fetch, self.runtime)
+        if self.embedding_position is not None:
+            self.embedding_position.load(fetch, self.runtime)
         for layer in self.layers:
             layer.load(fetch, self.runtime)
         self.final_norm.load(fetch, self.runtime)
@@ -57,6 +69,8 @@ class DecoderModel:
         """True when every part says that its forward only launches work on the current stream from
         device-side arrays of the step (so a step can be captured once and replayed)."""
         parts = [self.embedding, self.final_norm, self.head]
+        if self.embedding_position is not None:
+            parts.append(self.embedding_position)
         for layer in self.layers:
             parts.append(layer)
             parts.extend(layer.parts())
@@ -80,6 +94,8 @@ class DecoderModel:
         if not self.loaded:
             raise RuntimeError("model weights are not loaded")
         h = self.embedding.forward(step.token_ids)
+        if self.embedding_position is not None:
+            self.embedding_position.encode_embeddings(h, step)
         stream = ResidualStream(h)
         for run, index in enumerate(self.order):
             self.layers[index].forward(stream, step, caches[run])

@@ -35,6 +35,8 @@ class ModelPlan:
     cache_from: dict[int, int] = field(default_factory=dict)   # run index -> earlier run index whose cache it reads
     ignore_weights: tuple[str, ...] = ()             # glob patterns of tensors a checkpoint may carry unused
     vocab_size: int = 0
+    embedding_position: PartSpec | None = None       # a position encoding applied to the embedded tokens
+    embedding_position_prefix: str = ""
 
     def run_order(self) -> tuple[int, ...]:
         return self.order if self.order else tuple(range(len(self.layers)))
@@ -53,6 +55,8 @@ def collect_weight_specs(plan: ModelPlan) -> list[WeightSpec]:
     """Every tensor the plan's parts declare, each name once (no device needed)."""
     specs: list[WeightSpec] = []
     specs += build_part("embedding", plan.embedding, prefix=plan.embedding_prefix).weight_specs()
+    if plan.embedding_position is not None:
+        specs += build_part("position", plan.embedding_position, prefix=plan.embedding_position_prefix).weight_specs()
     for layer in plan.layers:
         specs += build_part("block", layer.block, prefix=layer.prefix).weight_specs()
     specs += build_part("norm", plan.final_norm, prefix=plan.final_norm_prefix).weight_specs()
