@@ -89,7 +89,7 @@ def main() -> int:
     def decode_run(batch: int, steps: int, warmup: int) -> tuple[float, float]:
         """Fill ``batch`` requests up to context - (warmup + steps), then time ``steps`` decode steps.
         Returns (seconds, mean context length during the timed steps)."""
-        prompt_len = args.context - (warmup + steps)
+        prompt_len = args.context - (warmup + steps + 1)
         ids = [f"b{batch}_{i}" for i in range(batch)]
         for rid in ids:
             runner.begin(rid)
@@ -98,16 +98,26 @@ def main() -> int:
                 runner.step([StepEntry(rid, tokens[at:at + 2048], [])])
         last = torch.randint(0, config.vocab_size, (batch,), generator=gen).tolist()
 
-        def one_step(tokens: list[int]) -> list[int]:
-            logits = runner.step([StepEntry(rid, [tok], [0]) for rid, tok in zip(ids, tokens)])
-            return sampler.sample(logits, greedy)
+        placeholders = [StepEntry(rid, [0], [0]) for rid in ids]
 
+        def launch(previous):
+            """One decode step and its greedy pick, launched without waiting: the step takes the previous
+            pick straight from the device; the host reads every pick one step late."""
+            if isinstance(previous, list):
+                logits = runner.step([StepEntry(rid, [tok], [0]) for rid, tok in zip(ids, previous)])
+            else:
+                logits = runner.step(placeholders, device_tokens=previous.device)
+            return sampler.sample_async(logits, greedy)
+
+        newest = launch(last)
         for _ in range(warmup):
-            last = one_step(last)
+            older, newest = newest, launch(newest)
+            older.tolist()
         sync()
         start = time.perf_counter()
         for _ in range(steps):
-            last = one_step(last)
+            older, newest = newest, launch(newest)
+            older.tolist()
         sync()
         seconds = time.perf_counter() - start
         for rid in ids:

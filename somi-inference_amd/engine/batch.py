@@ -154,16 +154,29 @@ class StaticStep:
         self.table_widths = list(table_widths)
         sections, infos, widths = _layout(entries, cache, self.table_widths)
         self.sizes = [s.size for s in sections]
-        self.host = torch.empty(sum(self.sizes), dtype=torch.int32).pin_memory()
+        # Staging in pinned memory, several buffers in turn: the copy to the device is asynchronous, so the
+        # host can lay out the next step while the device still runs this one.  A buffer is written again
+        # only after the copy that read it has finished (its event).
+        self.hosts = [torch.empty(sum(self.sizes), dtype=torch.int32).pin_memory() for _ in range(self.STAGING)]
+        self.copied: list[torch.cuda.Event | None] = [None] * self.STAGING
+        self.turn = 0
         self.device_buffer = torch.empty(sum(self.sizes), dtype=torch.int32, device=device)
         # kernels that size their launch by the context use the widest the tables allow
         self.batch = _views(self.device_buffer, self.sizes, infos, widths, len(cache.groups), cache.block_size,
                             max_context=max(self.table_widths, default=1) * cache.block_size)
         self._fill(sections, infos)
 
+    STAGING = 4
+
     def _fill(self, sections, infos) -> None:
-        self.host.copy_(torch.from_numpy(np.concatenate(sections)))
-        self.device_buffer.copy_(self.host)      # blocking: the staging buffer is free again on return
+        turn, self.turn = self.turn, (self.turn + 1) % self.STAGING
+        if self.copied[turn] is not None:
+            self.copied[turn].synchronize()
+        np.concatenate(sections, out=self.hosts[turn].numpy())
+        self.device_buffer.copy_(self.hosts[turn], non_blocking=True)     # in stream order, after the last replay
+        event = torch.cuda.Event()
+        event.record()
+        self.copied[turn] = event
         self.batch.entries = infos
 
     def update(self, entries: list[StepEntry], cache: CacheManager) -> StepBatch:

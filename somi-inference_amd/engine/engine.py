@@ -11,11 +11,22 @@ mixed batch, and a finished request's pages are free for the very next step.
 from __future__ import annotations
 
 from collections import deque
+from dataclasses import dataclass
 
 from ..sampling.sampler import Sampler
 from .batch import StepEntry
 from .request import Request, RequestStatus
-from .scheduler import Scheduler, SchedulerOutput
+from .scheduler import ScheduledPortion, Scheduler, SchedulerOutput
+
+UNREAD = -1       # stands in a request's output for a token that is drawn but not yet read from the device
+
+
+@dataclass
+class _UnreadStep:
+    """The sampled portions of a launched step whose tokens the host has not read yet."""
+    portions: list[ScheduledPortion]
+    places: list[int]             # index of each portion's stand-in in its request's output_tokens
+    tokens: object                # sampling.PendingTokens
 
 
 class Engine:
@@ -26,40 +37,100 @@ class Engine:
         self.eos_token_id = -1 if eos_token_id is None else int(eos_token_id)   # -1: nothing ends a request early
         self.num_steps = 0
         self.last_output: SchedulerOutput | None = None
+        # Running ahead: while only decoding requests run, step n + 1 is launched with step n's tokens
+        # still on the device, and step n's tokens are read (and checked for EOS) while n + 1 runs.  A
+        # request that turns out to have ended at n has then run one token too far; that token is dropped.
+        self.run_ahead = bool(getattr(runner, "accepts_device_tokens", False)) and hasattr(sampler, "sample_async")
+        self.steps_run_ahead = 0
+        self._unread: _UnreadStep | None = None
 
     def add_request(self, request: Request) -> None:
         self.scheduler.add_request(request)
 
-    def _check_finished(self, request: Request, token: int) -> None:
+    def _check_finished(self, request: Request, token: int, count: int | None = None) -> None:
+        """``count``: how many tokens the request has with this one (its output may already hold a stand-in
+        for a later one)."""
+        count = len(request.output_tokens) if count is None else count
         if token == self.eos_token_id:
             self.scheduler.finish(request, "eos")
-        elif len(request.output_tokens) >= request.max_new_tokens:
+        elif count >= request.max_new_tokens:
             self.scheduler.finish(request, "length")
+
+    def _can_run_ahead(self) -> bool:
+        """The next step is known without the unread tokens' values: the same requests, one token each, nobody
+        waiting, nobody at its last token, no sampling rule that reads the history, pages free for all."""
+        unread, scheduler = self._unread, self.scheduler
+        if unread is None or scheduler.waiting or len(scheduler.running) > scheduler.max_num_batched_tokens:
+            return False
+        if [p.request for p in unread.portions] != scheduler.running:
+            return False
+        for request in scheduler.running:
+            if (request.num_pending != 1 or request.sampling_params.repetition_penalty != 1.0
+                    or len(request.output_tokens) >= request.max_new_tokens):
+                return False
+        return scheduler.cache.can_reserve([(r.request_id, 1) for r in scheduler.running])
+
+    def _read_unread(self) -> None:
+        """Read the tokens of the step that is still unread, put them in place and retire what ended."""
+        unread, self._unread = self._unread, None
+        if unread is None:
+            return
+        for portion, place, token in zip(unread.portions, unread.places, unread.tokens.tolist()):
+            request = portion.request
+            if request.status is RequestStatus.FINISHED:
+                continue                         # ended a step earlier: this was the token too far
+            request.output_tokens[place] = int(token)
+            self._check_finished(request, int(token), place + 1)
+            if request.status is RequestStatus.FINISHED:
+                del request.output_tokens[place + 1:]      # the stand-in of a step launched since
 
     def step(self) -> list[Request]:
         """One scheduling decision and one model step; returns the requests that finished in it."""
+        ahead = self._can_run_ahead()
+        if not ahead:
+            self._read_unread()
         output = self.scheduler.schedule()
         self.last_output = output
         self.num_steps += 1
         if not output.portions:
+            self._read_unread()
             return self.scheduler.drain_finished()
-        entries = [StepEntry(p.request.request_id, p.tokens, [len(p.tokens) - 1] if p.samples else [])
+        entries = [StepEntry(p.request.request_id, [max(t, 0) for t in p.tokens], [len(p.tokens) - 1] if p.samples else [])
                    for p in output.portions]
-        logits = self.runner.step(entries)
+        if ahead:
+            assert [p.request for p in output.portions] == [p.request for p in self._unread.portions]
+            logits = self.runner.step(entries, device_tokens=self._unread.tokens.device)
+            self.steps_run_ahead += 1
+        else:
+            logits = self.runner.step(entries)
         sampled = [p for p in output.portions if p.samples]
         for portion in output.portions:
             portion.request.num_computed += len(portion.tokens)
         if sampled:
-            tokens = self.sampler.sample(
+            draw = self.sampler.sample_async if self.run_ahead else self.sampler.sample
+            tokens = draw(
                 logits,
                 [p.request.sampling_params for p in sampled],
                 token_histories=[p.request.all_tokens for p in sampled],
                 seeds=[p.request.seed for p in sampled],
                 counters=[len(p.request.output_tokens) for p in sampled],
             )
-            for portion, token in zip(sampled, tokens):
-                portion.request.output_tokens.append(int(token))
-                self._check_finished(portion.request, int(token))
+            if self.run_ahead:
+                older, self._unread = self._unread, None
+                places = []
+                for portion in sampled:
+                    places.append(len(portion.request.output_tokens))
+                    portion.request.output_tokens.append(UNREAD)
+                newest = _UnreadStep(sampled, places, tokens)
+                self._unread = older
+                self._read_unread()              # the step before, while this one runs
+                self._unread = newest
+            else:
+                for portion, token in zip(sampled, tokens):
+                    portion.request.output_tokens.append(int(token))
+                    self._check_finished(portion.request, int(token))
+        elif ahead:
+            self._read_unread()
         return self.scheduler.drain_finished()
 
     def run(self, requests: deque[tuple[int, Request]] | None = None) -> list[Request]:
@@ -75,4 +146,6 @@ class Engine:
                 self.add_request(requests.popleft()[1])
             finished.extend(self.step())
             step += 1
+        self._read_unread()
+        finished.extend(self.scheduler.drain_finished())
         return finished

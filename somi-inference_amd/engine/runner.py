@@ -34,6 +34,8 @@ class _DecodeGraph:
 
 
 class ModelRunner:
+    accepts_device_tokens = True      # step() may take its tokens from a device tensor the host has not read
+
     def __init__(self, model: DecoderModel, cache: CacheManager, *, decode_graphs: bool = True) -> None:
         self.model = model
         self.cache = cache
@@ -55,7 +57,7 @@ class ModelRunner:
         self.cache.free(request_id)
 
     # -------------------------------------------------------------------- step
-    def _validate(self, entries: list[StepEntry]) -> None:
+    def _validate(self, entries: list[StepEntry], device_tokens: torch.Tensor | None = None) -> None:
         if not entries:
             raise StepError("a step needs at least one entry")
         seen = set()
@@ -70,28 +72,41 @@ class ModelRunner:
             for token in entry.tokens:
                 # the reference's embedding lookup raises on out-of-range ids
                 # (tests/models/test_qwen2_error_handling.py:42-86)
-                if not 0 <= int(token) < self.vocab_size:
+                if device_tokens is None and not 0 <= int(token) < self.vocab_size:
                     raise StepError(f"request {entry.request_id!r}: token id {token} is outside [0, {self.vocab_size})")
             for w in entry.want:
                 if not 0 <= int(w) < len(entry.tokens):
                     raise StepError(f"request {entry.request_id!r}: wanted place {w} is outside its {len(entry.tokens)} tokens")
+        if device_tokens is not None:
+            if any(len(entry.tokens) != 1 for entry in entries):
+                raise StepError("tokens that are still on the device stand for entries of one token each")
+            if (device_tokens.dtype != torch.int32 or device_tokens.device != self.device
+                    or tuple(device_tokens.shape) != (len(entries),)):
+                raise StepError(f"device tokens must be {len(entries)} int32 values on {self.device}")
 
-    def step(self, entries: list[StepEntry]) -> torch.Tensor:
+    def step(self, entries: list[StepEntry], device_tokens: torch.Tensor | None = None) -> torch.Tensor:
         """Run the entries as one batch; float32 logits ``[sum(len(want)), vocab]`` in entry order.
 
         Raises :class:`OutOfPages` before anything changes if the pages for
         all entries are not free.
+
+        ``device_tokens``: the entries' (single) tokens as an int32 tensor that is still on the device,
+        typically what the sampler drew from the previous step's logits and the host has not read yet;
+        the ids in ``entries`` are then placeholders.  The step is laid out and launched without waiting
+        for the device, so the host works on step n + 1 while the device runs step n.
         """
-        self._validate(entries)
+        self._validate(entries, device_tokens)
         portions = [(e.request_id, len(e.tokens)) for e in entries]
         if not self.cache.can_reserve(portions):
             raise OutOfPages(f"the step needs more pages than are free ({self.cache.free_pages()} free)")
         for request_id, count in portions:
             self.cache.reserve(request_id, count)
         if self.decode_graphs and all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries):
-            logits = self._decode_with_graph(entries)
+            logits = self._decode_with_graph(entries, device_tokens)
         else:
             batch = build_step(entries, self.cache, self.device)
+            if device_tokens is not None:
+                batch.token_ids.copy_(device_tokens)
             logits = self.model.forward(batch, self.cache.layer_caches)
         for request_id, count in portions:
             self.cache.commit(request_id, count)
@@ -121,7 +136,7 @@ class ModelRunner:
         return rows
 
     # ------------------------------------------------------------- HIP graphs
-    def _decode_with_graph(self, entries: list[StepEntry]) -> torch.Tensor:
+    def _decode_with_graph(self, entries: list[StepEntry], device_tokens: torch.Tensor | None = None) -> torch.Tensor:
         """Replay (or first capture) the graph for this many single-token entries.
 
         The block tables of a captured step have a fixed width, the next power of two of pages that
@@ -139,6 +154,8 @@ class ModelRunner:
         held = self._graphs.get(key)
         if held is None:
             static = StaticStep(entries, self.cache, self.device, widths)
+            if device_tokens is not None:
+                static.batch.token_ids.copy_(device_tokens)
             # once outside a capture: lazy initialisation (library handles, first allocations) must
             # not happen while the stream is being recorded; the step's writes are simply redone
             self.model.forward(static.batch, self.cache.layer_caches)
@@ -149,6 +166,8 @@ class ModelRunner:
             held = self._graphs[key] = _DecodeGraph(static, graph, logits)
         else:
             held.static.update(entries, self.cache)
+            if device_tokens is not None:
+                held.static.batch.token_ids.copy_(device_tokens)      # on the stream, after the arrays' own copy
         held.graph.replay()
         self.graph_replays += 1
         return held.logits

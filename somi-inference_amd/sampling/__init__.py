@@ -2,6 +2,6 @@
 
 from .params import SamplingParams
 from .rng import uniform
-from .sampler import Sampler
+from .sampler import PendingTokens, Sampler
 
-__all__ = ["Sampler", "SamplingParams", "uniform"]
+__all__ = ["PendingTokens", "Sampler", "SamplingParams", "uniform"]

@@ -19,9 +19,30 @@ from .params import SamplingParams
 from .rng import uniform
 
 
+class PendingTokens:
+    """Sampled token ids that are on their way to the host: ``device`` can feed the next step at once,
+    ``tolist()`` waits for the copy (and only for it, not for work launched since)."""
+
+    def __init__(self, device: torch.Tensor, host: torch.Tensor, copied: torch.cuda.Event) -> None:
+        self.device, self._host, self._copied = device, host, copied
+
+    def tolist(self) -> list[int]:
+        self._copied.synchronize()
+        return self._host.tolist()
+
+
 class Sampler:
+    RING = 4      # host buffers per batch size: a result must be read before that many later ones are drawn
+
     def __init__(self) -> None:
         self._greedy_inputs: dict[tuple[int, torch.device], torch.Tensor] = {}
+        self._host_rings: dict[int, tuple[list[torch.Tensor], list[int]]] = {}
+
+    def _host_buffer(self, rows: int) -> torch.Tensor:
+        ring, turn = self._host_rings.setdefault(
+            rows, ([torch.empty(rows, dtype=torch.int32).pin_memory() for _ in range(self.RING)], [0]))
+        turn[0] = (turn[0] + 1) % self.RING
+        return ring[turn[0]]
 
     def _pick_inputs(self, plist: list[SamplingParams], seeds: list[int], counters: list[int],
                      device: torch.device) -> tuple[torch.Tensor, torch.Tensor]:
@@ -44,6 +65,14 @@ class Sampler:
         ``token_histories``: per row, the ids the repetition penalty looks at (sampler.py:80-102).
         ``seeds`` / ``counters``: per row, the request's seed and how many tokens it has drawn.
         """
+        if logits.dim() == 2 and logits.shape[0] == 0:
+            return []
+        return self.sample_async(logits, params, token_histories, seeds, counters).tolist()
+
+    def sample_async(self, logits: torch.Tensor, params: SamplingParams | list[SamplingParams],
+                     token_histories: list[list[int]] | None = None,
+                     seeds: list[int] | None = None, counters: list[int] | None = None) -> PendingTokens:
+        """The same, without waiting: the ids stay on the device and their copy to the host is under way."""
         if logits.dim() != 2:
             raise ValueError(f"logits must be 2D, got shape {tuple(logits.shape)}")
         rows, vocab = logits.shape
@@ -56,7 +85,7 @@ class Sampler:
         seeds = seeds if seeds is not None else [0] * rows
         counters = counters if counters is not None else [0] * rows
         if rows == 0:
-            return []
+            raise ValueError("nothing to sample")
 
         needs_copy = any(p.repetition_penalty != 1.0 and h for p, h in zip(plist, histories)) or any(
             p.temperature > 0.0 and (p.top_k != -1 or p.top_p != 1.0) for p in plist)
@@ -86,4 +115,9 @@ class Sampler:
                 work[row, order[remove]] = float("-inf")
 
         temperature, draws = self._pick_inputs(plist, seeds, counters, work.device)
-        return ops.sample(work, temperature, draws).tolist()
+        picked = ops.sample(work, temperature, draws)
+        host = self._host_buffer(rows)
+        host.copy_(picked, non_blocking=True)
+        copied = torch.cuda.Event()
+        copied.record()
+        return PendingTokens(picked, host, copied)

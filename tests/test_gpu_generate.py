@@ -169,3 +169,36 @@ def test_warm_up_tunes_library_products_without_changing_results(model_folders, 
     assert_greedy_matches(got, want, prompts, cfg, weights, exact=False)
     assert list(tmp_path.iterdir()) == []
     assert LLM(folder, dtype="float32", num_blocks=64, block_size=8).warm_up() == 0
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_running_ahead_of_the_device_gives_the_same_tokens(dtype, model_folders):
+    """While only decoding requests run, the engine launches step n + 1 before it has read step n's tokens.
+    With it switched off the same tokens come out: greedy and with temperature, with requests of different
+    lengths (so that some end while others go on) and with an end-of-sequence token that really occurs (so
+    that a request has run one token too far when the host finds out)."""
+    vocab = TINY["B"]["config"].vocab_size
+    prompts = [token_ids(vocab, n, 40 + n) for n in (3, 18, 33, 7)]
+
+    def run(ahead, **options):
+        llm = LLM(model_folders["B"], dtype=dtype, block_size=8, num_blocks=64, max_concurrent=4, **options)
+        llm.engine.run_ahead = ahead
+        out = [llm.generate(prompts, max_new_tokens=24, temperature=0.0),
+               llm.generate(prompts, max_new_tokens=24, temperature=0.9, top_k=20, seed=11),
+               llm.generate(prompts[:2], max_new_tokens=5, temperature=0.0) + llm.generate(prompts[2:], max_new_tokens=9, temperature=0.0)]
+        assert llm.kv_manager.free_pages() == [64]
+        llm.kv_manager.check_invariants()
+        return out, llm.engine.steps_run_ahead
+
+    want, none_ahead = run(False, eos_token_id=-1)
+    got, some_ahead = run(True, eos_token_id=-1)
+    assert none_ahead == 0 and some_ahead > 40
+    assert got == want
+    assert all(len(tokens) == 24 and min(tokens) >= 0 for tokens in got[0])
+    # an end-of-sequence token that occurs in the middle of the first request's greedy tokens
+    eos = want[0][0][10]
+    want_eos, _ = run(False, eos_token_id=eos)
+    got_eos, ahead_eos = run(True, eos_token_id=eos)
+    assert got_eos == want_eos and ahead_eos > 0
+    first = want_eos[0][0]
+    assert first[-1] == eos and len(first) <= 11 and eos not in first[:-1]

@@ -277,3 +277,42 @@ def test_one_layer_of_the_7b_sizes_under_all_cuttings(dtype, real_size_folder):
         entries = [StepEntry(rid, [tokens[len(p) + step]], [0]) for rid, p in prompts.items()]
         got = runner.step(entries).cpu()
         check(got, [len(p) + step for p in prompts.values()], f"7B layer sizes {dtype}: batched decode step {step}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_decoding_from_tokens_that_are_still_on_the_device(dtype, model_folders):
+    """A decode step may take its tokens from the sampler's device tensor before the host has read them (the
+    host then works one step ahead of the device): the same tokens come out as when every step waits."""
+    from somi_inference_amd.sampling import Sampler, SamplingParams
+    name = "B"
+    vocab = TINY[name]["config"].vocab_size
+    prompts = {"a": token_ids(vocab, 21, 1), "b": token_ids(vocab, 9, 2), "c": token_ids(vocab, 40, 3)}
+    sampler, greedy = Sampler(), SamplingParams(temperature=0.0)
+
+    def start(engine):
+        first = []
+        for rid, prompt in prompts.items():
+            engine.begin(rid)
+            first.append(sampler.sample(engine.step([StepEntry(rid, prompt, [len(prompt) - 1])]), greedy)[0])
+        return first
+
+    waiting, _ = make_engine(model_folders[name], dtype, block_size=8, num_blocks=40)
+    tokens, want = start(waiting), []
+    for _ in range(20):
+        tokens = sampler.sample(waiting.step([StepEntry(rid, [t], [0]) for rid, t in zip(prompts, tokens)]), greedy)
+        want.append(tokens)
+
+    ahead, _ = make_engine(model_folders[name], dtype, block_size=8, num_blocks=40)
+    tokens, got = start(ahead), []
+    placeholders = [StepEntry(rid, [0], [0]) for rid in prompts]
+    newest = sampler.sample_async(ahead.step([StepEntry(rid, [t], [0]) for rid, t in zip(prompts, tokens)]), greedy)
+    for _ in range(19):
+        older, newest = newest, sampler.sample_async(ahead.step(placeholders, device_tokens=newest.device), greedy)
+        got.append(older.tolist())
+    got.append(newest.tolist())
+    assert got == want
+    assert ahead.graph_replays > 0
+    with pytest.raises(StepError, match="one token each"):
+        ahead.step([StepEntry("a", [1, 2], [1])], device_tokens=newest.device[:1])
+    with pytest.raises(StepError, match="int32"):
+        ahead.step(placeholders, device_tokens=newest.device[:2])

@@ -12,6 +12,7 @@ import torch
 
 from somi_inference_amd.cache import CacheManager
 from somi_inference_amd.engine import Engine, Request, RequestStatus, Scheduler, SchedulerError
+from somi_inference_amd.engine.engine import UNREAD
 from somi_inference_amd.parts import PagedKVSpec
 from somi_inference_amd.sampling import SamplingParams
 
@@ -203,3 +204,84 @@ def test_bad_requests_are_refused():
     for bad in (dict(temperature=-1.0), dict(top_k=0), dict(top_p=0.0), dict(top_p=1.5), dict(repetition_penalty=0.0)):
         with pytest.raises(ValueError):                           # reference: sampler.py:20-25
             SamplingParams(**bad)
+
+
+class LateTokens:
+    """Stands in for tokens that are still on the device: they may be handed on, but reading them is counted."""
+
+    def __init__(self, values, log):
+        self.device, self._log = list(values), log
+
+    def tolist(self):
+        self._log.append("read")
+        return list(self.device)
+
+
+class AheadRunner(ScriptedRunner):
+    accepts_device_tokens = True
+
+    def step(self, entries, device_tokens=None):
+        if device_tokens is not None:
+            assert all(e.tokens == [0] for e in entries) and len(device_tokens) == len(entries)
+            for e, token in zip(entries, device_tokens):
+                e.tokens = [token]
+            self.log.append("launch ahead")
+        else:
+            self.log.append("launch")
+        return super().step(entries)
+
+
+class AheadSampler(ScriptedSampler):
+    def sample_async(self, logits, params, token_histories=None, seeds=None, counters=None):
+        return LateTokens(self.sample(logits, params, token_histories, seeds, counters), self.log)
+
+
+def ahead_engine(cache, scripts, *, ahead, eos=None, max_concurrent=4):
+    scheduler = Scheduler(cache, max_concurrent=max_concurrent, max_num_batched_tokens=64)
+    runner, sampler = AheadRunner(cache), AheadSampler(scripts)
+    runner.log = sampler.log = []
+    engine = Engine(runner, scheduler, sampler, eos)
+    assert engine.run_ahead
+    engine.run_ahead = ahead
+    return engine, runner
+
+
+@pytest.mark.parametrize("eos", [None, 33])
+def test_running_ahead_launches_the_next_step_before_reading_and_changes_no_token(eos):
+    """Two decoding requests of different lengths and a late arrival.  Running ahead, a decode step is
+    launched before the tokens of the step before are read; it falls back to reading first whenever a
+    request is at its last token, one is waiting or one has ended.  The model sees the same tokens at the
+    same places as without it, except that a request that ends on EOS has run one token too far."""
+    scripts = {0: [30, 31, 32, 33, 34, 35, 36], 1: [40, 41, 42, 43], 2: [50, 51, 52]}
+
+    def run(ahead):
+        cache = make_cache(num_blocks=16)
+        engine, runner = ahead_engine(cache, scripts, ahead=ahead, eos=eos)
+        arrivals = deque([(0, request(0, 5, 7)), (0, request(1, 3, 4)), (4, request(2, 6, 3))])
+        done = engine.run(arrivals)
+        assert cache.free_pages() == [16] and not cache.live_requests()
+        return {r.request_id: (r.output_tokens, r.finish_reason) for r in done}, runner, engine
+
+    want, plain_runner, plain = run(False)
+    got, runner, engine = run(True)
+    assert got == want and plain.steps_run_ahead == 0 and engine.steps_run_ahead >= 2
+    assert all(UNREAD not in tokens for tokens, _ in got.values())
+    if eos is None:
+        assert runner.calls == plain_runner.calls
+        assert got[0] == ([30, 31, 32, 33, 34, 35, 36], "length")
+    else:
+        assert got[0] == ([30, 31, 32, 33], "eos")
+        # the model was given every token it is given without running ahead, at the same place
+        given = {(rid, tuple(tokens)) for call in runner.calls for rid, tokens, _ in call}
+        assert {(rid, tuple(tokens)) for call in plain_runner.calls for rid, tokens, _ in call} <= given
+    log = runner.log
+    first = log.index("launch ahead")
+    assert log[first - 1] != "read" and log[first + 1] == "read"      # launched first, the older step read after
+
+
+def test_running_ahead_is_left_alone_when_a_sampling_rule_reads_the_history():
+    cache = make_cache(num_blocks=16)
+    engine, runner = ahead_engine(cache, {0: [30, 31, 32, 33]}, ahead=True)
+    done = engine.run(deque([(0, request(0, 5, 4, sampling_params=SamplingParams(repetition_penalty=1.3)))]))
+    assert done[0].output_tokens == [30, 31, 32, 33] and engine.steps_run_ahead == 0
+    assert "launch ahead" not in runner.log
