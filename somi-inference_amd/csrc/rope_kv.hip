@@ -12,44 +12,64 @@
 // positions of one channel with one load (the operand layout of the matrix cores for P.V).
 #include "common.h"
 
+#define ROPE_THREADS 256
+#define ROPE_MAX_HALF 256                      // rotary_dim / 2 at most
+
+// One workgroup per (token, group of heads): cos and sin of the token's angles are computed once into LDS
+// and serve every head of the group; the group's (head, channel pair) items are dealt to the threads.
 template <typename T>
-__global__ void __launch_bounds__(64)
+__global__ void __launch_bounds__(ROPE_THREADS)
 rope_kv_store_kernel(T* __restrict__ qkv, int64_t row_stride, const int* __restrict__ positions,
                      const int* __restrict__ slots, const float* __restrict__ inv_freq, int rot_half,
-                     int nq, int nkv, int D, T* __restrict__ kc, T* __restrict__ vc, int page_size) {
-    const int t = blockIdx.x;
-    const int hh = blockIdx.y;                 // 0..nq-1: q heads, then nkv k heads, then nkv v heads
-    T* src = qkv + (int64_t)t * row_stride + (int64_t)hh * D;
-    const float pos = (float)positions[t];
-
-    T* dst = nullptr;                          // cache row, when this head is a k or v head
-    if (hh >= nq) {
-        const int slot = slots[t];
-        if (slot < 0) return;                  // a token without a cache slot (padding)
-        const bool is_v = hh >= nq + nkv;
-        const int kvh = hh - nq - (is_v ? nkv : 0);
-        const int64_t page = slot / page_size, off = slot % page_size;
-        if (is_v) {
-            T* col = vc + (page * nkv + kvh) * (int64_t)D * page_size + off;
-            for (int d = threadIdx.x; d < D; d += 64) col[(int64_t)d * page_size] = src[d];
-            return;
-        }
-        dst = kc + ((page * nkv + kvh) * page_size + off) * D;
-    }
-    T* q_or_k = dst ? dst : src;               // q is rotated in place, k goes to its page
-    for (int j = threadIdx.x; j < rot_half; j += 64) {
-        const float x1 = to_float(src[j]), x2 = to_float(src[j + rot_half]);
-        float c = 1.f, s = 0.f;
-        if (inv_freq) {
+                     int nq, int nkv, int D, T* __restrict__ kc, T* __restrict__ vc, int page_size,
+                     int heads_per_block) {
+    __shared__ float cs[2][ROPE_MAX_HALF];
+    const int t = blockIdx.x, tid = threadIdx.x;
+    const int h0 = blockIdx.y * heads_per_block;               // heads 0..nq-1: q, then nkv k heads, then nkv v heads
+    const int h1 = min(h0 + heads_per_block, nq + 2 * nkv);
+    T* row = qkv + (int64_t)t * row_stride;
+    if (inv_freq) {
+        const float pos = (float)positions[t];
+        for (int j = tid; j < rot_half; j += ROPE_THREADS) {
             const float angle = pos * inv_freq[j];
-            c = cosf(angle);
-            s = sinf(angle);
+            cs[0][j] = cosf(angle);
+            cs[1][j] = sinf(angle);
         }
-        q_or_k[j] = from_float<T>(x1 * c - x2 * s);
-        q_or_k[j + rot_half] = from_float<T>(x2 * c + x1 * s);
     }
-    if (dst)                                   // pass-through tail of a partly rotated head
-        for (int d = 2 * rot_half + threadIdx.x; d < D; d += 64) dst[d] = src[d];
+    __syncthreads();
+    const int slot = nkv > 0 ? slots[t] : -1;                  // -1: a token without a cache slot (padding)
+    const int64_t page = slot >= 0 ? slot / page_size : 0, off = slot >= 0 ? slot % page_size : 0;
+
+    // q (in place) and k (into its page): rotate the pairs (j, j + rot_half)
+    const int rot0 = h0, rot1 = min(h1, nq + nkv);
+    if (rot_half > 0)
+        for (int item = tid; item < (rot1 - rot0) * rot_half; item += ROPE_THREADS) {
+            const int hh = rot0 + item / rot_half, j = item % rot_half;
+            const T* src = row + (int64_t)hh * D;
+            T* dst = row + (int64_t)hh * D;
+            if (hh >= nq) {
+                if (slot < 0) continue;
+                dst = kc + ((page * nkv + (hh - nq)) * page_size + off) * D;
+            }
+            const float x1 = to_float(src[j]), x2 = to_float(src[j + rot_half]);
+            const float c = cs[0][j], sn = cs[1][j];
+            dst[j] = from_float<T>(x1 * c - x2 * sn);
+            dst[j + rot_half] = from_float<T>(x2 * c + x1 * sn);
+        }
+    // k: the channels past the rotated ones go to the page as they are
+    const int k0 = max(h0, nq), k1 = min(h1, nq + nkv), rest = D - 2 * rot_half;
+    if (slot >= 0 && rest > 0)
+        for (int item = tid; item < (k1 - k0) * rest; item += ROPE_THREADS) {
+            const int hh = k0 + item / rest, d = 2 * rot_half + item % rest;
+            kc[((page * nkv + (hh - nq)) * page_size + off) * D + d] = row[(int64_t)hh * D + d];
+        }
+    // v: into its page, transposed
+    const int v0 = max(h0, nq + nkv), v1 = h1;
+    if (slot >= 0)
+        for (int item = tid; item < (v1 - v0) * D; item += ROPE_THREADS) {
+            const int hh = v0 + item / D, d = item % D;
+            vc[((page * nkv + (hh - nq - nkv)) * (int64_t)D + d) * page_size + off] = row[(int64_t)hh * D + d];
+        }
 }
 
 // qkv: [n_tokens, row_stride] with q heads, k heads, v heads side by side (row_stride >= (nq+2nkv)*D).
@@ -66,17 +86,22 @@ extern "C" int somi_rope_kv_store(void* qkv, int dtype, int64_t row_stride, cons
     SOMI_REQUIRE(nkv == 0 || (k_cache && v_cache && slots && page_size > 0),
                  "rope_kv_store: cache pointers, slots and page size are needed when k/v heads are given");
     SOMI_REQUIRE(nq + 2 * nkv <= 65535, "rope_kv_store: too many heads");
+    SOMI_REQUIRE(rotary_dim / 2 <= ROPE_MAX_HALF, "rope_kv_store: rotary_dim %d is more than %d", rotary_dim,
+                 2 * ROPE_MAX_HALF);
     if (n_tokens == 0 || nq + 2 * nkv == 0) return 0;
-    const dim3 grid(n_tokens, nq + 2 * nkv);
+    // about two thousand workgroups: one head each for a few tokens, all heads of a token for long portions
+    const int heads = nq + 2 * nkv;
+    const int heads_per_block = max(1, min(heads, (int)(((int64_t)n_tokens * heads + 2047) / 2048)));
+    const dim3 grid(n_tokens, ceil_div(heads, heads_per_block));
     const int rot_half = inv_freq ? rotary_dim / 2 : 0;
     if (dtype == SOMI_F32)
-        hipLaunchKernelGGL(rope_kv_store_kernel<float>, grid, dim3(64), 0, stream, (float*)qkv, row_stride,
+        hipLaunchKernelGGL(rope_kv_store_kernel<float>, grid, dim3(ROPE_THREADS), 0, stream, (float*)qkv, row_stride,
                            positions, slots, inv_freq, rot_half, nq, nkv, D, (float*)k_cache, (float*)v_cache,
-                           page_size);
+                           page_size, heads_per_block);
     else if (dtype == SOMI_BF16)
-        hipLaunchKernelGGL(rope_kv_store_kernel<bf16>, grid, dim3(64), 0, stream, (bf16*)qkv, row_stride,
+        hipLaunchKernelGGL(rope_kv_store_kernel<bf16>, grid, dim3(ROPE_THREADS), 0, stream, (bf16*)qkv, row_stride,
                            positions, slots, inv_freq, rot_half, nq, nkv, D, (bf16*)k_cache, (bf16*)v_cache,
-                           page_size);
+                           page_size, heads_per_block);
     else
         return somi_fail("rope_kv_store: unknown dtype %d", dtype);
     SOMI_LAUNCH_CHECK("rope_kv_store");
