@@ -28,6 +28,14 @@ HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E bandwidth
 PEAK_FLOPS = {"bfloat16": 2.5e15, "float32": 157.3e12}   # dense MFMA peaks
 
 
+# layer sizes of the Qwen2.5 family: (layers, hidden, heads, kv heads, head_dim, intermediate, rms_norm_eps)
+LAYER_SIZES = {
+    "7b": (28, 3584, 28, 4, 128, 18944, 1e-6),
+    "14b": (48, 5120, 40, 8, 128, 13824, 1e-5),
+    "32b": (64, 5120, 40, 8, 128, 27648, 1e-6),
+}
+
+
 def parse_args() -> argparse.Namespace:
     p = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     p.add_argument("--gpus", type=int, default=1)
@@ -35,6 +43,8 @@ def parse_args() -> argparse.Namespace:
     p.add_argument("--warmup", type=int, default=8)
     p.add_argument("--batch", type=int, default=8)
     p.add_argument("--context", type=int, default=4096, help="context length the timed decode steps end at")
+    p.add_argument("--sizes", default="7b", choices=sorted(LAYER_SIZES),
+                   help="layer sizes: Qwen2.5-7B (the default and the headline), -14B or -32B")
     p.add_argument("--layers", type=int, default=None, help="run fewer layers than the configuration has")
     p.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     p.add_argument("--block-size", type=int, default=16)
@@ -62,11 +72,12 @@ def main() -> int:
     from somi_inference_amd.models import make_runner, random_model
     from somi_inference_amd.sampling import Sampler, SamplingParams
 
-    full_layers = 28
+    full_layers, hidden, heads, kv_heads, head_dim, intermediate, eps = LAYER_SIZES[args.sizes]
     layers = args.layers or full_layers
-    config = Qwen2Config(vocab_size=152064, hidden_size=3584, intermediate_size=18944, num_hidden_layers=layers,
-                         num_attention_heads=28, num_key_value_heads=4, head_dim=128, rope_theta=1e6,
-                         rms_norm_eps=1e-6, tie_word_embeddings=False, max_position_embeddings=32768)
+    config = Qwen2Config(vocab_size=152064, hidden_size=hidden, intermediate_size=intermediate,
+                         num_hidden_layers=layers, num_attention_heads=heads, num_key_value_heads=kv_heads,
+                         head_dim=head_dim, rope_theta=1e6, rms_norm_eps=eps, tie_word_embeddings=False,
+                         max_position_embeddings=32768)
     torch.manual_seed(args.seed)
     model = random_model(config, seed=args.seed, dtype=args.dtype)
     elem = 2 if args.dtype == "bfloat16" else 4
@@ -154,13 +165,14 @@ def main() -> int:
                    "ms": round(seconds * 1000.0, 3), "frac": round(flops / seconds / PEAK_FLOPS[args.dtype], 4)}
 
     line = {
-        "metric": "decode tok/s at batch 8, Qwen2.5-7B layer sizes (plus prefill tok/s at 2,048 tokens, batch 1/64 points)",
+        "metric": f"decode tok/s at batch {args.batch}, Qwen2.5-{args.sizes.upper()} layer sizes "
+                  f"(plus prefill tok/s at {args.prefill_tokens:,} tokens, batch 1/64 points)",
         "value": round(main_run["tok_s"], 2), "unit": "tokens/s", "n_gpus": 1,
         "steps": main_run["steps"], "warmup": main_run["warmup"], "ms_per_step": round(main_run["ms"], 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
         "data": "synthetic: seeded random N(0,0.02) weights, seeded uniform token ids; caches filled by running the prompts",
-        "config": {"model": "Qwen2.5-7B layer sizes (random weights)", "global_batch": args.batch,
+        "config": {"model": f"Qwen2.5-{args.sizes.upper()} layer sizes (random weights)", "global_batch": args.batch,
                    "seq_len": args.context, "parallelism": "single GPU", "layers": layers,
                    "layers_of_config": full_layers, "hidden_size": config.hidden_size,
                    "intermediate_size": config.intermediate_size, "num_attention_heads": config.num_attention_heads,
