@@ -52,6 +52,9 @@ def parse_args() -> argparse.Namespace:
     p.add_argument("--seed", type=int, default=0)
     p.add_argument("--no-points", action="store_true", help="skip the batch 1 / batch 64 decode points")
     p.add_argument("--no-prefill", action="store_true", help="skip the prefill measurement")
+    p.add_argument("--serving", type=int, default=0, metavar="REQUESTS",
+                   help="also run this many requests (prompts of 128 to 2,048 tokens, 256 new tokens each) through "
+                        "the scheduler with portions of 512, and report it under 'serving'")
     p.add_argument("--no-tune", action="store_true",
                    help="leave the library's matrix products of the prompt portions at its own heuristic")
     return p.parse_args()
@@ -164,6 +167,36 @@ def main() -> int:
         prefill = {"value": round(args.prefill_tokens / seconds, 1), "tokens": args.prefill_tokens,
                    "ms": round(seconds * 1000.0, 3), "frac": round(flops / seconds / PEAK_FLOPS[args.dtype], 4)}
 
+    serving = None
+    if args.serving > 0:
+        # continuous batching through the engine's own scheduler: everything arrives at once, prompts are cut
+        # into portions of 512 under a budget of 2,048 tokens a step, finished requests free their pages
+        from collections import deque
+
+        from somi_inference_amd.engine import Engine, Request, Scheduler
+        lengths = torch.randint(128, 2049, (args.serving,), generator=gen).tolist()
+        new_tokens = 256
+        # the pool made for the decode runs serves here too; at most as many requests at once as fit whole
+        per_request = (2048 + new_tokens + args.block_size - 1) // args.block_size + 1
+        concurrent = max(1, min(args.serving, max(batches), num_blocks // per_request))
+        scheduler = Scheduler(runner.cache, max_concurrent=concurrent, max_num_batched_tokens=2048, chunk=512)
+        engine = Engine(runner, scheduler, sampler, eos_token_id=-1)
+        arrivals = deque((0, Request(f"s{i}", torch.randint(0, config.vocab_size, (n,), generator=gen).tolist(),
+                                     new_tokens, greedy, seed=i)) for i, n in enumerate(lengths))
+        if tuned:
+            runner.tune_library_products(512)
+        sync()
+        start = time.perf_counter()
+        done = engine.run(arrivals)
+        sync()
+        seconds = time.perf_counter() - start
+        generated = sum(len(r.output_tokens) for r in done)
+        serving = {"requests": len(done), "prompt_tokens": sum(lengths), "generated_tokens": generated,
+                   "seconds": round(seconds, 3), "generated_tok_s": round(generated / seconds, 1),
+                   "total_tok_s": round((generated + sum(lengths)) / seconds, 1), "steps": engine.num_steps,
+                   "steps_run_ahead": engine.steps_run_ahead, "max_concurrent": concurrent,
+                   "preemptions": sum(r.num_preemptions for r in done)}
+
     line = {
         "metric": f"decode tok/s at batch {args.batch}, Qwen2.5-{args.sizes.upper()} layer sizes "
                   f"(plus prefill tok/s at {args.prefill_tokens:,} tokens, batch 1/64 points)",
@@ -185,6 +218,8 @@ def main() -> int:
     }
     if prefill is not None:
         line["prefill"] = prefill
+    if serving is not None:
+        line["serving"] = serving
     print(json.dumps(line))
     return 0
 
