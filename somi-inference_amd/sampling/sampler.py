@@ -36,11 +36,12 @@ class Sampler:
 
     def __init__(self) -> None:
         self._greedy_inputs: dict[tuple[int, torch.device], torch.Tensor] = {}
-        self._host_rings: dict[int, tuple[list[torch.Tensor], list[int]]] = {}
+        self._host_rings: dict[tuple[int, torch.dtype], tuple[list[torch.Tensor], list[int]]] = {}
 
-    def _host_buffer(self, rows: int) -> torch.Tensor:
+    def _host_buffer(self, size: int, dtype: torch.dtype) -> torch.Tensor:
+        """Pinned host memory, a few buffers per size in turn: copies to and from it do not wait for the device."""
         ring, turn = self._host_rings.setdefault(
-            rows, ([torch.empty(rows, dtype=torch.int32).pin_memory() for _ in range(self.RING)], [0]))
+            (size, dtype), ([torch.empty(size, dtype=dtype).pin_memory() for _ in range(self.RING)], [0]))
         turn[0] = (turn[0] + 1) % self.RING
         return ring[turn[0]]
 
@@ -53,8 +54,10 @@ class Sampler:
             if held is None:
                 held = self._greedy_inputs[(rows, device)] = torch.zeros(2 * rows, dtype=torch.float32, device=device)
         else:
-            held = torch.tensor([p.temperature for p in plist] + [uniform(s, c) for s, c in zip(seeds, counters)],
-                                dtype=torch.float32).to(device)
+            staged = self._host_buffer(2 * rows, torch.float32)
+            staged.copy_(torch.tensor([p.temperature for p in plist] + [uniform(s, c) for s, c in zip(seeds, counters)],
+                                      dtype=torch.float32))
+            held = staged.to(device, non_blocking=True)
         return held[:rows], held[rows:]
 
     def sample(self, logits: torch.Tensor, params: SamplingParams | list[SamplingParams],
@@ -116,7 +119,7 @@ class Sampler:
 
         temperature, draws = self._pick_inputs(plist, seeds, counters, work.device)
         picked = ops.sample(work, temperature, draws)
-        host = self._host_buffer(rows)
+        host = self._host_buffer(rows, torch.int32)
         host.copy_(picked, non_blocking=True)
         copied = torch.cuda.Event()
         copied.record()
