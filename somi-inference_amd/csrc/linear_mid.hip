@@ -26,7 +26,6 @@ typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
 #define SOMI_BUFFER_WORD3 0x00020000u            // raw buffer, 32-bit elements, no swizzle
 #define SOMI_OUT_OF_RANGE 0x80000000u
 #define MID_WAVES 4
-#define MID_CK 64
 
 // D[row = (lane / 16) * 4 + i][col = lane % 16]: a lane holds four consecutive output columns of row
 // (lane % 16) of each 16-row tile of x, for each of its wavefront's strips.
@@ -63,13 +62,16 @@ __device__ __forceinline__ void mid_epilogue(const f32x4 (&acc)[NS][MT], const f
     }
 }
 
-template <int MT, int NS, typename TO, bool SWIGLU, bool TAIL>
+template <int MT, int NS, int CK, int DEPTH, typename TO, bool SWIGLU, bool TAIL>
 __global__ void __launch_bounds__(MID_WAVES * 64, 2)
 linear_mid_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, const float* __restrict__ bias,
                   TO* __restrict__ out, int M, int N, int K, int chunks_per_split, float* __restrict__ partial) {
-    constexpr int ROW_BYTES = MID_CK * 2;          // 128 bytes of a row in a chunk
-    constexpr int XL = (MT + 1) / 2;               // loads of x per thread: 256 threads fetch 32 rows at a time
-    constexpr int WLD = 2 * NS;                    // loads of w per thread: a wavefront fetches 8 rows at a time
+    constexpr int ROW_BYTES = CK * 2;              // bytes of a row in a chunk: 128 or 256
+    constexpr int LPR = ROW_BYTES / 16;            // lanes that read one row: 8 or 16
+    constexpr int WRPI = 64 / LPR;                 // rows a wavefront fetches with one load: 8 or 4
+    constexpr int XRPI = 256 / LPR;                // rows the workgroup fetches with one load: 32 or 16
+    constexpr int WLD = NS * 16 / WRPI;            // loads of w per thread and chunk
+    constexpr int XL = (MT * 16 + XRPI - 1) / XRPI;   // loads of x per thread and chunk
     constexpr int X_BYTES = MT * 16 * ROW_BYTES, W_BYTES = NS * 16 * ROW_BYTES;
     __shared__ __attribute__((aligned(16))) char xs[2][X_BYTES];
     __shared__ __attribute__((aligned(16))) char ws[MID_WAVES][W_BYTES];
@@ -85,29 +87,30 @@ linear_mid_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, const 
     const __amdgpu_buffer_rsrc_t xres = __builtin_amdgcn_make_buffer_rsrc(
         (void*)x, 0, (int)((int64_t)M * K * 2), SOMI_BUFFER_WORD3);
 
-    // w: lane l of a wavefront reads 16 bytes of row (l / 8) of each group of 8 rows; x: thread t reads
-    // 16 bytes of row (t / 8) of each group of 32 rows.  Both land in LDS rows of 128 bytes whose 16-byte
-    // pieces are XOR-swizzled with bits of the row number.
-    const int lchunk = lane & 7;
+    // w: LPR lanes of a wavefront read one row's bytes of the chunk, 16 each; x: the same with all 256
+    // threads.  Both land in LDS rows whose 16-byte pieces are XOR-swizzled with bits of the row number, so
+    // that neither these row-wise writes nor the column-wise operand reads collide.
+    const int lchunk = lane % LPR;
+    auto swizzle = [](int row16) { return CK == 128 ? (row16 & 15) : ((row16 & 7) ^ (row16 >> 3)); };
     unsigned wgoff[WLD];
     int wsoff[WLD];
 #pragma unroll
     for (int i = 0; i < WLD; ++i) {
-        const int row16 = (i & 1) * 8 + (lane >> 3), strip = i >> 1;
-        wgoff[i] = ((unsigned)((wave * NS + strip) * 16 + row16) * (unsigned)K + lchunk * 8) * 2u;
-        wsoff[i] = (strip * 16 + row16) * ROW_BYTES + ((lchunk ^ ((row16 & 7) ^ (row16 >> 3))) << 4);
+        const int row = i * WRPI + lane / LPR;     // row among the wavefront's NS * 16
+        wgoff[i] = ((unsigned)(wave * NS * 16 + row) * (unsigned)K + lchunk * 8) * 2u;
+        wsoff[i] = row * ROW_BYTES + ((lchunk ^ swizzle(row & 15)) << 4);
     }
     unsigned xgoff[XL];
     int xsoff[XL];
     bool xkeep[XL];
 #pragma unroll
     for (int j = 0; j < XL; ++j) {
-        const int row = j * 32 + (tid >> 3);
+        const int row = j * XRPI + tid / LPR;
         xgoff[j] = ((unsigned)row * (unsigned)K + lchunk * 8) * 2u;
-        xsoff[j] = row * ROW_BYTES + ((lchunk ^ ((row & 7) ^ ((row >> 3) & 1))) << 4);
+        xsoff[j] = row * ROW_BYTES + ((lchunk ^ swizzle(row & 15)) << 4);
         xkeep[j] = row < MT * 16;
     }
-    const int rswz = (r & 7) ^ (r >> 3);
+    const int rswz = swizzle(r);
 
     f32x4 acc[NS][MT];
 #pragma unroll
@@ -115,7 +118,7 @@ linear_mid_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, const 
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) acc[s][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    const int chunks = (K + MID_CK - 1) / MID_CK;
+    const int chunks = (K + CK - 1) / CK;
     const int first = split * chunks_per_split;
     const int count = max(0, min(chunks_per_split, chunks - first));       // the same for every wavefront
 
@@ -124,7 +127,7 @@ linear_mid_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, const 
         u32x4 xv[XL];
     };
     auto issue = [&](Stage& st, int at) {
-        const int k0 = (first + at) * MID_CK;
+        const int k0 = (first + at) * CK;
         const bool inside = !TAIL || k0 + lchunk * 8 < K;
 #pragma unroll
         for (int i = 0; i < WLD; ++i)
@@ -142,59 +145,65 @@ linear_mid_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, const 
         for (int j = 0; j < XL; ++j)
             if (xkeep[j]) *reinterpret_cast<u32x4*>(xs[buf] + xsoff[j]) = st.xv[j];
     };
-    // the k-values of the chunk are dealt to the two products as 16-byte pieces 2g and 2g + 1 of lane
+    // the k-values of a 64-wide block are dealt to the two products as 16-byte pieces 2g and 2g + 1 of lane
     // group g: any order serves as long as w and x use the same
     auto compute = [&](int buf) {
-        bf16x8 xa[MT], xb[MT];
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-            const char* row = xs[buf] + (mt * 16 + r) * ROW_BYTES;
-            xa[mt] = *reinterpret_cast<const bf16x8*>(row + (((2 * g) ^ rswz) << 4));
-            xb[mt] = *reinterpret_cast<const bf16x8*>(row + (((2 * g + 1) ^ rswz) << 4));
-        }
-#pragma unroll
-        for (int s = 0; s < NS; ++s) {
-            const char* row = ws[wave] + (s * 16 + r) * ROW_BYTES;
-            const bf16x8 wa = *reinterpret_cast<const bf16x8*>(row + (((2 * g) ^ rswz) << 4));
-            const bf16x8 wb = *reinterpret_cast<const bf16x8*>(row + (((2 * g + 1) ^ rswz) << 4));
+        for (int cb = 0; cb < CK / 64; ++cb) {
+            bf16x8 xa[MT], xb[MT];
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) {
-                acc[s][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa, xa[mt], acc[s][mt], 0, 0, 0);
-                acc[s][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wb, xb[mt], acc[s][mt], 0, 0, 0);
+                const char* row = xs[buf] + (mt * 16 + r) * ROW_BYTES;
+                xa[mt] = *reinterpret_cast<const bf16x8*>(row + (((cb * 8 + 2 * g) ^ rswz) << 4));
+                xb[mt] = *reinterpret_cast<const bf16x8*>(row + (((cb * 8 + 2 * g + 1) ^ rswz) << 4));
+            }
+#pragma unroll
+            for (int s = 0; s < NS; ++s) {
+                const char* row = ws[wave] + (s * 16 + r) * ROW_BYTES;
+                const bf16x8 wa = *reinterpret_cast<const bf16x8*>(row + (((cb * 8 + 2 * g) ^ rswz) << 4));
+                const bf16x8 wb = *reinterpret_cast<const bf16x8*>(row + (((cb * 8 + 2 * g + 1) ^ rswz) << 4));
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) {
+                    acc[s][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa, xa[mt], acc[s][mt], 0, 0, 0);
+                    acc[s][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wb, xb[mt], acc[s][mt], 0, 0, 0);
+                }
             }
         }
     };
-    // One barrier per chunk: chunk i goes to buffer i % 2; a wavefront that writes buffer i % 2 has
+    // One barrier per chunk: chunk i goes to x buffer i % 2; a wavefront that writes buffer i % 2 has
     // passed the barrier of chunk i - 1, so every wavefront is done reading chunk i - 2 from it.
-    auto step = [&](Stage& st, int buf, int refill) {
-        stash(st, buf);
-        if (refill >= 0) issue(st, refill);
+    // DEPTH chunks are in flight in registers: set d holds chunk `at + d`.  The loop is entered on one
+    // path only, with every set issued, so that the waits inside it count loads exactly.
+    Stage st[DEPTH];
+    int done = 0;                                    // chunks computed so far: the x buffer of the next one is done % 2
+    auto step = [&](Stage& stage, int refill) {
+        stash(stage, done & 1);
+        if (refill >= 0) issue(stage, refill);
         __syncthreads();
-        compute(buf);
+        compute(done & 1);
+        ++done;
     };
-
-    Stage A, B;
-    if (count >= 2) {
-        issue(A, 0);
-        issue(B, 1);
+    if (count >= DEPTH) {
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d) issue(st[d], d);
         int at = 0;
-        for (; at + 3 < count; at += 2) {            // entered on one path, so the waits count loads exactly
-            stash(A, 0);
-            issue(A, at + 2);
-            __syncthreads();
-            compute(0);
-            stash(B, 1);
-            issue(B, at + 3);
-            __syncthreads();
-            compute(1);
+        for (; at + 2 * DEPTH - 1 < count; at += DEPTH) {
+#pragma unroll
+            for (int d = 0; d < DEPTH; ++d) step(st[d], at + DEPTH + d);
         }
-        const bool third = at + 2 < count;           // two or three chunks are left
-        step(A, 0, third ? at + 2 : -1);
-        step(B, 1, -1);
-        if (third) step(A, 0, -1);
-    } else if (count == 1) {
-        issue(A, 0);
-        step(A, 0, -1);
+        // DEPTH to 2 * DEPTH - 1 chunks are left
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d) step(st[d], (d < DEPTH - 1 && at + DEPTH + d < count) ? at + DEPTH + d : -1);
+#pragma unroll
+        for (int d = 0; d < DEPTH - 1; ++d)
+            if (at + DEPTH + d < count) step(st[d], -1);
+    } else {
+#pragma unroll
+        for (int d = 0; d < DEPTH - 1; ++d)
+            if (d < count) issue(st[d], d);
+#pragma unroll
+        for (int d = 0; d < DEPTH - 1; ++d)
+            if (d < count) step(st[d], -1);
     }
 
     if (splits > 1) {
@@ -230,40 +239,45 @@ linear_mid_reduce_kernel(const float* __restrict__ partial, const float* __restr
     mid_epilogue<MT, NS, TO, SWIGLU>(acc, bias, out, M, N, tile * (64 * NS), wave, lane);
 }
 
-template <int MT, int NS, typename TO, bool SW, bool TL>
+template <int MT, int NS, int CK, int DEPTH, typename TO, bool SW, bool TL>
 static void mid_launch_kernel(const void* x, const void* w, const float* bias, void* out, int M, int N, int K,
                               int splits, int chunks_per_split, float* partial, hipStream_t stream) {
     const dim3 grid(ceil_div(N, 64 * NS), splits), block(MID_WAVES * 64);
-    hipLaunchKernelGGL((linear_mid_kernel<MT, NS, TO, SW, TL>), grid, block, 0, stream, (const bf16*)x,
+    hipLaunchKernelGGL((linear_mid_kernel<MT, NS, CK, DEPTH, TO, SW, TL>), grid, block, 0, stream, (const bf16*)x,
                        (const bf16*)w, bias, (TO*)out, M, N, K, chunks_per_split, partial);
     if (splits > 1)
         hipLaunchKernelGGL((linear_mid_reduce_kernel<MT, NS, TO, SW>), dim3(grid.x), block, 0, stream,
                            (const float*)partial, bias, (TO*)out, M, N, splits);
 }
 
-template <int MT, int NS, typename TO>
+template <int MT, int NS, int CK, int DEPTH, typename TO>
 static int mid_launch(const void* x, const void* w, const float* bias, void* out, int M, int N, int K, int splits,
-                      int chunks_per_split, bool swiglu, float* partial, hipStream_t stream) {
-    const bool tail = K % MID_CK != 0;
+                      bool swiglu, float* partial, hipStream_t stream) {
+    const bool tail = K % CK != 0;
+    const int chunks_per_split = ceil_div(ceil_div(K, CK), splits);
     if constexpr (NS >= 2) {
         if (swiglu) {
-            if (tail) mid_launch_kernel<MT, NS, TO, true, true>(x, w, bias, out, M, N, K, splits, chunks_per_split, partial, stream);
-            else mid_launch_kernel<MT, NS, TO, true, false>(x, w, bias, out, M, N, K, splits, chunks_per_split, partial, stream);
+            if (tail) mid_launch_kernel<MT, NS, CK, DEPTH, TO, true, true>(x, w, bias, out, M, N, K, splits, chunks_per_split, partial, stream);
+            else mid_launch_kernel<MT, NS, CK, DEPTH, TO, true, false>(x, w, bias, out, M, N, K, splits, chunks_per_split, partial, stream);
             SOMI_LAUNCH_CHECK("linear_mid");
             return 0;
         }
     }
-    if (tail) mid_launch_kernel<MT, NS, TO, false, true>(x, w, bias, out, M, N, K, splits, chunks_per_split, partial, stream);
-    else mid_launch_kernel<MT, NS, TO, false, false>(x, w, bias, out, M, N, K, splits, chunks_per_split, partial, stream);
+    if (tail) mid_launch_kernel<MT, NS, CK, DEPTH, TO, false, true>(x, w, bias, out, M, N, K, splits, chunks_per_split, partial, stream);
+    else mid_launch_kernel<MT, NS, CK, DEPTH, TO, false, false>(x, w, bias, out, M, N, K, splits, chunks_per_split, partial, stream);
     SOMI_LAUNCH_CHECK("linear_mid");
     return 0;
 }
 
+#ifndef SOMI_MID_NO_ENTRY_POINTS
+#define MID_CK 64                                // K values per chunk and chunks in flight of the shapes that are built
+#define MID_DEPTH 2
+
 template <int MT, typename TO>
 static int mid_strips(const void* x, const void* w, const float* bias, void* out, int M, int N, int K, int strips,
-                      int splits, int chunks_per_split, bool swiglu, float* partial, hipStream_t stream) {
-    if (strips >= 2) return mid_launch<MT, 2, TO>(x, w, bias, out, M, N, K, splits, chunks_per_split, swiglu, partial, stream);
-    return mid_launch<MT, 1, TO>(x, w, bias, out, M, N, K, splits, chunks_per_split, swiglu, partial, stream);
+                      int splits, bool swiglu, float* partial, hipStream_t stream) {
+    if (strips >= 2) return mid_launch<MT, 2, MID_CK, MID_DEPTH, TO>(x, w, bias, out, M, N, K, splits, swiglu, partial, stream);
+    return mid_launch<MT, 1, MID_CK, MID_DEPTH, TO>(x, w, bias, out, M, N, K, splits, swiglu, partial, stream);
 }
 
 // Floats of workspace one launch needs: the partial sums of every split (nothing for one split).
@@ -275,7 +289,9 @@ static int64_t mid_workspace_floats(int M, int N, int strips, int splits) {
 
 // The launch shape: strips per wavefront and splits of K.  Two strips where the columns still give every
 // compute unit a workgroup; K is split until there are about two workgroups per compute unit, in
-// pieces of at least 8 chunks, within the workspace.
+// pieces of at least 8 chunks, within the workspace.  Chosen by whole decode steps of 64 requests at 7B
+// layer sizes (7.7 ms with this rule: down in 8 splits, gate_up in 2; 8.0 ms with at most 5 or 3 splits,
+// 7.9 ms with twice as many); timing the kernel alone in a loop ranks the shapes differently.
 static void mid_shape(int M, int N, int K, bool swiglu, int64_t workspace_floats, int* strips, int* splits) {
     const int chunks = ceil_div(K, MID_CK);
     int ns = (swiglu || ceil_div(N, 128) >= 256) ? 2 : 1;
@@ -305,11 +321,10 @@ static int mid_check(const void* x, const void* w, int out_dtype, int M, int N, 
 static int mid_dispatch(const void* x, const void* w, const float* bias, void* out, int out_dtype, int M, int N, int K,
                         int strips, int splits, bool swiglu, float* partial, hipStream_t stream) {
     const int mt = ceil_div(M, 16);
-    const int chunks_per_split = ceil_div(ceil_div(K, MID_CK), splits);
 #define SOMI_MID(MT)                                                                                                 \
     return out_dtype == SOMI_BF16                                                                                    \
-               ? mid_strips<MT, bf16>(x, w, bias, out, M, N, K, strips, splits, chunks_per_split, swiglu, partial, stream) \
-               : mid_strips<MT, float>(x, w, bias, out, M, N, K, strips, splits, chunks_per_split, swiglu, partial, stream)
+               ? mid_strips<MT, bf16>(x, w, bias, out, M, N, K, strips, splits, swiglu, partial, stream) \
+               : mid_strips<MT, float>(x, w, bias, out, M, N, K, strips, splits, swiglu, partial, stream)
     switch (mt) {
         case 1: SOMI_MID(1);
         case 2: SOMI_MID(2);
@@ -347,3 +362,4 @@ extern "C" int somi_linear_mid_shaped(const void* x, const void* w, const float*
     if (M == 0) return 0;
     return mid_dispatch(x, w, bias, out, out_dtype, M, N, K, strips, splits, swiglu != 0, workspace, stream);
 }
+#endif
