@@ -205,7 +205,10 @@ attention_prefill_kernel(const bf16* __restrict__ q, int64_t q_stride, const bf1
 //   K tile in LDS: [32 keys][D + 8] (rows padded by 16 bytes: the 16 rows a 16-byte read touches fall into
 //   different banks); V tile: [D channels][32 + 4 keys].
 #define PREFILL_LDS_PAGES 2048     // block-table entries of the visible range kept in LDS (else read from memory)
-template <int DT>
+#ifndef PREFILL_WIDE_GROUPS
+#define PREFILL_WIDE_GROUPS 768    // from this many 128-query groups on, workgroups take 128 queries, else 64
+#endif
+template <int DT, int QB>
 __global__ void __launch_bounds__(256, 2)
 attention_prefill_lds_kernel(const bf16* __restrict__ q, int64_t q_stride, const bf16* __restrict__ kc,
                              const bf16* __restrict__ vc, const int* __restrict__ block_table, int max_blocks,
@@ -213,7 +216,7 @@ attention_prefill_lds_kernel(const bf16* __restrict__ q, int64_t q_stride, const
                              int nkv, int page_size, int window, float scale_log2, bf16* __restrict__ out) {
     constexpr int D = DT * 16;
     constexpr int QK_STEPS = (DT + 1) / 2;
-    constexpr int QB = 2, QW = QB * 16, WAVES = 4, QG = WAVES * QW;     // 128 queries per workgroup
+    constexpr int QW = QB * 16, WAVES = 4, QG = WAVES * QW;             // 64 or 128 queries per workgroup
     constexpr int KROW = D + 8, VROW = 32 + 4;                          // padded LDS rows, in elements
     constexpr int K_CHUNKS = 32 * D / 8;                                // 16-byte pieces of a key tile
     constexpr int K_PER_THREAD = (K_CHUNKS + 255) / 256;
@@ -224,12 +227,16 @@ attention_prefill_lds_kernel(const bf16* __restrict__ q, int64_t q_stride, const
     __shared__ __attribute__((aligned(16))) bf16 vs[2][D * VROW];
     __shared__ int pages[PREFILL_LDS_PAGES];
 
-    const int e = blockIdx.y, h = blockIdx.z;
+    // Workgroups are handed out in the order of blockIdx.x, then y, then z: heads vary fastest (the query
+    // heads of one key/value head run side by side and share its tiles in L2) and the query groups go from
+    // the latest, which see the most keys, to the earliest, so that the compute units fill up with long
+    // workgroups first and the short ones land beside them.
+    const int h = blockIdx.x, e = blockIdx.y;
     const int kvh = h / (nq / nkv);
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, r = lane & 15, g = lane >> 4;
     const int start = entry_start[e];
     const int len = entry_start[e + 1] - start;
-    const int group = gridDim.x - 1 - blockIdx.x;           // the longest (latest) query groups start first
+    const int group = gridDim.z - 1 - blockIdx.z;
     const int g0 = group * QG;
     if (g0 >= len) return;                                  // the whole workgroup leaves together
     const int pos0 = entry_first_pos[e];
@@ -449,10 +456,18 @@ static int launch_prefill_lds(const void* q, int64_t q_stride, const void* kc, c
                               int max_blocks, const int* entry_start, const int* entry_first_pos, int n_entries,
                               int max_entry_len, int nq, int nkv, int page_size, int window, float scale, void* out,
                               hipStream_t stream) {
-    const dim3 grid(ceil_div(max_entry_len, 128), n_entries, nq);
-    hipLaunchKernelGGL((attention_prefill_lds_kernel<DT>), grid, dim3(256), 0, stream, (const bf16*)q, q_stride,
-                       (const bf16*)kc, (const bf16*)vc, block_table, max_blocks, entry_start, entry_first_pos, nq, nkv,
-                       page_size, window, scale * 1.44269504088896341f, (bf16*)out);
+    // 128 queries per workgroup read every key and value tile half as often as 64 do, but the longest
+    // workgroup sets the time: with few workgroups the smaller ones spread better over the compute units.
+    const bool wide = (int64_t)ceil_div(max_entry_len, 128) * n_entries * nq >= PREFILL_WIDE_GROUPS;
+    const dim3 grid(nq, n_entries, ceil_div(max_entry_len, wide ? 128 : 64));
+    if (wide)
+        hipLaunchKernelGGL((attention_prefill_lds_kernel<DT, 2>), grid, dim3(256), 0, stream, (const bf16*)q, q_stride,
+                           (const bf16*)kc, (const bf16*)vc, block_table, max_blocks, entry_start, entry_first_pos, nq,
+                           nkv, page_size, window, scale * 1.44269504088896341f, (bf16*)out);
+    else
+        hipLaunchKernelGGL((attention_prefill_lds_kernel<DT, 1>), grid, dim3(256), 0, stream, (const bf16*)q, q_stride,
+                           (const bf16*)kc, (const bf16*)vc, block_table, max_blocks, entry_start, entry_first_pos, nq,
+                           nkv, page_size, window, scale * 1.44269504088896341f, (bf16*)out);
     SOMI_LAUNCH_CHECK("attention_prefill_lds");
     return 0;
 }
@@ -488,6 +503,7 @@ extern "C" int somi_attention_prefill(const void* q, int64_t q_stride, const voi
     SOMI_REQUIRE(page_size > 0 && page_size % 4 == 0, "attention_prefill: page size %d must be a multiple of 4", page_size);
     SOMI_REQUIRE(window >= 0, "attention_prefill: window must be >= 0");
     SOMI_REQUIRE(n_entries <= 65535 && nq <= 65535, "attention_prefill: too many entries or heads");
+    SOMI_REQUIRE(max_entry_len <= 65535 * 128, "attention_prefill: a portion of %d tokens is too long", max_entry_len);
     SOMI_REQUIRE((uintptr_t)q % 16 == 0 && (q_stride * 2) % 16 == 0 && (uintptr_t)k_cache % 16 == 0 &&
                  (uintptr_t)v_cache % 8 == 0 && (uintptr_t)out % 8 == 0,
                  "attention_prefill: q, k, v and out must be 16-byte aligned");
