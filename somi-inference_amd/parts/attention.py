@@ -25,6 +25,7 @@ from .registry import build_part
 
 class GroupedQueryAttention(Mixer):
     graph_safe = True
+    takes_normed_rows = True      # x only goes through the q/k/v projection, which norms rows while loading them
 
     def __init__(self, prefix: str, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  position: PartSpec, qkv_bias: bool = True, out_bias: bool = False,
@@ -94,4 +95,4 @@ class GroupedQueryAttention(Mixer):
         attended = attention_kernels.paged_attention(
             qkv, self.num_heads, cache.k, cache.v, view.block_table, step,
             window=self.window or 0, scale=self.scale)
-        return self.out(attended)
+        return self.out.deferred(attended)        # the residual stream may add it in the kernel that computes it

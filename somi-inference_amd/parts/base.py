@@ -147,13 +147,19 @@ class Mixer(Part):
     def cache_spec(self) -> PagedKVSpec | FixedStateSpec | None:
         return None
 
+    takes_normed_rows = False      # True: x may arrive as parts.linear.NormedRows (rows still to be normed)
+
     def forward(self, x: torch.Tensor, step: Any, cache: LayerCache | None) -> torch.Tensor:
-        """x: [N, H] compute dtype -> [N, H] compute dtype."""
+        """x: [N, H] compute dtype -> [N, H] compute dtype, or a parts.linear.DeferredProduct of that shape
+        (the part's last projection, left for the residual stream to compute and add in one kernel)."""
         raise NotImplementedError
 
 
 class FeedForward(Part):
+    takes_normed_rows = False
+
     def forward(self, x: torch.Tensor, step: Any) -> torch.Tensor:
+        """x: [N, H] -> [N, H], or a DeferredProduct, as for a mixer."""
         raise NotImplementedError
 
 

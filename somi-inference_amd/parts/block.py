@@ -32,7 +32,7 @@ class PreNormBlock(Block):
         return [self.mixer_norm, self.mixer, self.ffn_norm, self.feed_forward]
 
     def forward(self, stream: ResidualStream, step, cache: LayerCache | None) -> None:
-        x = stream.normed(self.mixer_norm)
+        x = stream.normed(self.mixer_norm, lazy=getattr(self.mixer, "takes_normed_rows", False))
         stream.add(self.mixer.forward(x, step, cache))
-        x = stream.normed(self.ffn_norm)
+        x = stream.normed(self.ffn_norm, lazy=getattr(self.feed_forward, "takes_normed_rows", False))
         stream.add(self.feed_forward.forward(x, step))

@@ -8,7 +8,7 @@ from ..kernels import linear as linear_kernels
 from ..kernels import ops
 from ..weights.spec import MATRIX, WeightSpec
 from .base import FeedForward, Fetch, Runtime
-from .linear import Projection
+from .linear import NormedRows, Projection
 
 
 class SwiGLU(FeedForward):
@@ -16,6 +16,7 @@ class SwiGLU(FeedForward):
     ``[2I, H]`` matrix, gate rows first, as the reference merges them at load
     (somi_inference/models/qwen2_adapter.py:183-190, 244-248; qwen2.py:228 chunks the result)."""
     graph_safe = True
+    takes_normed_rows = True
 
     def __init__(self, prefix: str, hidden_size: int, intermediate_size: int) -> None:
         super().__init__(prefix)
@@ -45,9 +46,15 @@ class SwiGLU(FeedForward):
             self.gate_up = Projection.stacked([gate, up])
         self.down = Projection(fetch(self.name("down_proj.weight")))
 
-    def forward(self, x: torch.Tensor, step=None) -> torch.Tensor:
+    def forward(self, x, step=None):
+        if isinstance(x, NormedRows):
+            if self.interleaved and self.gate_up.fusable(x.h.shape[0]):
+                # norm, gate_up and SiLU . up in one kernel
+                return self.down.deferred(ops.linear_scaled(x.weighted, x.norm.eps, x.stats, self.gate_up.weight,
+                                                            swiglu=True))
+            x = x.materialize()
         if not self.interleaved:
-            return self.down(ops.silu_mul(self.gate_up(x)))
+            return self.down.deferred(ops.silu_mul(self.gate_up(x)))
         if x.shape[0] <= linear_kernels.SKINNY_ROWS and x.data_ptr() % 16 == 0:
-            return self.down(linear_kernels.linear_swiglu(x, self.gate_up.weight))
-        return self.down(ops.silu_mul(self.gate_up(x), block=self.INTERLEAVE))
+            return self.down.deferred(linear_kernels.linear_swiglu(x, self.gate_up.weight))
+        return self.down.deferred(ops.silu_mul(self.gate_up(x), block=self.INTERLEAVE))

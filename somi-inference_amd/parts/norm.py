@@ -13,6 +13,7 @@ class RMSNorm(Norm):
     """y = w * x * rsqrt(mean(x^2) + eps), no mean subtraction, no bias
     (qwen2.py:55-62).  Square, mean, rsqrt and scale are float32."""
     graph_safe = True
+    fusable = True        # weight * (h / sqrt(mean(h^2) + eps)): what a projection can apply while it loads h
 
     def __init__(self, prefix: str, hidden_size: int, eps: float,
                  init: tuple[float, float] = (1.0, 0.1)) -> None:

@@ -31,6 +31,11 @@ def close(got, want, dtype):
     torch.testing.assert_close(got.float().cpu(), want, atol=rel * max(scale, 1e-3), rtol=rel)
 
 
+def rows(out):
+    """A part's output as a tensor: its last projection may come back not yet computed."""
+    return out.materialize() if hasattr(out, "materialize") else out
+
+
 def load_random(part, dtype, seed=0, scale=None):
     """Load a part from seeded random tensors; returns them as float32 CPU tensors for the plain side."""
     source = RandomSource(part.weight_specs(), seed)
@@ -71,7 +76,7 @@ def test_swiglu_part(dtype):
     assert tuple(ffn.gate_up.weight.shape) == (400, 72)              # merged weight (2I, H): reference test_qwen2_mlp.py:17-20
     x = torch.randn(9, 72, device=DEV).to(DT[dtype])
     want = plain.swiglu(x.float().cpu(), w["m.gate_proj.weight"], w["m.up_proj.weight"], w["m.down_proj.weight"])
-    close(ffn.forward(x), want, dtype)
+    close(rows(ffn.forward(x)), want, dtype)
 
 
 def attention_setup(dtype, nq, nkv, d, hidden, window=None, theta=1e4, block_size=4, seed=0):
@@ -96,7 +101,7 @@ def test_attention_part_whole_and_in_portions(dtype, nq, nkv, d, hidden, window)
         for size in sizes:
             cache.reserve("r", size)
             step = build_step([StepEntry("r", [0] * size, [])], cache, DEV)
-            outs.append(attn.forward(x[at:at + size].contiguous(), step, cache.layer_caches[0]))
+            outs.append(rows(attn.forward(x[at:at + size].contiguous(), step, cache.layer_caches[0])))
             cache.commit("r", size)
             at += size
         cache.free("r")
@@ -132,8 +137,8 @@ def test_attention_part_far_key_among_hundreds_and_window_edge(dtype):
                      cache.layer_caches[0])
         cache.commit("r", length - 1)
         cache.reserve("r", 1)
-        got = attn.forward(x[length - 1:].contiguous(), build_step([StepEntry("r", [0], [])], cache, DEV),
-                           cache.layer_caches[0])
+        got = rows(attn.forward(x[length - 1:].contiguous(), build_step([StepEntry("r", [0], [])], cache, DEV),
+                                cache.layer_caches[0]))
         if dtype == "float32":
             torch.testing.assert_close(got.cpu(), want[-1:], atol=1e-4, rtol=1e-3)
         else:
@@ -259,3 +264,51 @@ def test_rotary_part_offers_the_reference_table():
     assert rotary_dim == 8 and inv_freq.dtype == torch.float32
     # reference: cos_cached[1][1] = cos(1e6^-0.25) for dim 8 (tests/models/test_qwen2.py:75-88)
     assert inv_freq.cpu().tolist() == pytest.approx([1.0, 1e6 ** -0.25, 1e6 ** -0.5, 1e6 ** -0.75], rel=1e-6)
+
+
+def test_a_few_bfloat16_rows_take_the_add_and_the_norm_inside_the_products():
+    """Decode-sized steps in bfloat16: a block's last projections arrive at the residual stream uncomputed and are
+    added to it by the kernel that computes them; the next norm is applied by the projection that reads the
+    rows.  The stream ends up where separate add and norm kernels put it (up to the rounding of the deltas to
+    bfloat16, which the fused way skips)."""
+    from somi_inference_amd.parts.linear import DeferredProduct, NormedRows
+    hidden, inter = 96, 160
+    ffn = SwiGLU("m", hidden_size=hidden, intermediate_size=inter)
+    w = load_random(ffn, "bfloat16", scale=4.0)
+    norm = RMSNorm("n", hidden_size=hidden, eps=1e-5)
+    wn = load_random(norm, "bfloat16")
+    h0 = torch.randn(7, hidden, device=DEV)
+    x = norm.forward(h0)
+    out = ffn.forward(x)
+    assert isinstance(out, DeferredProduct) and out.shape == (7, hidden)
+    # the fused way through the stream
+    stream = ResidualStream(h0.clone())
+    stream.add(out)
+    lazy = stream.normed(norm, lazy=True)
+    assert isinstance(lazy, NormedRows)
+    lazy_rows = lazy.materialize().float()                       # before the stream moves on
+    assert torch.equal(lazy.weighted, (norm.weight * stream.h).to(torch.bfloat16))
+    second = ffn.forward(lazy)                                   # norm + gate_up + SiLU.up in one kernel
+    assert isinstance(second, DeferredProduct)
+    stream.add(second)
+    fused = stream.settle().clone()
+    # the separate way
+    plain_stream = ResidualStream(h0.clone())
+    plain_stream.add(out.materialize())
+    x2 = plain_stream.normed(norm)
+    assert torch.is_tensor(x2)
+    torch.testing.assert_close(lazy_rows, x2.float(), atol=2e-2, rtol=2e-2)
+    plain_stream.add(rows(ffn.forward(x2)))
+    separate = plain_stream.settle()
+    scale = float(separate.abs().max())
+    torch.testing.assert_close(fused, separate, atol=scale * 2 ** -6, rtol=2 ** -6)
+    # against float32 formulas
+    h1 = h0.cpu() + plain.swiglu(x.float().cpu(), w["m.gate_proj.weight"], w["m.up_proj.weight"], w["m.down_proj.weight"])
+    x2_plain = plain.rms_norm(h1, wn["n.weight"], 1e-5)
+    h2 = h1 + plain.swiglu(x2_plain, w["m.gate_proj.weight"], w["m.up_proj.weight"], w["m.down_proj.weight"])
+    close(fused, h2, "bfloat16")
+    # many rows, or float32, stay with the separate kernels
+    assert torch.is_tensor(ffn.forward(torch.randn(40, hidden, device=DEV).to(torch.bfloat16)))
+    ffn32 = SwiGLU("m", hidden_size=hidden, intermediate_size=inter)
+    load_random(ffn32, "float32")
+    assert torch.is_tensor(ffn32.forward(torch.randn(7, hidden, device=DEV)))
