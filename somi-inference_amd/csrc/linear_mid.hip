@@ -269,6 +269,8 @@ static int mid_launch(const void* x, const void* w, const float* bias, void* out
     return 0;
 }
 
+// A program that measures other shapes (chunk sizes, depths) can include this file with SOMI_MID_NO_ENTRY_POINTS
+// defined and instantiate the launchers above itself; the library builds what follows.
 #ifndef SOMI_MID_NO_ENTRY_POINTS
 #define MID_CK 64                                // K values per chunk and chunks in flight of the shapes that are built
 #define MID_DEPTH 2

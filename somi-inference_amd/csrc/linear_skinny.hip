@@ -235,6 +235,8 @@ static int skinny_launch(const void* x, const void* w, const float* bias, void* 
     return 0;
 }
 
+// A program that measures other shapes (chunk sizes, depths) can include this file with SOMI_SKINNY_NO_ENTRY_POINTS
+// defined and instantiate the launchers above itself; the library builds what follows.
 #ifndef SOMI_SKINNY_NO_ENTRY_POINTS
 // The shapes that are built: 1, 2 or 4 strips with chunks of 64, two chunks in flight.
 template <int MT, typename TO>
