@@ -215,28 +215,35 @@ def test_captured_decode_steps_replay_like_eager_steps(dtype, model_folders):
     assert graphed.graph_replays >= 24
 
 
-@pytest.fixture(scope="module")
-def real_size_folder(tmp_path_factory):
-    """One layer of the 7B layer sizes (hidden 3584, 28 query heads over 4 key/value heads of 128, intermediate
-    18944) with a small vocabulary, so that the kernels run at the shapes they are tuned for."""
+REAL_SIZES = {
+    # one layer of the 7B layer sizes: the shapes the kernels are tuned for
+    "7b": dict(hidden_size=3584, intermediate_size=18944, num_hidden_layers=1, num_attention_heads=28,
+               num_key_value_heads=4, head_dim=128, rope_theta=1e6, rms_norm_eps=1e-6, tie_word_embeddings=False),
+    # two layers of the 0.5B layer sizes: heads of 64, 7 query heads per key/value head, tied embeddings
+    "0.5b": dict(hidden_size=896, intermediate_size=4864, num_hidden_layers=2, num_attention_heads=14,
+                 num_key_value_heads=2, head_dim=64, rope_theta=1e6, rms_norm_eps=1e-6, tie_word_embeddings=True),
+}
+
+
+@pytest.fixture(scope="module", params=sorted(REAL_SIZES))
+def real_size_folder(request, tmp_path_factory):
+    """Layers of real layer sizes with a small vocabulary and random weights."""
     from somi_inference_amd.config import Qwen2Config
     from somi_inference_amd.weights import write_random_model
-    config = Qwen2Config(vocab_size=1031, hidden_size=3584, intermediate_size=18944, num_hidden_layers=1,
-                         num_attention_heads=28, num_key_value_heads=4, head_dim=128, rope_theta=1e6,
-                         rms_norm_eps=1e-6, tie_word_embeddings=False)
-    folder = str(tmp_path_factory.mktemp("real") / "one_layer_7b")
+    config = Qwen2Config(vocab_size=1031, **REAL_SIZES[request.param])
+    folder = str(tmp_path_factory.mktemp("real") / f"layers_{request.param}")
     write_random_model(folder, config, seed=5)
-    return {"float32": peaky_folder(folder, folder + "_peaky", factor=3.0), "bfloat16": folder}, config
+    return {"float32": peaky_folder(folder, folder + "_peaky", factor=3.0), "bfloat16": folder}, config, request.param
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_one_layer_of_the_7b_sizes_under_all_cuttings(dtype, real_size_folder):
+def test_layers_of_real_sizes_under_all_cuttings(dtype, real_size_folder):
     """With sums over up to 18,944 terms the order of float32 additions shows: the float32 engine is held to
     the accuracy of the plain float32 implementation itself, both measured against the plain implementation
     in float64 (its error may be a few times the plain one's, not more).  The float32 run uses sharpened
     attention (single keys decide); in bfloat16 that sharpening amplifies the rounding of q and k into
     per-cent changes of the weights, so the bfloat16 run uses the weights as drawn."""
-    folders, config = real_size_folder
+    folders, config, sizes = real_size_folder
     folder = folders[dtype]
     cfg, weights = plain.read_model(folder)
     tokens = token_ids(config.vocab_size, 333, 8)
@@ -263,9 +270,9 @@ def test_one_layer_of_the_7b_sizes_under_all_cuttings(dtype, real_size_folder):
     runner, _ = make_engine(folder, dtype, 16, 64, max_requests=4)
     everything = list(range(len(tokens)))
     whole = run_portions(runner, "w", tokens, [333])
-    check(whole, everything, f"7B layer sizes {dtype}: whole prompt")
+    check(whole, everything, f"{sizes} layer sizes {dtype}: whole prompt")
     cut = run_portions(runner, "c", tokens, [150, 2, 37, 1, 1, 64, 9, 33] + [1] * 36)
-    check(cut, everything, f"7B layer sizes {dtype}: portions and decoded tokens")
+    check(cut, everything, f"{sizes} layer sizes {dtype}: portions and decoded tokens")
     if dtype == "float32":
         assert torch.equal(cut, whole)
     # three requests decoding together after prompts of different lengths
@@ -276,7 +283,7 @@ def test_one_layer_of_the_7b_sizes_under_all_cuttings(dtype, real_size_folder):
     for step in range(20):
         entries = [StepEntry(rid, [tokens[len(p) + step]], [0]) for rid, p in prompts.items()]
         got = runner.step(entries).cpu()
-        check(got, [len(p) + step for p in prompts.values()], f"7B layer sizes {dtype}: batched decode step {step}")
+        check(got, [len(p) + step for p in prompts.values()], f"{sizes} layer sizes {dtype}: batched decode step {step}")
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
