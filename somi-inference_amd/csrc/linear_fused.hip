@@ -1,4 +1,4 @@
-// Two forms of the few-rows product of linear_skinny.hip (at most 16 rows) that take the RMSNorm and the
+// Two forms of the few-rows product of linear_skinny.hip (at most 64 rows) that take the RMSNorm and the
 // residual add of a pre-norm block into the products around them, so that a decode step launches no
 // kernel of its own for either.  RMSNorm is weight * h * s with one scale s = 1 / sqrt(mean(h^2) + eps) per
 // row, and a product is linear in that scale: norm(h) . W^T = s * ((weight * h) . W^T).  So
@@ -6,7 +6,7 @@
 //   * the product INTO the residual stream (o_proj, down_proj):  h[m, n] += x[m, :] . w[n, :] (+ bias[n]) in
 //     float32; the workgroup also writes the rows the next product reads, x'[m, n] = bfloat16(weight[n] *
 //     h[m, n]) with the next norm's weight (no scale yet), and, for each row, the sum of squares of the new h
-//     over its columns (`stats`: [workgroups][16] float32);
+//     over its columns (`stats`: [workgroups][16 * ceil(M / 16)] float32);
 //   * the product OUT OF the residual stream (q/k/v, gate_up):  out = s * (x' . w^T) (+ bias), where s comes
 //     from the producer's partial sums, added in workgroup order (a fixed order), and is applied to the
 //     float32 sums (before the bias, before SiLU in the gated form).
@@ -21,8 +21,8 @@
 #include "common.h"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
-typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
 typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
 
 #define SOMI_BUFFER_WORD3 0x00020000u            // raw buffer, 32-bit elements, no swizzle
@@ -32,20 +32,21 @@ typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
 #define FUSED_SCALED 1
 #define FUSED_RESIDUAL 2
 
-template <int NS, int MODE, typename TO, bool SWIGLU, bool TAIL>
+template <int MT, int NS, int MODE, typename TO, bool SWIGLU, bool TAIL>
 __global__ void __launch_bounds__(FUSED_MAX_WAVES * 64)
 linear_fused_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, const float* __restrict__ bias,
                     TO* __restrict__ out, float* __restrict__ h, const float* __restrict__ norm_w, float eps,
                     const float* __restrict__ stats_in, int stats_blocks, float* __restrict__ stats_out,
                     bf16* __restrict__ xnext, int M, int N, int K) {
     extern __shared__ __attribute__((aligned(16))) char lds[];
-    __shared__ float row_scale[16];
+    __shared__ float row_scale[64];
+    __shared__ float part[FUSED_MAX_WAVES * 4 * 16 * MT];
     constexpr bool SCALED = MODE == FUSED_SCALED;
     constexpr int ROW_BYTES = FUSED_CK * 2;        // a row of a chunk in LDS: 64 bfloat16
-    constexpr int WL = 2;                          // loads per 16 rows of w: 8 lanes read the 128 bytes of a row
-    constexpr int XL = 2;                          // loads of the 16 rows of x
-    constexpr int WAVE_BYTES = 16 * (NS + 1) * ROW_BYTES;
-    constexpr int NW = NS * WL;
+    constexpr int ROWS = 16 * MT;                  // rows of x the kernel is built for
+    constexpr int WAVE_BYTES = 16 * (NS + MT) * ROW_BYTES;
+    constexpr int NL = (NS + MT) * 2;              // loads per lane and chunk: 8 lanes read the 128 bytes of a row
+    constexpr int TILES = NS * MT;
 
     const int waves = blockDim.x >> 6;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -60,92 +61,102 @@ linear_fused_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, cons
         (void*)x, 0, (int)((int64_t)M * K * 2), SOMI_BUFFER_WORD3);
 
     auto swizzle = [](int row16) { return (row16 & 7) ^ (row16 >> 3); };
-    // lane l reads 16 bytes (8 values) of row (l / 8) of each group of 8 rows
+    // lane l reads 16 bytes (8 values) of row (l / 8) of each group of 8 rows; tiles 0..NS-1 are w, the others x
     const int lchunk = lane & 7;
-    unsigned wgoff[NW];
-    int wsoff[NW];
+    unsigned goff[NL];
+    int soff[NL];
 #pragma unroll
-    for (int i = 0; i < NW; ++i) {
-        const int row16 = (i % WL) * 8 + (lane >> 3), tile = i / WL;
-        wgoff[i] = ((unsigned)(tile * 16 + row16) * (unsigned)K + lchunk * 8) * 2u;
-        wsoff[i] = (tile * 16 + row16) * ROW_BYTES + ((lchunk ^ swizzle(row16)) << 4);
-    }
-    unsigned xgoff[XL];
-    int xsoff[XL];
-#pragma unroll
-    for (int j = 0; j < XL; ++j) {
-        const int row16 = j * 8 + (lane >> 3);
-        xgoff[j] = ((unsigned)row16 * (unsigned)K + lchunk * 8) * 2u;
-        xsoff[j] = (NS * 16 + row16) * ROW_BYTES + ((lchunk ^ swizzle(row16)) << 4);
+    for (int i = 0; i < NL; ++i) {
+        const int tile = i / 2, row16 = (i % 2) * 8 + (lane >> 3);
+        const int row = tile < NS ? tile * 16 + row16 : (tile - NS) * 16 + row16;
+        goff[i] = ((unsigned)row * (unsigned)K + lchunk * 8) * 2u;
+        soff[i] = (tile * 16 + row16) * ROW_BYTES + ((lchunk ^ swizzle(row16)) << 4);
     }
     const int rswz = swizzle(r);
 
-    f32x4 acc[NS];
+    f32x4 acc[NS][MT];
 #pragma unroll
-    for (int s = 0; s < NS; ++s) acc[s] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int s = 0; s < NS; ++s)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) acc[s][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
     const int chunks = (K + FUSED_CK - 1) / FUSED_CK;
     const int mine_n = wave < chunks ? (chunks - wave + waves - 1) / waves : 0;
 
-    struct Stage {
-        u32x4 wv[NW];
-        u32x4 xv[XL];
-    };
-    auto issue = [&](Stage& st, int at) {
+    auto issue = [&](u32x4 (&st)[NL], int at) {
         const int k0 = (wave + at * waves) * FUSED_CK;
         const bool inside = !TAIL || k0 + lchunk * 8 < K;
 #pragma unroll
-        for (int i = 0; i < NW; ++i)
-            st.wv[i] = __builtin_amdgcn_raw_buffer_load_b128(
-                wres, inside ? wgoff[i] + (unsigned)k0 * 2u : SOMI_OUT_OF_RANGE, 0, 0);
-#pragma unroll
-        for (int j = 0; j < XL; ++j)
-            st.xv[j] = __builtin_amdgcn_raw_buffer_load_b128(
-                xres, inside ? xgoff[j] + (unsigned)k0 * 2u : SOMI_OUT_OF_RANGE, 0, 0);
+        for (int i = 0; i < NL; ++i)
+            st[i] = __builtin_amdgcn_raw_buffer_load_b128(
+                i < NS * 2 ? wres : xres, inside ? goff[i] + (unsigned)k0 * 2u : SOMI_OUT_OF_RANGE, 0, 0);
     };
-    auto stash = [&](const Stage& st) {
+    auto stash = [&](const u32x4 (&st)[NL]) {
 #pragma unroll
-        for (int i = 0; i < NW; ++i) *reinterpret_cast<u32x4*>(mine + wsoff[i]) = st.wv[i];
-#pragma unroll
-        for (int j = 0; j < XL; ++j) *reinterpret_cast<u32x4*>(mine + xsoff[j]) = st.xv[j];
+        for (int i = 0; i < NL; ++i) *reinterpret_cast<u32x4*>(mine + soff[i]) = st[i];
     };
     auto operand = [&](int tile, int c) -> bf16x8 {
         return *reinterpret_cast<const bf16x8*>(mine + (tile * 16 + r) * ROW_BYTES + ((c ^ rswz) << 4));
     };
     auto compute = [&]() {
-        const bf16x8 xa = operand(NS, 2 * g), xb = operand(NS, 2 * g + 1);
+        bf16x8 xa[MT], xb[MT];
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            xa[mt] = operand(NS + mt, 2 * g);
+            xb[mt] = operand(NS + mt, 2 * g + 1);
+        }
 #pragma unroll
         for (int s = 0; s < NS; ++s) {
             const bf16x8 wa = operand(s, 2 * g), wb = operand(s, 2 * g + 1);
-            acc[s] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa, xa, acc[s], 0, 0, 0);
-            acc[s] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wb, xb, acc[s], 0, 0, 0);
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                acc[s][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa, xa[mt], acc[s][mt], 0, 0, 0);
+                acc[s][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wb, xb[mt], acc[s][mt], 0, 0, 0);
+            }
         }
     };
 
-    // two chunks in flight
-    Stage A, B;
-    if (mine_n >= 1) issue(A, 0);                    // the first loads are under way while the scales are worked out
+    u32x4 A[NL], B[NL];
+    if (mine_n >= 1) issue(A, 0);                    // the first loads are under way while what follows is fetched
     if (mine_n >= 2) issue(B, 1);
-    // The rows' scales come from the producer's partial sums of squares, added in a fixed order: thread t
-    // adds the workgroups t / 16, t / 16 + threads / 16, ... of row t % 16, then 16 threads add those in thread
-    // order.  The first loads go out here, before the weight stream, and are only looked at after it.
+    // The rows' scales come from the producer's partial sums of squares [stats_blocks][ROWS], added in a fixed
+    // order: lane l of wavefront v adds the rows MT (l % 16) .. + MT - 1 (one load) of the workgroups
+    // 4 v + l / 16, that + 4 waves, ...; then a thread per row adds those sums in order.  The first loads go
+    // out here, before the weight stream, and are only looked at after it.
     constexpr int EARLY = 8;
-    float early[EARLY];
-    const int stride_b = blockDim.x >> 4;
+    float early[EARLY][MT];
+    const int stats_group = wave * 4 + g, stats_groups = waves * 4;
+    auto stats_load = [&](float (&to)[MT], int block) {
+        const float* from = stats_in + (int64_t)block * ROWS + r * MT;
+        if (block < stats_blocks) {
+            __builtin_memcpy(&to[0], __builtin_assume_aligned(from, MT == 3 ? 4 : 4 * MT), 4 * MT);
+        } else {
+#pragma unroll
+            for (int j = 0; j < MT; ++j) to[j] = 0.f;
+        }
+    };
     if (SCALED) {
 #pragma unroll
-        for (int i = 0; i < EARLY; ++i) {
-            const int b = (threadIdx.x >> 4) + i * stride_b;
-            early[i] = b < stats_blocks ? stats_in[b * 16 + (threadIdx.x & 15)] : 0.f;
-        }
+        for (int i = 0; i < EARLY; ++i) stats_load(early[i], stats_group + i * stats_groups);
     }
-    // the product into the stream: this thread's element of h, fetched ahead of its use in the epilogue
-    const bool one_pass = (int)blockDim.x >= NS * 256;
-    float h_before = 0.f;
-    if (MODE == FUSED_RESIDUAL && one_pass && (int)threadIdx.x < NS * 256) {
-        const int idx = threadIdx.x, l = (idx >> 2) & 63;
-        const int n = n0 + (idx >> 8) * 16 + (l >> 4) * 4 + (idx & 3), m = l & 15;
-        if (n < N && m < M) h_before = h[(int64_t)m * N + n];
+    // The end of the kernel deals the sums out four consecutive columns (one lane's share of a tile) to a thread;
+    // they are one access where the row length and the addresses keep them aligned and inside together.
+    const bool whole = (N & 3) == 0 && (((uintptr_t)bias | (uintptr_t)h | (uintptr_t)norm_w) & 15) == 0 &&
+                       (((uintptr_t)xnext | (uintptr_t)out) & 7) == 0;
+    auto load4 = [&](const float* from, int n) -> f32x4 {
+        if (whole) return *reinterpret_cast<const f32x4*>(from);
+        f32x4 v;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] = n + i < N ? from[i] : 0.f;
+        return v;
+    };
+    // the product into the stream: this thread's elements of h, fetched ahead of their use
+    const bool one_pass = (int)blockDim.x >= TILES * 64;
+    f32x4 h_before = {0.f, 0.f, 0.f, 0.f};
+    if (MODE == FUSED_RESIDUAL && one_pass && (int)threadIdx.x < TILES * 64) {
+        const int tile = threadIdx.x >> 6;
+        const int n = n0 + (tile / MT) * 16 + g * 4, m = (tile % MT) * 16 + r;
+        if (n < N && m < M) h_before = load4(h + (int64_t)m * N + n, n);
     }
 
     if (mine_n >= 2) {
@@ -173,36 +184,50 @@ linear_fused_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, cons
         compute();
     }
 
-    __shared__ float part[FUSED_MAX_WAVES * 64];
     if (SCALED) {
-        float mine_sum = 0.f;
+        float mine_sum[MT];
 #pragma unroll
-        for (int i = 0; i < EARLY; ++i) mine_sum += early[i];
-        for (int b = (threadIdx.x >> 4) + EARLY * stride_b; b < stats_blocks; b += stride_b)
-            mine_sum += stats_in[b * 16 + (threadIdx.x & 15)];
-        part[threadIdx.x] = mine_sum;
+        for (int j = 0; j < MT; ++j) mine_sum[j] = 0.f;
+#pragma unroll
+        for (int i = 0; i < EARLY; ++i)
+#pragma unroll
+            for (int j = 0; j < MT; ++j) mine_sum[j] += early[i][j];
+        for (int b = stats_group + EARLY * stats_groups; b < stats_blocks; b += stats_groups) {
+            float more[MT];
+            stats_load(more, b);
+#pragma unroll
+            for (int j = 0; j < MT; ++j) mine_sum[j] += more[j];
+        }
+#pragma unroll
+        for (int j = 0; j < MT; ++j) part[stats_group * ROWS + r * MT + j] = mine_sum[j];
     }
     __syncthreads();                                 // every wavefront is done with its staging space
-    float* red = reinterpret_cast<float*>(lds);      // [waves][NS][64 lanes][4]
+    float* red = reinterpret_cast<float*>(lds);      // [waves][TILES][64 lanes][4]
 #pragma unroll
-    for (int s = 0; s < NS; ++s) *reinterpret_cast<f32x4*>(red + ((wave * NS + s) * 64 + lane) * 4) = acc[s];
-    if (SCALED && threadIdx.x < 16) {
+    for (int s = 0; s < NS; ++s)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+            *reinterpret_cast<f32x4*>(red + ((wave * TILES + s * MT + mt) * 64 + lane) * 4) = acc[s][mt];
+    if (SCALED && threadIdx.x < ROWS) {
         float sum = 0.f;
-        for (int i = threadIdx.x; i < (int)blockDim.x; i += 16) sum += part[i];
+        for (int group = 0; group < stats_groups; ++group) sum += part[group * ROWS + threadIdx.x];
         row_scale[threadIdx.x] = 1.0f / sqrtf(sum / (float)K + eps);
     }
     __syncthreads();
     if (SWIGLU) {
         // gate and up rows interleaved in blocks of 16: strips 2p and 2p + 1 are gate and up of the same columns
         const int n_out = N / 2;
-        for (int idx = threadIdx.x; idx < (NS / 2) * 256; idx += blockDim.x) {
-            const int pair = idx >> 8, l = (idx >> 2) & 63, i = idx & 3;
+        for (int idx = threadIdx.x; idx < (NS / 2) * MT * 256; idx += blockDim.x) {
+            const int pair = idx / (MT * 256), rest = idx % (MT * 256);
+            const int mt = rest >> 8, l = (rest >> 2) & 63, i = rest & 3;
+            const int at_gate = ((2 * pair) * MT + mt) * 256 + (rest & 255);
+            const int at_up = ((2 * pair + 1) * MT + mt) * 256 + (rest & 255);
             float gate = 0.f, up = 0.f;
             for (int wv = 0; wv < waves; ++wv) {
-                gate += red[(wv * NS + 2 * pair) * 256 + (idx & 255)];
-                up += red[(wv * NS + 2 * pair + 1) * 256 + (idx & 255)];
+                gate += red[wv * TILES * 256 + at_gate];
+                up += red[wv * TILES * 256 + at_up];
             }
-            const int n = n0 / 2 + pair * 16 + (l >> 4) * 4 + i, m = l & 15;
+            const int n = n0 / 2 + pair * 16 + (l >> 4) * 4 + i, m = mt * 16 + (l & 15);
             if (SCALED) {
                 gate *= row_scale[m];
                 up *= row_scale[m];
@@ -211,48 +236,66 @@ linear_fused_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, cons
         }
         return;
     }
-    // D[row = (lane / 16) * 4 + i][col = lane % 16]: element idx of strip s is column n0 + 16 s + (l / 16) * 4 + i
-    // of row l % 16 of x
-    for (int idx = threadIdx.x; idx < NS * 256; idx += blockDim.x) {
-        float sum = 0.f;
-        for (int wv = 0; wv < waves; ++wv) sum += red[wv * NS * 256 + idx];
-        const int s = idx >> 8, l = (idx >> 2) & 63, i = idx & 3;
-        const int n = n0 + s * 16 + (l >> 4) * 4 + i, m = l & 15;
+    // D[row = (lane / 16) * 4 + i][col = lane % 16]: lane l of tile (s, mt) holds the columns
+    // n0 + 16 s + (l / 16) * 4 .. + 3 of row 16 mt + l % 16 of x
+    for (int item = threadIdx.x; item < TILES * 64; item += blockDim.x) {
+        f32x4 sum = {0.f, 0.f, 0.f, 0.f};
+        for (int wv = 0; wv < waves; ++wv) sum += *reinterpret_cast<const f32x4*>(red + (wv * TILES * 64 + item) * 4);
+        const int tile = item >> 6, l = item & 63;
+        const int n = n0 + (tile / MT) * 16 + (l >> 4) * 4, m = (tile % MT) * 16 + (l & 15);
         float square = 0.f;
         if (SCALED) sum *= row_scale[m];
         if (n < N && m < M) {
-            if (bias) sum += bias[n];
+            if (bias) sum += load4(bias + n, n);
+            const int64_t at = (int64_t)m * N + n;
             if (MODE == FUSED_RESIDUAL) {
-                const float now = (one_pass ? h_before : h[(int64_t)m * N + n]) + sum;
-                h[(int64_t)m * N + n] = now;
-                if (xnext) xnext[(int64_t)m * N + n] = (bf16)(norm_w[n] * now);
-                square = now * now;
+                const f32x4 now = (one_pass ? h_before : load4(h + at, n)) + sum;
+                const f32x4 scaled = xnext ? load4(norm_w + n, n) * now : now;
+                if (whole) {
+                    *reinterpret_cast<f32x4*>(h + at) = now;
+                    if (xnext) {
+                        bf16x4 next;
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) next[i] = (bf16)scaled[i];
+                        *reinterpret_cast<bf16x4*>(xnext + at) = next;
+                    }
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        if (n + i >= N) continue;
+                        h[at + i] = now[i];
+                        if (xnext) xnext[at + i] = (bf16)scaled[i];
+                    }
+                }
+#pragma unroll
+                for (int i = 0; i < 4; ++i) square += n + i < N ? now[i] * now[i] : 0.f;
             } else {
-                out[(int64_t)m * N + n] = from_float<TO>(sum);
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    if (n + i < N) out[at + i] = from_float<TO>(sum[i]);
             }
         }
-        if (MODE == FUSED_RESIDUAL) red[idx] = square;     // only this thread read red[idx] of wavefront 0
+        if (MODE == FUSED_RESIDUAL) part[item] = square;
     }
     if (MODE == FUSED_RESIDUAL) {
         __syncthreads();
-        if (threadIdx.x < 16) {                      // row m: its squares over the workgroup's columns, in column order
-            const int m = threadIdx.x;
+        if (threadIdx.x < ROWS) {                    // a row's squares over the workgroup's columns, in column order
+            const int mt = threadIdx.x >> 4, rr = threadIdx.x & 15;
             float total = 0.f;
             for (int s = 0; s < NS; ++s)
-                for (int gg = 0; gg < 4; ++gg)
-                    for (int i = 0; i < 4; ++i) total += red[s * 256 + (gg * 16 + m) * 4 + i];
-            stats_out[blockIdx.x * 16 + m] = total;
+                for (int gg = 0; gg < 4; ++gg) total += part[(s * MT + mt) * 64 + gg * 16 + rr];
+            stats_out[blockIdx.x * ROWS + threadIdx.x] = total;
         }
     }
 }
 
-static size_t fused_lds(int strips, int waves) {
-    const size_t staging = (size_t)16 * (strips + 1) * FUSED_CK * 2, sums = (size_t)strips * 1024;
+static size_t fused_lds(int mt, int strips, int waves) {
+    const size_t staging = (size_t)16 * (strips + mt) * FUSED_CK * 2, sums = (size_t)strips * mt * 1024;
     return waves * (staging > sums ? staging : sums);
 }
 
-// The launch shape is linear_skinny.hip's for at most 16 rows: 8 wavefronts split K, two strips per
-// workgroup where that leaves a workgroup for most compute units (one for very few rows and very many columns).
+// The launch shape is linear_skinny.hip's: 8 wavefronts split K; two strips per workgroup where that leaves a
+// workgroup for most compute units (one for very few rows and very many columns).
 static int fused_strips(int M, int N, bool swiglu) {
     const int blocks16 = ceil_div(N, 16);
     int strips = 1;
@@ -268,30 +311,48 @@ static int fused_waves(int K) {
     return waves;
 }
 
+template <int MT, int NS, int MODE, typename TO, bool SW, bool TL>
+static void fused_launch_kernel(const void* x, const void* w, const float* bias, void* out, float* h,
+                                const float* norm_w, float eps, const float* stats_in, int stats_blocks,
+                                float* stats_out, void* xnext, int M, int N, int K, hipStream_t stream) {
+    const int waves = fused_waves(K);
+    const dim3 grid(ceil_div(N, 16 * NS)), block(waves * 64);
+    const size_t smem = fused_lds(MT, NS, waves);
+    if (smem > 64 * 1024)                            // beyond the default limit of dynamic LDS
+        (void)hipFuncSetAttribute((const void*)linear_fused_kernel<MT, NS, MODE, TO, SW, TL>,
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    hipLaunchKernelGGL((linear_fused_kernel<MT, NS, MODE, TO, SW, TL>), grid, block, smem, stream, (const bf16*)x,
+                       (const bf16*)w, bias, (TO*)out, h, norm_w, eps, stats_in, stats_blocks, stats_out, (bf16*)xnext,
+                       M, N, K);
+}
+
 template <int NS, int MODE, typename TO, bool SW>
 static int fused_launch(const void* x, const void* w, const float* bias, void* out, float* h, const float* norm_w,
                         float eps, const float* stats_in, int stats_blocks, float* stats_out, void* xnext, int M, int N,
                         int K, hipStream_t stream) {
-    const int waves = fused_waves(K);
-    const dim3 grid(ceil_div(N, 16 * NS)), block(waves * 64);
-    const size_t smem = fused_lds(NS, waves);
-    if (K % FUSED_CK != 0)
-        hipLaunchKernelGGL((linear_fused_kernel<NS, MODE, TO, SW, true>), grid, block, smem, stream, (const bf16*)x,
-                           (const bf16*)w, bias, (TO*)out, h, norm_w, eps, stats_in, stats_blocks, stats_out, (bf16*)xnext,
-                           M, N, K);
-    else
-        hipLaunchKernelGGL((linear_fused_kernel<NS, MODE, TO, SW, false>), grid, block, smem, stream, (const bf16*)x,
-                           (const bf16*)w, bias, (TO*)out, h, norm_w, eps, stats_in, stats_blocks, stats_out, (bf16*)xnext,
-                           M, N, K);
+    const bool tail = K % FUSED_CK != 0;
+#define SOMI_FUSED(MT)                                                                                               \
+    if (tail) fused_launch_kernel<MT, NS, MODE, TO, SW, true>(x, w, bias, out, h, norm_w, eps, stats_in, stats_blocks,  \
+                                                              stats_out, xnext, M, N, K, stream);                   \
+    else fused_launch_kernel<MT, NS, MODE, TO, SW, false>(x, w, bias, out, h, norm_w, eps, stats_in, stats_blocks,     \
+                                                          stats_out, xnext, M, N, K, stream);                       \
+    break
+    switch (ceil_div(M, 16)) {
+        case 1: SOMI_FUSED(1);
+        case 2: SOMI_FUSED(2);
+        case 3: SOMI_FUSED(3);
+        default: SOMI_FUSED(4);
+    }
+#undef SOMI_FUSED
     SOMI_LAUNCH_CHECK("linear_fused");
     return 0;
 }
 
 static int fused_check(const void* x, const void* w, int M, int N, int K) {
     SOMI_REQUIRE(M >= 0 && N > 0 && K > 0, "linear_fused: bad sizes M=%d N=%d K=%d", M, N, K);
-    SOMI_REQUIRE(M <= 16, "linear_fused: at most 16 rows, got %d", M);
+    SOMI_REQUIRE(M <= 64, "linear_fused: at most 64 rows, got %d", M);
     SOMI_REQUIRE(K % 8 == 0, "linear_fused: K (%d) must be a multiple of 8", K);
-    SOMI_REQUIRE((int64_t)K * 4 * 64 < (int64_t)1 << 31, "linear_fused: K (%d) is too large", K);
+    SOMI_REQUIRE((int64_t)K * 2 * 64 < (int64_t)1 << 31, "linear_fused: K (%d) is too large", K);
     SOMI_REQUIRE(((uintptr_t)x % 16 == 0) && ((uintptr_t)w % 16 == 0), "linear_fused: x and w must be 16-byte aligned");
     return 0;
 }
@@ -300,9 +361,9 @@ static int fused_check(const void* x, const void* w, int M, int N, int K) {
 extern "C" int somi_linear_residual_blocks(int M, int N) { return ceil_div(N, 16 * fused_strips(M, N, false)); }
 
 // h[m, n] += x[m, :] . w[n, :] (+ bias[n]).  x: [M, K] bfloat16; w: [N, K] bfloat16; bias: [N] float32 or null;
-// h: [M, N] float32, in and out; stats: [somi_linear_residual_blocks(M, N)][16] float32, out: per workgroup and
-// row the sum of squares of the new h over the workgroup's columns (rows M..15: 0); xnext: [M, N] bfloat16, out,
-// = norm_w[n] * h[m, n] (norm_w: [N] float32), or null.  M <= 16.
+// h: [M, N] float32, in and out; stats: [somi_linear_residual_blocks(M, N)][16 ceil(M / 16)] float32, out: per
+// workgroup and row the sum of squares of the new h over the workgroup's columns (rows from M on: 0); xnext:
+// [M, N] bfloat16, out, = norm_w[n] * h[m, n] (norm_w: [N] float32), or null.  M <= 64.
 extern "C" int somi_linear_residual(const void* x, const void* w, const float* bias, float* h, float* stats,
                                     const float* norm_w, void* xnext, int M, int N, int K, hipStream_t stream) {
     if (fused_check(x, w, M, N, K)) return 1;
@@ -316,12 +377,12 @@ extern "C" int somi_linear_residual(const void* x, const void* w, const float* b
 
 // out = s * (x . w^T) (+ bias) with the row scales s[m] = 1 / sqrt(sum of stats[:, m] / K + eps), or with swiglu
 // (w: [2 I, K], gate and up rows interleaved in blocks of 16, no bias) out[m, i] = silu(s g) * (s u) for the gate
-// and up products g, u.  x: [M, K] bfloat16, the rows somi_linear_residual wrote as xnext; stats:
-// [stats_blocks][16] float32 from the same call; out: bfloat16.  M <= 16.
+// and up products g, u.  x: [M, K] bfloat16, the rows a product into the stream wrote as xnext; stats:
+// [stats_blocks][16 ceil(M / 16)] float32 from the same call; out: bfloat16.  M <= 64.
 extern "C" int somi_linear_scaled(const void* x, float eps, const float* stats, int stats_blocks, const void* w,
                                   const float* bias, void* out, int M, int N, int K, int swiglu, hipStream_t stream) {
     if (fused_check(x, w, M, N, K)) return 1;
-    SOMI_REQUIRE(stats && stats_blocks > 0, "linear_scaled: the row statistics are needed");
+    SOMI_REQUIRE(stats && stats_blocks > 0 && (uintptr_t)stats % 16 == 0, "linear_scaled: the row statistics are needed, 16-byte aligned");
     SOMI_REQUIRE(!swiglu || (N % 32 == 0 && bias == nullptr), "linear_scaled: the gated form needs whole pairs of strips and no bias");
     if (M == 0) return 0;
     const int strips = fused_strips(M, N, swiglu != 0);

@@ -29,6 +29,22 @@ def linear_swiglu(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
     return ops.linear_skinny_swiglu(x, weight)
 
 
+def linear_residual(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, h: torch.Tensor,
+                    next_norm_weight: torch.Tensor | None = None) -> tuple[torch.Tensor, torch.Tensor | None]:
+    """h += x @ weight.T (+ bias) in place, by the kernel that :func:`linear` would take for the sizes; see
+    :func:`ops.linear_residual`."""
+    mid = _mid_is_faster(x.shape[0], weight.shape[0], x.shape[1])
+    return ops.linear_residual(x, weight, bias, h, next_norm_weight, mid=mid)
+
+
+def linear_scaled(x: torch.Tensor, eps: float, stats: torch.Tensor, weight: torch.Tensor,
+                  bias: torch.Tensor | None = None, swiglu: bool = False) -> torch.Tensor:
+    """The product of rows that are still to be normed, by the kernel that :func:`linear` would take for the
+    sizes; see :func:`ops.linear_scaled`."""
+    mid = _mid_is_faster(x.shape[0], weight.shape[0], x.shape[1])
+    return ops.linear_scaled(x, eps, stats, weight, bias, swiglu, mid=mid)
+
+
 def linear(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None,
            out_dtype: torch.dtype | None = None, bias_lowp: torch.Tensor | None = None) -> torch.Tensor:
     """x @ weight.T (+ bias).

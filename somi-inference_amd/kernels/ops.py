@@ -294,57 +294,6 @@ def linear_skinny_swiglu(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
     return out
 
 
-FUSED_MAX_ROWS = 16       # what the products fused with the residual add and the norm take
-
-
-def linear_residual(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, h: torch.Tensor,
-                    next_norm_weight: torch.Tensor | None = None) -> tuple[torch.Tensor, torch.Tensor | None]:
-    """h += x @ weight.T (+ bias) in float32, in place, for at most 16 bfloat16 rows.  Returns the row statistics
-    ``[workgroups, 16]`` (per workgroup and row the sum of squares of the new h over the workgroup's columns) and,
-    with ``next_norm_weight``, the rows ``bfloat16(next_norm_weight * h)`` that :func:`linear_scaled` reads."""
-    _need(x, "linear input", torch.bfloat16)
-    m, k = x.shape
-    _need(weight, "linear weight", torch.bfloat16)
-    n = weight.shape[0]
-    if weight.shape[1] != k:
-        raise KernelError(f"linear: input has {k} features, weight expects {weight.shape[1]}")
-    if bias is not None:
-        _need(bias, "linear bias", torch.float32, (n,))
-    _need(h, "residual stream", torch.float32, (m, n))
-    lib = library()
-    stats = torch.empty((lib.somi_linear_residual_blocks(m, n), 16), dtype=torch.float32, device=x.device)
-    weighted = None
-    if next_norm_weight is not None:
-        _need(next_norm_weight, "norm weight", torch.float32, (n,))
-        weighted = torch.empty((m, n), dtype=torch.bfloat16, device=x.device)
-    _check(lib.somi_linear_residual(_ptr(x), _ptr(weight), _ptr(bias), _ptr(h), _ptr(stats), _ptr(next_norm_weight),
-                                    _ptr(weighted), m, n, k, _stream()))
-    return stats, weighted
-
-
-def linear_scaled(x: torch.Tensor, eps: float, stats: torch.Tensor, weight: torch.Tensor,
-                  bias: torch.Tensor | None = None, swiglu: bool = False) -> torch.Tensor:
-    """s * (x @ weight.T) (+ bias) -> bfloat16 with the row scales s = 1 / sqrt(stats.sum(0) / K + eps): the
-    product of RMS-normed rows when x holds ``norm_weight * h`` and stats the sums of squares of h, both from
-    :func:`linear_residual`.  At most 16 rows.  With ``swiglu`` weight is [2 I, K] with gate and up rows
-    interleaved in blocks of 16 and the result is silu(s g) * (s u) for the gate and up products g, u."""
-    _need(x, "linear input", torch.bfloat16)
-    m, k = x.shape
-    _need(weight, "linear weight", torch.bfloat16)
-    n = weight.shape[0]
-    if weight.shape[1] != k or (swiglu and n % 32):
-        raise KernelError(f"linear_scaled: weight {tuple(weight.shape)} does not fit input width {k}")
-    if bias is not None:
-        _need(bias, "linear bias", torch.float32, (n,))
-    _need(stats, "row statistics", torch.float32)
-    if stats.dim() != 2 or stats.shape[1] != 16:
-        raise KernelError(f"linear_scaled: row statistics must be [blocks, 16], got {tuple(stats.shape)}")
-    out = torch.empty((m, n // 2 if swiglu else n), dtype=torch.bfloat16, device=x.device)
-    _check(library().somi_linear_scaled(_ptr(x), ctypes.c_float(eps), _ptr(stats), stats.shape[0], _ptr(weight),
-                                        _ptr(bias), _ptr(out), m, n, k, 1 if swiglu else 0, _stream()))
-    return out
-
-
 MID_WORKSPACE_FLOATS = 8 << 20        # 32 MB per device: partial sums of a split K (the kernel splits less if it is short)
 _mid_workspaces: dict[torch.device, torch.Tensor] = {}
 
@@ -355,6 +304,77 @@ def _mid_workspace(device: torch.device) -> torch.Tensor:
     if held is None:
         held = _mid_workspaces[device] = torch.empty((MID_WORKSPACE_FLOATS,), dtype=torch.float32, device=device)
     return held
+
+
+FUSED_MAX_ROWS = 64       # what the products fused with the residual add and the norm take
+
+
+def _stats_width(rows: int) -> int:
+    return 16 * ((rows + 15) // 16)
+
+
+def linear_residual(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, h: torch.Tensor,
+                    next_norm_weight: torch.Tensor | None = None, mid: bool = False
+                    ) -> tuple[torch.Tensor, torch.Tensor | None]:
+    """h += x @ weight.T (+ bias) in float32, in place, for at most 64 bfloat16 rows.  Returns the row statistics
+    ``[workgroups, 16 ceil(M / 16)]`` (per workgroup and row the sum of squares of the new h over the workgroup's
+    columns) and, with ``next_norm_weight``, the rows ``bfloat16(next_norm_weight * h)`` that :func:`linear_scaled`
+    reads.  ``mid``: by the kernel that shares x inside a workgroup and splits K over workgroups."""
+    _need(x, "linear input", torch.bfloat16)
+    m, k = x.shape
+    _need(weight, "linear weight", torch.bfloat16)
+    n = weight.shape[0]
+    if weight.shape[1] != k:
+        raise KernelError(f"linear: input has {k} features, weight expects {weight.shape[1]}")
+    if bias is not None:
+        _need(bias, "linear bias", torch.float32, (n,))
+    _need(h, "residual stream", torch.float32, (m, n))
+    lib = library()
+    blocks = lib.somi_linear_mid_residual_tiles(m, n, k) if mid else lib.somi_linear_residual_blocks(m, n)
+    stats = torch.empty((blocks, _stats_width(m)), dtype=torch.float32, device=x.device)
+    weighted = None
+    if next_norm_weight is not None:
+        _need(next_norm_weight, "norm weight", torch.float32, (n,))
+        weighted = torch.empty((m, n), dtype=torch.bfloat16, device=x.device)
+    if mid:
+        workspace = _mid_workspace(x.device)
+        _check(lib.somi_linear_mid_residual(_ptr(x), _ptr(weight), _ptr(bias), _ptr(h), _ptr(stats),
+                                            _ptr(next_norm_weight), _ptr(weighted), m, n, k, _ptr(workspace),
+                                            ctypes.c_int64(workspace.numel()), _stream()))
+    else:
+        _check(lib.somi_linear_residual(_ptr(x), _ptr(weight), _ptr(bias), _ptr(h), _ptr(stats),
+                                        _ptr(next_norm_weight), _ptr(weighted), m, n, k, _stream()))
+    return stats, weighted
+
+
+def linear_scaled(x: torch.Tensor, eps: float, stats: torch.Tensor, weight: torch.Tensor,
+                  bias: torch.Tensor | None = None, swiglu: bool = False, mid: bool = False) -> torch.Tensor:
+    """s * (x @ weight.T) (+ bias) -> bfloat16 with the row scales s = 1 / sqrt(stats.sum(0) / K + eps): the
+    product of RMS-normed rows when x holds ``norm_weight * h`` and stats the sums of squares of h, both from
+    :func:`linear_residual`.  At most 64 rows.  With ``swiglu`` weight is [2 I, K] with gate and up rows
+    interleaved in blocks of 16 and the result is silu(s g) * (s u) for the gate and up products g, u.
+    ``mid``: by the kernel that shares x inside a workgroup and splits K over workgroups."""
+    _need(x, "linear input", torch.bfloat16)
+    m, k = x.shape
+    _need(weight, "linear weight", torch.bfloat16)
+    n = weight.shape[0]
+    if weight.shape[1] != k or (swiglu and n % 32):
+        raise KernelError(f"linear_scaled: weight {tuple(weight.shape)} does not fit input width {k}")
+    if bias is not None:
+        _need(bias, "linear bias", torch.float32, (n,))
+    _need(stats, "row statistics", torch.float32)
+    if stats.dim() != 2 or stats.shape[1] != _stats_width(m):
+        raise KernelError(f"linear_scaled: row statistics must be [blocks, {_stats_width(m)}], got {tuple(stats.shape)}")
+    out = torch.empty((m, n // 2 if swiglu else n), dtype=torch.bfloat16, device=x.device)
+    if mid:
+        workspace = _mid_workspace(x.device)
+        _check(library().somi_linear_mid_scaled(_ptr(x), ctypes.c_float(eps), _ptr(stats), stats.shape[0],
+                                                _ptr(weight), _ptr(bias), _ptr(out), m, n, k, 1 if swiglu else 0,
+                                                _ptr(workspace), ctypes.c_int64(workspace.numel()), _stream()))
+    else:
+        _check(library().somi_linear_scaled(_ptr(x), ctypes.c_float(eps), _ptr(stats), stats.shape[0], _ptr(weight),
+                                            _ptr(bias), _ptr(out), m, n, k, 1 if swiglu else 0, _stream()))
+    return out
 
 
 def linear_mid(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None,

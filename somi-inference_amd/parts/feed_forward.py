@@ -50,8 +50,8 @@ class SwiGLU(FeedForward):
         if isinstance(x, NormedRows):
             if self.interleaved and self.gate_up.fusable(x.h.shape[0]):
                 # norm, gate_up and SiLU . up in one kernel
-                return self.down.deferred(ops.linear_scaled(x.weighted, x.norm.eps, x.stats, self.gate_up.weight,
-                                                            swiglu=True))
+                return self.down.deferred(linear_kernels.linear_scaled(x.weighted, x.norm.eps, x.stats,
+                                                                       self.gate_up.weight, swiglu=True))
             x = x.materialize()
         if not self.interleaved:
             return self.down.deferred(ops.silu_mul(self.gate_up(x)))

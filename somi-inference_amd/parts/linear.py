@@ -41,7 +41,7 @@ class DeferredProduct:
     def add_to(self, h: torch.Tensor, next_norm=None) -> "NormedRows | None":
         """h += the product, in place.  With the norm that follows, returns its rows, still to be normed."""
         weight = next_norm.weight if next_norm is not None else None
-        stats, weighted = ops.linear_residual(self.x, self.projection.weight, self.projection.bias, h, weight)
+        stats, weighted = linear_kernels.linear_residual(self.x, self.projection.weight, self.projection.bias, h, weight)
         return NormedRows(h, weighted, stats, next_norm) if next_norm is not None else None
 
 
@@ -68,7 +68,7 @@ class Projection:
     def __call__(self, x: "torch.Tensor | NormedRows", out_dtype: torch.dtype | None = None) -> torch.Tensor:
         if isinstance(x, NormedRows):
             if out_dtype in (None, torch.bfloat16) and self.fusable(x.h.shape[0]):
-                return ops.linear_scaled(x.weighted, x.norm.eps, x.stats, self.weight, self.bias)
+                return linear_kernels.linear_scaled(x.weighted, x.norm.eps, x.stats, self.weight, self.bias)
             x = x.materialize()
         return linear_kernels.linear(x, self.weight, self.bias, out_dtype, self.bias_lowp)
 

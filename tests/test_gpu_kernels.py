@@ -408,8 +408,11 @@ def test_linear_mid_with_the_gate_fused_in(m, inter, k):
     torch.testing.assert_close(got.float(), ops.linear_skinny_swiglu(x, merged).float(), atol=scale * 2 ** -7, rtol=2 ** -6)
 
 
-@pytest.mark.parametrize("m, hidden, n_out, inter", [(1, 64, 72, 48), (8, 3584, 4608, 256), (16, 200, 33, 160), (5, 1000, 503, 96)])
-def test_products_fused_with_the_residual_add_and_the_norm(m, hidden, n_out, inter):
+@pytest.mark.parametrize("mid", [False, True], ids=["skinny", "mid"])
+@pytest.mark.parametrize("m, hidden, n_out, inter", [(1, 64, 72, 48), (8, 3584, 4608, 256), (16, 200, 33, 160), (5, 1000, 503, 96),
+                                                     (17, 1000, 503, 96), (40, 200, 33, 160), (33, 520, 1056, 4112),
+                                                     (64, 3584, 4608, 1024), (48, 1536, 256, 18944)])
+def test_products_fused_with_the_residual_add_and_the_norm(m, hidden, n_out, inter, mid):
     """h += x.W1^T (+ b) with the rows' sums of squares and the next norm's weighted rows as by-products, then
     rmsnorm(h).W2^T as the product of those rows scaled per row: against float32 formulas and against the
     unfused kernels (norm, then product)."""
@@ -420,31 +423,32 @@ def test_products_fused_with_the_residual_add_and_the_norm(m, hidden, n_out, int
     norm_w = 1.0 + rnd(hidden, seed=5, scale=0.1)
     want_h = h + F.linear(x.float(), w1.float(), b1)
     got_h = h.clone()
-    stats, weighted = ops.linear_residual(x, w1, b1, got_h, norm_w)
+    stats, weighted = ops.linear_residual(x, w1, b1, got_h, norm_w, mid=mid)
     torch.testing.assert_close(got_h, want_h, atol=2e-5 * float(want_h.abs().max()) * math.sqrt(inter), rtol=1e-5)
-    assert stats.shape[1] == 16 and float(stats[:, m:].abs().max() if m < 16 else 0.0) == 0.0
+    width = 16 * ((m + 15) // 16)
+    assert stats.shape[1] == width and float(stats[:, m:].abs().max() if m < width else 0.0) == 0.0
     torch.testing.assert_close(stats.sum(dim=0)[:m], got_h.pow(2).sum(dim=1), rtol=1e-5, atol=1e-6)
     assert torch.equal(weighted, (norm_w * got_h).to(torch.bfloat16))
     no_bias = h.clone()
-    assert ops.linear_residual(x, w1, None, no_bias)[1] is None
+    assert ops.linear_residual(x, w1, None, no_bias, mid=mid)[1] is None
     torch.testing.assert_close(no_bias, h + F.linear(x.float(), w1.float()), atol=2e-5 * float(want_h.abs().max()) * math.sqrt(inter), rtol=1e-5)
 
     w2, b2 = rnd(n_out, hidden, dtype="bfloat16", seed=6, scale=0.05), rnd(n_out, seed=7)
     normed = ops.rmsnorm(got_h, norm_w, eps, torch.bfloat16)                      # the unfused way
     unfused = ops.linear_skinny(normed, w2, b2)
-    fused = ops.linear_scaled(weighted, eps, stats, w2, b2)
+    fused = ops.linear_scaled(weighted, eps, stats, w2, b2, mid=mid)
     want = F.linear(plain_rms(got_h, norm_w, eps), w2.float(), b2)               # float32 throughout
     scale = float(want.abs().max())
     torch.testing.assert_close(fused.float(), want, atol=scale * 2 ** -6, rtol=2 ** -6)
     torch.testing.assert_close(fused.float(), unfused.float(), atol=scale * 2 ** -6, rtol=2 ** -6)
     gate, up = rnd(inter, hidden, dtype="bfloat16", seed=8, scale=0.1), rnd(inter, hidden, dtype="bfloat16", seed=9, scale=0.1)
     merged = torch.stack([gate.view(-1, 16, hidden), up.view(-1, 16, hidden)], dim=1).reshape(-1, hidden).contiguous()
-    gated = ops.linear_scaled(weighted, eps, stats, merged, swiglu=True)
+    gated = ops.linear_scaled(weighted, eps, stats, merged, swiglu=True, mid=mid)
     exact = plain_rms(got_h, norm_w, eps)
     want_gated = F.silu(exact @ gate.float().t()) * (exact @ up.float().t())
     torch.testing.assert_close(gated.float(), want_gated, atol=float(want_gated.abs().max()) * 2 ** -5, rtol=2 ** -5)
-    with pytest.raises(KernelError, match="16 rows"):
-        ops.linear_residual(rnd(17, inter, dtype="bfloat16"), w1, None, rnd(17, hidden))
+    with pytest.raises(KernelError, match="64 rows"):
+        ops.linear_residual(rnd(65, inter, dtype="bfloat16"), w1, None, rnd(65, hidden), mid=mid)
 
 
 def plain_rms(h, w, eps):

@@ -266,7 +266,8 @@ def test_rotary_part_offers_the_reference_table():
     assert inv_freq.cpu().tolist() == pytest.approx([1.0, 1e6 ** -0.25, 1e6 ** -0.5, 1e6 ** -0.75], rel=1e-6)
 
 
-def test_a_few_bfloat16_rows_take_the_add_and_the_norm_inside_the_products():
+@pytest.mark.parametrize("n_rows", [7, 40, 64])
+def test_a_few_bfloat16_rows_take_the_add_and_the_norm_inside_the_products(n_rows):
     """Decode-sized steps in bfloat16: a block's last projections arrive at the residual stream uncomputed and are
     added to it by the kernel that computes them; the next norm is applied by the projection that reads the
     rows.  The stream ends up where separate add and norm kernels put it (up to the rounding of the deltas to
@@ -277,10 +278,10 @@ def test_a_few_bfloat16_rows_take_the_add_and_the_norm_inside_the_products():
     w = load_random(ffn, "bfloat16", scale=4.0)
     norm = RMSNorm("n", hidden_size=hidden, eps=1e-5)
     wn = load_random(norm, "bfloat16")
-    h0 = torch.randn(7, hidden, device=DEV)
+    h0 = torch.randn(n_rows, hidden, device=DEV)
     x = norm.forward(h0)
     out = ffn.forward(x)
-    assert isinstance(out, DeferredProduct) and out.shape == (7, hidden)
+    assert isinstance(out, DeferredProduct) and out.shape == (n_rows, hidden)
     # the fused way through the stream
     stream = ResidualStream(h0.clone())
     stream.add(out)
@@ -308,7 +309,7 @@ def test_a_few_bfloat16_rows_take_the_add_and_the_norm_inside_the_products():
     h2 = h1 + plain.swiglu(x2_plain, w["m.gate_proj.weight"], w["m.up_proj.weight"], w["m.down_proj.weight"])
     close(fused, h2, "bfloat16")
     # many rows, or float32, stay with the separate kernels
-    assert torch.is_tensor(ffn.forward(torch.randn(40, hidden, device=DEV).to(torch.bfloat16)))
+    assert torch.is_tensor(ffn.forward(torch.randn(70, hidden, device=DEV).to(torch.bfloat16)))
     ffn32 = SwiGLU("m", hidden_size=hidden, intermediate_size=inter)
     load_random(ffn32, "float32")
     assert torch.is_tensor(ffn32.forward(torch.randn(7, hidden, device=DEV)))
