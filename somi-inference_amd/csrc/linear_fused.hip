@@ -11,11 +11,16 @@
 //     from the producer's partial sums, added in workgroup order (a fixed order), and is applied to the
 //     float32 sums (before the bias, before SiLU in the gated form).
 //
+// A third form is the q/k/v product whose end also applies the rotary position encoding to q and k and stores
+// k and v in their cache pages (what rope_kv.hip does in a kernel of its own): a workgroup then owns the two
+// 16-column strips of a head that are rotated together, columns j and j + D/2, instead of 32 neighbours.
+//
 // Against norm.hip the only difference is where the rounding to bfloat16 happens: on weight * h instead
 // of weight * h * s (the same relative error; bfloat16 has float32's range, so the unscaled rows fit).
 //
 // Reference: somi_inference/models/qwen2.py:55-62 (RMSNorm), :333-339 (h = h + attn(norm(h)); h = h +
-// mlp(norm(h))), :209-229 (gate_up with SiLU).  The streaming of w (coalesced buffer loads, two chunks in
+// mlp(norm(h))), :209-229 (gate_up with SiLU), :95-113 and :286-293 (rotation of q and k), core/paged_attention.py:
+// 246-292 (k and v of a token land in its page).  The streaming of w (coalesced buffer loads, two chunks in
 // flight, a wavefront-private swizzled LDS tile, K split over the wavefronts, sums joined through LDS in
 // wavefront order) is that of linear_skinny.hip.
 #include "common.h"
@@ -32,12 +37,22 @@ typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
 #define FUSED_SCALED 1
 #define FUSED_RESIDUAL 2
 
-template <int MT, int NS, int MODE, typename TO, bool SWIGLU, bool TAIL>
+// What the q/k/v product needs to rotate q and k and to store k and v (the arguments of rope_kv.hip).
+struct FusedRope {
+    const int* positions;     // [M]
+    const int* slots;         // [M]: page * page_size + offset of the token's k and v, or -1 for no store
+    const float* inv_freq;    // [D / 2]
+    bf16* k_cache;            // [pages, nkv, page_size, D]
+    bf16* v_cache;            // [pages, nkv, D, page_size]
+    int nq, nkv, D, page_size;
+};
+
+template <int MT, int NS, int MODE, typename TO, bool SWIGLU, bool TAIL, bool ROPE = false>
 __global__ void __launch_bounds__(FUSED_MAX_WAVES * 64)
 linear_fused_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, const float* __restrict__ bias,
                     TO* __restrict__ out, float* __restrict__ h, const float* __restrict__ norm_w, float eps,
                     const float* __restrict__ stats_in, int stats_blocks, float* __restrict__ stats_out,
-                    bf16* __restrict__ xnext, int M, int N, int K) {
+                    bf16* __restrict__ xnext, int M, int N, int K, FusedRope rope) {
     extern __shared__ __attribute__((aligned(16))) char lds[];
     __shared__ float row_scale[64];
     __shared__ float part[FUSED_MAX_WAVES * 4 * 16 * MT];
@@ -51,10 +66,14 @@ linear_fused_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, cons
     const int waves = blockDim.x >> 6;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int r = lane & 15, g = lane >> 4;
-    const int n0 = blockIdx.x * (16 * NS);
+    // with the rotation, workgroup b owns the columns j .. j + 15 and j + D/2 .. of head b / (D / 32)
+    const int rope_blocks = ROPE ? rope.D / 32 : 1;
+    const int rope_head = blockIdx.x / rope_blocks, rope_j = (blockIdx.x % rope_blocks) * 16;
+    const int n0 = ROPE ? rope_head * rope.D + rope_j : blockIdx.x * (16 * NS);
+    const int strip_step = ROPE ? rope.D / 2 : 16;           // rows of w from one strip to the next
     char* mine = lds + wave * WAVE_BYTES;
 
-    const int rows_here = min(16 * NS, N - n0);
+    const int rows_here = ROPE ? N - n0 : min(16 * NS, N - n0);
     const __amdgpu_buffer_rsrc_t wres = __builtin_amdgcn_make_buffer_rsrc(
         (void*)(w + (int64_t)n0 * K), 0, (int)((int64_t)rows_here * K * 2), SOMI_BUFFER_WORD3);
     const __amdgpu_buffer_rsrc_t xres = __builtin_amdgcn_make_buffer_rsrc(
@@ -68,7 +87,7 @@ linear_fused_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, cons
 #pragma unroll
     for (int i = 0; i < NL; ++i) {
         const int tile = i / 2, row16 = (i % 2) * 8 + (lane >> 3);
-        const int row = tile < NS ? tile * 16 + row16 : (tile - NS) * 16 + row16;
+        const int row = tile < NS ? tile * strip_step + row16 : (tile - NS) * 16 + row16;
         goff[i] = ((unsigned)row * (unsigned)K + lchunk * 8) * 2u;
         soff[i] = (tile * 16 + row16) * ROW_BYTES + ((lchunk ^ swizzle(row16)) << 4);
     }
@@ -214,6 +233,70 @@ linear_fused_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, cons
         row_scale[threadIdx.x] = 1.0f / sqrtf(sum / (float)K + eps);
     }
     __syncthreads();
+    if constexpr (ROPE) {
+        // lane l of row tile mt holds the channels j .. j + 3 (j = rope_j + (l / 16) * 4) of row 16 mt + l % 16 in the
+        // first strip and the channels they are rotated with, j + D/2 .., in the second
+        const int D = rope.D, nq = rope.nq, nkv = rope.nkv;
+        for (int item = threadIdx.x; item < MT * 64; item += blockDim.x) {
+            const int mt = item >> 6, l = item & 63, m = mt * 16 + (l & 15), j = rope_j + (l >> 4) * 4;
+            f32x4 lo = {0.f, 0.f, 0.f, 0.f}, hi = lo;
+            for (int wv = 0; wv < waves; ++wv) {
+                lo += *reinterpret_cast<const f32x4*>(red + ((wv * TILES + mt) * 64 + l) * 4);
+                hi += *reinterpret_cast<const f32x4*>(red + ((wv * TILES + MT + mt) * 64 + l) * 4);
+            }
+            if (m >= M) continue;
+            if (SCALED) {
+                lo *= row_scale[m];
+                hi *= row_scale[m];
+            }
+            if (bias) {
+                lo += load4(bias + rope_head * D + j, 0);
+                hi += load4(bias + rope_head * D + D / 2 + j, 0);
+            }
+            bf16x4 first, second;
+            if (rope_head < nq + nkv) {                    // q and k heads: x' = x cos + rotate_half(x) sin
+                const float pos = (float)rope.positions[m];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    // the product is rounded to bfloat16 before it is rotated, as where the rotation is a kernel
+                    // of its own: k in the cache does not depend on which of the two wrote it
+                    const float x1 = to_float((bf16)lo[i]), x2 = to_float((bf16)hi[i]);
+                    const float angle = pos * rope.inv_freq[j + i];
+                    const float c = cosf(angle), sn = sinf(angle);
+                    first[i] = (bf16)(x1 * c - x2 * sn);
+                    second[i] = (bf16)(x2 * c + x1 * sn);
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    first[i] = (bf16)lo[i];
+                    second[i] = (bf16)hi[i];
+                }
+            }
+            if (rope_head < nq) {
+                bf16* to = reinterpret_cast<bf16*>(out) + (int64_t)m * nq * D + rope_head * D + j;
+                *reinterpret_cast<bf16x4*>(to) = first;
+                *reinterpret_cast<bf16x4*>(to + D / 2) = second;
+                continue;
+            }
+            const int slot = rope.slots[m];
+            if (slot < 0) continue;
+            const int64_t page = slot / rope.page_size, off = slot % rope.page_size;
+            if (rope_head < nq + nkv) {
+                bf16* to = rope.k_cache + ((page * nkv + (rope_head - nq)) * rope.page_size + off) * D + j;
+                *reinterpret_cast<bf16x4*>(to) = first;
+                *reinterpret_cast<bf16x4*>(to + D / 2) = second;
+            } else {                                       // v is kept transposed inside a page
+                bf16* to = rope.v_cache + ((page * nkv + (rope_head - nq - nkv)) * D + j) * rope.page_size + off;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    to[(int64_t)i * rope.page_size] = first[i];
+                    to[(int64_t)(D / 2 + i) * rope.page_size] = second[i];
+                }
+            }
+        }
+        return;
+    }
     if (SWIGLU) {
         // gate and up rows interleaved in blocks of 16: strips 2p and 2p + 1 are gate and up of the same columns
         const int n_out = N / 2;
@@ -311,31 +394,33 @@ static int fused_waves(int K) {
     return waves;
 }
 
-template <int MT, int NS, int MODE, typename TO, bool SW, bool TL>
+template <int MT, int NS, int MODE, typename TO, bool SW, bool TL, bool ROPE>
 static void fused_launch_kernel(const void* x, const void* w, const float* bias, void* out, float* h,
                                 const float* norm_w, float eps, const float* stats_in, int stats_blocks,
-                                float* stats_out, void* xnext, int M, int N, int K, hipStream_t stream) {
+                                float* stats_out, void* xnext, int M, int N, int K, const FusedRope& rope,
+                                hipStream_t stream) {
     const int waves = fused_waves(K);
-    const dim3 grid(ceil_div(N, 16 * NS)), block(waves * 64);
+    const dim3 grid(ROPE ? (rope.nq + 2 * rope.nkv) * (rope.D / 32) : ceil_div(N, 16 * NS)), block(waves * 64);
     const size_t smem = fused_lds(MT, NS, waves);
     if (smem > 64 * 1024)                            // beyond the default limit of dynamic LDS
-        (void)hipFuncSetAttribute((const void*)linear_fused_kernel<MT, NS, MODE, TO, SW, TL>,
+        (void)hipFuncSetAttribute((const void*)linear_fused_kernel<MT, NS, MODE, TO, SW, TL, ROPE>,
                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-    hipLaunchKernelGGL((linear_fused_kernel<MT, NS, MODE, TO, SW, TL>), grid, block, smem, stream, (const bf16*)x,
-                       (const bf16*)w, bias, (TO*)out, h, norm_w, eps, stats_in, stats_blocks, stats_out, (bf16*)xnext,
-                       M, N, K);
+    hipLaunchKernelGGL((linear_fused_kernel<MT, NS, MODE, TO, SW, TL, ROPE>), grid, block, smem, stream,
+                       (const bf16*)x, (const bf16*)w, bias, (TO*)out, h, norm_w, eps, stats_in, stats_blocks, stats_out,
+                       (bf16*)xnext, M, N, K, rope);
 }
 
-template <int NS, int MODE, typename TO, bool SW>
+template <int NS, int MODE, typename TO, bool SW, bool ROPE = false>
 static int fused_launch(const void* x, const void* w, const float* bias, void* out, float* h, const float* norm_w,
                         float eps, const float* stats_in, int stats_blocks, float* stats_out, void* xnext, int M, int N,
-                        int K, hipStream_t stream) {
+                        int K, hipStream_t stream, const FusedRope& rope = FusedRope{}) {
     const bool tail = K % FUSED_CK != 0;
 #define SOMI_FUSED(MT)                                                                                               \
-    if (tail) fused_launch_kernel<MT, NS, MODE, TO, SW, true>(x, w, bias, out, h, norm_w, eps, stats_in, stats_blocks,  \
-                                                              stats_out, xnext, M, N, K, stream);                   \
-    else fused_launch_kernel<MT, NS, MODE, TO, SW, false>(x, w, bias, out, h, norm_w, eps, stats_in, stats_blocks,     \
-                                                          stats_out, xnext, M, N, K, stream);                       \
+    if (tail) fused_launch_kernel<MT, NS, MODE, TO, SW, true, ROPE>(x, w, bias, out, h, norm_w, eps, stats_in,          \
+                                                                    stats_blocks, stats_out, xnext, M, N, K, rope,    \
+                                                                    stream);                                          \
+    else fused_launch_kernel<MT, NS, MODE, TO, SW, false, ROPE>(x, w, bias, out, h, norm_w, eps, stats_in,             \
+                                                                stats_blocks, stats_out, xnext, M, N, K, rope, stream); \
     break
     switch (ceil_div(M, 16)) {
         case 1: SOMI_FUSED(1);
@@ -391,4 +476,33 @@ extern "C" int somi_linear_scaled(const void* x, float eps, const float* stats, 
     if (strips >= 2)
         return fused_launch<2, FUSED_SCALED, bf16, false>(x, w, bias, out, nullptr, nullptr, eps, stats, stats_blocks, nullptr, nullptr, M, N, K, stream);
     return fused_launch<1, FUSED_SCALED, bf16, false>(x, w, bias, out, nullptr, nullptr, eps, stats, stats_blocks, nullptr, nullptr, M, N, K, stream);
+}
+
+// The q/k/v product with the rotary encoding and the cache store in its end.  x: [M, K] bfloat16; w:
+// [(nq + 2 nkv) D, K] bfloat16, the rows of the q heads, then the k heads, then the v heads; bias: float32 or
+// null.  With stats (from a product into the stream, see somi_linear_scaled) the sums are scaled per row
+// first; with stats == null x is used as it is.  q: [M, nq D] bfloat16, out, rotated; k (rotated) and v go to
+// their pages: k_cache [pages, nkv, page_size, D], v_cache [pages, nkv, D, page_size], slot of row m =
+// page * page_size + offset or -1.  positions: [M] int32; inv_freq: [D / 2] float32 (the whole head is
+// rotated).  D must be a multiple of 32, M <= 64.
+extern "C" int somi_linear_rope_store(const void* x, float eps, const float* stats, int stats_blocks, const void* w,
+                                      const float* bias, void* q, const int* positions, const int* slots,
+                                      const float* inv_freq, void* k_cache, void* v_cache, int nq, int nkv, int D,
+                                      int page_size, int M, int K, hipStream_t stream) {
+    SOMI_REQUIRE(nq > 0 && nkv > 0 && D > 0 && D % 32 == 0, "linear_rope_store: head_dim (%d) must be a multiple of 32", D);
+    const int64_t columns = (int64_t)(nq + 2 * nkv) * D;
+    SOMI_REQUIRE(columns * K * 2 < (int64_t)1 << 31, "linear_rope_store: the weight is too large");
+    const int N = (int)columns;
+    if (fused_check(x, w, M, N, K)) return 1;
+    SOMI_REQUIRE(q && positions && slots && inv_freq && k_cache && v_cache && page_size > 0,
+                 "linear_rope_store: q, positions, slots, inv_freq and the caches are needed");
+    SOMI_REQUIRE((uintptr_t)q % 8 == 0 && (uintptr_t)k_cache % 8 == 0, "linear_rope_store: q and the k cache must be 8-byte aligned");
+    SOMI_REQUIRE(!stats || (stats_blocks > 0 && (uintptr_t)stats % 16 == 0), "linear_rope_store: bad row statistics");
+    if (M == 0) return 0;
+    const FusedRope rope{positions, slots, inv_freq, (bf16*)k_cache, (bf16*)v_cache, nq, nkv, D, page_size};
+    if (stats)
+        return fused_launch<2, FUSED_SCALED, bf16, false, true>(x, w, bias, q, nullptr, nullptr, eps, stats, stats_blocks,
+                                                                nullptr, nullptr, M, N, K, stream, rope);
+    return fused_launch<2, 0, bf16, false, true>(x, w, bias, q, nullptr, nullptr, 0.f, nullptr, 0, nullptr, nullptr, M, N, K,
+                                                 stream, rope);
 }

@@ -377,6 +377,38 @@ def linear_scaled(x: torch.Tensor, eps: float, stats: torch.Tensor, weight: torc
     return out
 
 
+def linear_rope_store(x: torch.Tensor, eps: float, stats: torch.Tensor | None, weight: torch.Tensor,
+                      bias: torch.Tensor | None, positions: torch.Tensor, slots: torch.Tensor, inv_freq: torch.Tensor,
+                      nq: int, nkv: int, head_dim: int, k_cache: torch.Tensor, v_cache: torch.Tensor) -> torch.Tensor:
+    """The q/k/v product of at most 64 bfloat16 rows with the rotary encoding of q and k and the store of k and v
+    into their cache pages in its end -> q [M, nq * D], rotated.  weight: [(nq + 2 nkv) * D, K], q heads, k
+    heads, v heads.  With ``stats`` x holds ``norm_weight * h`` and the sums are scaled per row as in
+    :func:`linear_scaled`; without, x is used as it is.  The whole head is rotated (inv_freq: [D / 2]); D must be
+    a multiple of 32."""
+    _need(x, "linear input", torch.bfloat16)
+    m, k = x.shape
+    _need(weight, "q/k/v weight", torch.bfloat16, ((nq + 2 * nkv) * head_dim, k))
+    if bias is not None:
+        _need(bias, "q/k/v bias", torch.float32, (weight.shape[0],))
+    if stats is not None:
+        _need(stats, "row statistics", torch.float32)
+        if stats.dim() != 2 or stats.shape[1] != _stats_width(m):
+            raise KernelError(f"linear_rope_store: row statistics must be [blocks, {_stats_width(m)}], got {tuple(stats.shape)}")
+    _need(positions, "positions", torch.int32, (m,))
+    _need(slots, "slot mapping", torch.int32, (m,))
+    _need(inv_freq, "inv_freq", torch.float32, (head_dim // 2,))
+    _need(k_cache, "k cache", torch.bfloat16)
+    if k_cache.dim() != 4 or k_cache.shape[1] != nkv or k_cache.shape[3] != head_dim:
+        raise KernelError(f"linear_rope_store: cache shape {tuple(k_cache.shape)} != [pages, {nkv}, page, {head_dim}]")
+    _need(v_cache, "v cache", torch.bfloat16, _v_shape(k_cache))
+    q = torch.empty((m, nq * head_dim), dtype=torch.bfloat16, device=x.device)
+    _check(library().somi_linear_rope_store(_ptr(x), ctypes.c_float(eps), _ptr(stats),
+                                            stats.shape[0] if stats is not None else 0, _ptr(weight), _ptr(bias),
+                                            _ptr(q), _ptr(positions), _ptr(slots), _ptr(inv_freq), _ptr(k_cache),
+                                            _ptr(v_cache), nq, nkv, head_dim, k_cache.shape[2], m, k, _stream()))
+    return q
+
+
 def linear_mid(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None,
                out_dtype: torch.dtype | None = None, swiglu: bool = False) -> torch.Tensor:
     """x @ weight.T (+ bias) for at most 64 bfloat16 rows, x shared by the wavefronts of a workgroup, K split

@@ -19,7 +19,7 @@ from ..kernels import attention as attention_kernels
 from ..kernels import ops
 from ..weights.spec import MATRIX, VECTOR, WeightSpec
 from .base import Fetch, LayerCache, Mixer, PagedKVSpec, PartSpec, Runtime
-from .linear import Projection
+from .linear import NormedRows, Projection
 from .registry import build_part
 
 
@@ -82,17 +82,39 @@ class GroupedQueryAttention(Mixer):
             raise ValueError(f"{self.prefix}: attention needs a paged cache")
         view = step.paged[cache.group]
         nkv_new = 0 if self.shares_cache else self.num_kv_heads
-        qkv = self.qkv(x)                                   # [N, (nq + 2 nkv) * D]
         rotation = self.position.rotation_table()
-        if rotation is None:
-            self.position.encode_qk(qkv, step, self.num_heads, nkv_new, self.head_dim)
-            inv_freq, rotary_dim = None, 0
-        else:
-            inv_freq, rotary_dim = rotation
-        ops.rope_kv_store(qkv, step.positions, view.slot_mapping if nkv_new else None, inv_freq, rotary_dim,
-                          self.num_heads, nkv_new, self.head_dim,
-                          cache.k if nkv_new else None, cache.v if nkv_new else None)
+        qkv = self._project_rotate_store(x, step, view, cache, rotation)     # a few rows: one kernel
+        if qkv is None:
+            qkv = self.qkv(x)                               # [N, (nq + 2 nkv) * D]
+            if rotation is None:
+                self.position.encode_qk(qkv, step, self.num_heads, nkv_new, self.head_dim)
+                inv_freq, rotary_dim = None, 0
+            else:
+                inv_freq, rotary_dim = rotation
+            ops.rope_kv_store(qkv, step.positions, view.slot_mapping if nkv_new else None, inv_freq, rotary_dim,
+                              self.num_heads, nkv_new, self.head_dim,
+                              cache.k if nkv_new else None, cache.v if nkv_new else None)
         attended = attention_kernels.paged_attention(
             qkv, self.num_heads, cache.k, cache.v, view.block_table, step,
             window=self.window or 0, scale=self.scale)
         return self.out.deferred(attended)        # the residual stream may add it in the kernel that computes it
+
+    def _project_rotate_store(self, x, step, view, cache: LayerCache, rotation) -> torch.Tensor | None:
+        """q of the step's tokens, rotated, with k and v in their pages, by the q/k/v product itself; None where
+        that kernel does not apply (many rows, float32, a head that is not rotated as a whole, no k/v of its own)."""
+        if rotation is None or self.shares_cache:
+            return None
+        inv_freq, rotary_dim = rotation
+        rows = x.shape[0]
+        if (rotary_dim != self.head_dim or self.head_dim % 32 or cache.k.dtype != torch.bfloat16
+                or not self.qkv.fusable(rows)):
+            return None
+        if isinstance(x, NormedRows):
+            weighted, eps, stats = x.weighted, x.norm.eps, x.stats
+        elif x.dtype == torch.bfloat16 and x.data_ptr() % 16 == 0:
+            weighted, eps, stats = x, 0.0, None
+        else:
+            return None
+        return ops.linear_rope_store(weighted, eps, stats, self.qkv.weight, self.qkv.bias, step.positions,
+                                     view.slot_mapping, inv_freq, self.num_heads, self.num_kv_heads, self.head_dim,
+                                     cache.k, cache.v)

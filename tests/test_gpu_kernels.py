@@ -451,5 +451,64 @@ def test_products_fused_with_the_residual_add_and_the_norm(m, hidden, n_out, int
         ops.linear_residual(rnd(65, inter, dtype="bfloat16"), w1, None, rnd(65, hidden), mid=mid)
 
 
+@pytest.mark.parametrize("scaled", [True, False], ids=["normed", "as-is"])
+@pytest.mark.parametrize("m, nq, nkv, d, hidden, page", [(1, 4, 2, 32, 64, 16), (9, 12, 2, 64, 200, 8), (16, 3, 3, 128, 520, 4),
+                                                         (37, 5, 1, 96, 1000, 16), (64, 28, 4, 128, 3584, 16)])
+def test_qkv_product_with_the_rotation_and_the_cache_store(m, nq, nkv, d, hidden, page, scaled):
+    """q/k/v projection, rotary encoding and cache write in one kernel: against the float32 formulas (norm as a
+    row scale, product, rotation) and against the three separate kernels."""
+    eps, theta, pages = 1e-5, 1e4, 12
+    n_out = (nq + 2 * nkv) * d
+    w, b = rnd(n_out, hidden, dtype="bfloat16", seed=2, scale=0.05), rnd(n_out, seed=3)
+    positions = i32([(7 * t * t + 3) % 5000 for t in range(m)])
+    slot_list = [(11 * t + 5) % (pages * page) for t in range(m)]            # distinct: 11 is coprime to the pool
+    assert len(set(slot_list)) == m
+    slot_list[m // 2] = -1 if m > 2 else slot_list[m // 2]                     # a token without a slot is not stored
+    slots = i32(slot_list)
+    inv_freq = plain.rope_inv_freq(d, theta).to(DEV)
+    if scaled:                                   # rows still to be normed, as a product into the stream leaves them
+        h = rnd(m, hidden, seed=4, scale=2.0)
+        norm_w = 1.0 + rnd(hidden, seed=5, scale=0.1)
+        x = (norm_w * h).to(torch.bfloat16)
+        stats = torch.zeros(3, 16 * ((m + 15) // 16), device=DEV)
+        stats[1, :m] = h.pow(2).sum(dim=1)
+        exact_x = x.float() * torch.rsqrt(h.pow(2).mean(dim=1, keepdim=True) + eps)
+    else:
+        x, stats = rnd(m, hidden, dtype="bfloat16", seed=4), None
+        exact_x = x.float()
+    kc = torch.zeros(pages, nkv, page, d, dtype=torch.bfloat16, device=DEV)
+    vc = torch.zeros(pages, nkv, d, page, dtype=torch.bfloat16, device=DEV)
+    q = ops.linear_rope_store(x, eps, stats, w, b, positions, slots, inv_freq, nq, nkv, d, kc, vc)
+    heads = F.linear(exact_x, w.float(), b).view(m, nq + 2 * nkv, d).cpu()
+    cos, sin = plain.rope_cos_sin(positions.cpu(), d, theta)
+    want_q = plain.apply_rope(heads[:, :nq].transpose(0, 1), cos, sin).transpose(0, 1)
+    want_k = plain.apply_rope(heads[:, nq:nq + nkv].transpose(0, 1), cos, sin).transpose(0, 1)
+    scale = float(heads.abs().max())
+    tol = dict(atol=scale * 2 ** -7, rtol=2 ** -7)
+    torch.testing.assert_close(q.float().view(m, nq, d).cpu(), want_q, **tol)
+    for t, slot in enumerate(slot_list):
+        if slot < 0:
+            continue
+        pg, off = divmod(slot, page)
+        torch.testing.assert_close(kc[pg, :, off].float().cpu(), want_k[t], **tol)
+        torch.testing.assert_close(vc[pg, :, :, off].float().cpu(), heads[t, nq + nkv:], **tol)
+    written = torch.zeros(pages * page, dtype=torch.bool)
+    written[[slot for slot in slot_list if slot >= 0]] = True
+    for cache in (kc.permute(0, 2, 1, 3), vc.permute(0, 3, 1, 2)):
+        untouched = cache.float().reshape(pages * page, -1).cpu()[~written]
+        assert float(untouched.abs().sum()) == 0.0, "a slot that was not addressed was written"
+    # the separate kernels: product (with the norm as a row scale), then rotation and store
+    kc2, vc2 = torch.zeros_like(kc), torch.zeros_like(vc)
+    qkv = ops.linear_scaled(x, eps, stats, w, b) if scaled else ops.linear_skinny(x, w, b)
+    ops.rope_kv_store(qkv, positions, slots, inv_freq, d, nq, nkv, d, kc2, vc2)
+    # the same sums in the same order, rounded at the same places: the same bits
+    assert torch.equal(q, qkv[:, :nq * d]) and torch.equal(kc, kc2) and torch.equal(vc, vc2)
+    with pytest.raises(KernelError, match="multiple of 32"):
+        ops.linear_rope_store(x, eps, stats, rnd(4 * 48, hidden, dtype="bfloat16"), None, positions, slots,
+                              plain.rope_inv_freq(48, theta).to(DEV), 2, 1, 48,
+                              torch.zeros(2, 1, page, 48, dtype=torch.bfloat16, device=DEV),
+                              torch.zeros(2, 1, 48, page, dtype=torch.bfloat16, device=DEV))
+
+
 def plain_rms(h, w, eps):
     return w * h * torch.rsqrt(h.pow(2).mean(dim=-1, keepdim=True) + eps)
