@@ -39,15 +39,28 @@ __device__ __forceinline__ bf16x8 pjoin(short4_t lo, short4_t hi) {
     return u.wide;
 }
 
+// Maxima of scores, which are never NaN (keys that must not be seen are -inf): the bare instructions, without
+// the quieting of signalling NaNs that fmaxf adds to each operand.
+__device__ __forceinline__ float max2(float a, float b) {
+    float r;
+    asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+    return r;
+}
+__device__ __forceinline__ float max3(float a, float b, float c) {
+    float r;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+
 // Maximum / sum over the four lane groups (lanes l, l ^ 16, l ^ 32, l ^ 48) with the row-swap instructions
 // of gfx950: v_permlane16_swap exchanges odd 16-lane rows of one operand with even rows of the other,
 // v_permlane32_swap the upper and lower halves; no LDS round trip.
 typedef __attribute__((ext_vector_type(2))) unsigned u32x2;
 __device__ __forceinline__ float group_max(float v) {
     u32x2 a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
-    v = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+    v = max2(__uint_as_float(a[0]), __uint_as_float(a[1]));
     u32x2 b = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
-    return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+    return max2(__uint_as_float(b[0]), __uint_as_float(b[1]));
 }
 __device__ __forceinline__ float group_sum(float v) {
     u32x2 a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
@@ -203,7 +216,8 @@ attention_prefill_kernel(const bf16* __restrict__ q, int64_t q_stride, const bf1
 // from LDS, then store it into the other LDS buffer; one barrier per step.  Every key and value is read
 // from L2/HBM once per 128 queries instead of once per wavefront.
 //   K tile in LDS: [32 keys][D + 8] (rows padded by 16 bytes: the 16 rows a 16-byte read touches fall into
-//   different banks); V tile: [D channels][32 + 4 keys].
+//   different banks); V tile: [D channels][32 + 8 keys] (a row is 20 dwords: the 32 lanes that an 8-byte
+//   read serves at once, 16 channels x 2 key groups, fall into different banks).
 #define PREFILL_LDS_PAGES 2048     // block-table entries of the visible range kept in LDS (else read from memory)
 #ifndef PREFILL_WIDE_GROUPS
 #define PREFILL_WIDE_GROUPS 768    // from this many 128-query groups on, workgroups take 128 queries, else 64
@@ -217,7 +231,7 @@ attention_prefill_lds_kernel(const bf16* __restrict__ q, int64_t q_stride, const
     constexpr int D = DT * 16;
     constexpr int QK_STEPS = (DT + 1) / 2;
     constexpr int QW = QB * 16, WAVES = 4, QG = WAVES * QW;             // 64 or 128 queries per workgroup
-    constexpr int KROW = D + 8, VROW = 32 + 4;                          // padded LDS rows, in elements
+    constexpr int KROW = D + 8, VROW = 32 + 8;                          // padded LDS rows, in elements
     constexpr int K_CHUNKS = 32 * D / 8;                                // 16-byte pieces of a key tile
     constexpr int K_PER_THREAD = (K_CHUNKS + 255) / 256;
     constexpr int V_PER_THREAD = (D + 31) / 32;                         // 8-byte pieces (4 keys of a channel): a
@@ -250,12 +264,20 @@ attention_prefill_lds_kernel(const bf16* __restrict__ q, int64_t q_stride, const
     // table read from memory before its own loads can start.
     // (power-of-two page size and at most PREFILL_LDS_PAGES pages in reach: the launcher's duty.  A read of
     // the table from memory inside the loop would make every tile wait for all loads issued before it.)
+    // The list covers the 32-key tiles whole: before the first visible key the table's own entries (pages that
+    // a window has released read as page 0), past the last one the last page again.  So every key of a tile
+    // has an address that may be read, and keys outside the visible range need no clamp: their scores are
+    // masked.
     const int shift = __builtin_ctz(page_size);
-    const int page_lo = lo >> shift, page_count = (wg_last >> shift) - page_lo + 1;
-    for (int i = tid; i < page_count; i += 256) pages[i] = table[page_lo + i];
+    const int page_lo = (lo & ~31) >> shift, page_last = wg_last >> shift;
+    const int page_count = (((wg_last | 31) >> shift) - page_lo) + 1;
+    for (int i = tid; i < page_count; i += 256) pages[i] = table[min(page_lo + i, page_last)];
     __syncthreads();
     auto page_of = [&](int pos) -> int64_t { return pages[(pos >> shift) - page_lo]; };
     auto page_offset = [&](int pos) { return pos & (page_size - 1); };
+    const int64_t page_stride = (int64_t)nkv * page_size * D;          // elements from one page to the next
+    const bf16* k_head = kc + (int64_t)kvh * page_size * D;
+    const bf16* v_head = vc + (int64_t)kvh * page_size * D;
 
     // this wavefront's queries
     const int q0 = g0 + wave * QW;
@@ -284,27 +306,25 @@ attention_prefill_lds_kernel(const bf16* __restrict__ q, int64_t q_stride, const
         for (int dt = 0; dt < DT; ++dt) acc[qb][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
 
-    // staging registers of the next tile
-    bf16x8 kreg[K_PER_THREAD];
-    short4_t vreg[V_PER_THREAD];
-    auto fetch = [&](int j0) {
+    // staging registers of the next two tiles: a tile's loads are issued two steps before it is used, so that
+    // their latency has two steps of arithmetic to hide behind
+    bf16x8 kregs[2][K_PER_THREAD];
+    short4_t vregs[2][V_PER_THREAD];
+    auto fetch = [&](bf16x8 (&kreg)[K_PER_THREAD], short4_t (&vreg)[V_PER_THREAD], int j0) {
 #pragma unroll
         for (int i = 0; i < K_PER_THREAD; ++i) {
             const int c = tid + i * 256;
             if (K_CHUNKS % 256 == 0 || c < K_CHUNKS) {
                 const int row = c / (D / 8), col = c % (D / 8);
-                int pos = j0 + row;
-                pos = pos < lo ? lo : (pos > wg_last ? wg_last : pos);
-                const int64_t page = page_of(pos);
-                kreg[i] = pld8(kc + ((page * nkv + kvh) * page_size + page_offset(pos)) * (int64_t)D + col * 8);
+                const int pos = j0 + row;
+                kreg[i] = pld8(k_head + page_of(pos) * page_stride + (page_offset(pos) * D + col * 8));
             }
         }
         {
             const int kg = tid & 7;
             int vpos = j0 + kg * 4;
             vpos = vpos < vlo ? vlo : (vpos > vhi ? vhi : vpos);
-            const int64_t page = page_of(vpos);
-            const bf16* vbase = vc + (page * nkv + kvh) * (int64_t)D * page_size + page_offset(vpos);
+            const bf16* vbase = v_head + page_of(vpos) * page_stride + page_offset(vpos);
 #pragma unroll
             for (int i = 0; i < V_PER_THREAD; ++i) {
                 const int d = (tid >> 3) + 32 * i;
@@ -312,7 +332,7 @@ attention_prefill_lds_kernel(const bf16* __restrict__ q, int64_t q_stride, const
             }
         }
     };
-    auto stash = [&](int buf) {
+    auto stash = [&](const bf16x8 (&kreg)[K_PER_THREAD], const short4_t (&vreg)[V_PER_THREAD], int buf) {
 #pragma unroll
         for (int i = 0; i < K_PER_THREAD; ++i) {
             const int c = tid + i * 256;
@@ -332,13 +352,16 @@ attention_prefill_lds_kernel(const bf16* __restrict__ q, int64_t q_stride, const
     };
 
     const int j_begin = lo & ~31;
-    fetch(j_begin);
-    stash(0);
+    fetch(kregs[0], vregs[0], j_begin);
+    if (j_begin + 32 <= wg_last) fetch(kregs[1], vregs[1], j_begin + 32);
+    stash(kregs[0], vregs[0], 0);
     __syncthreads();
-    int buf = 0;
-    for (int j0 = j_begin; j0 <= wg_last; j0 += 32, buf ^= 1) {
+    // one step: the tile at j0 is in LDS buffer `buf`, the next one is on its way into register set `next`,
+    // and the set that was stored last takes the loads of the tile after that
+    auto step = [&](int j0, int buf, bf16x8 (&knext)[K_PER_THREAD], short4_t (&vnext)[V_PER_THREAD],
+                    bf16x8 (&kfree)[K_PER_THREAD], short4_t (&vfree)[V_PER_THREAD]) {
         const bool more = j0 + 32 <= wg_last;
-        if (more) fetch(j0 + 32);
+        if (j0 + 64 <= wg_last) fetch(kfree, vfree, j0 + 64);
         if (active && j0 <= w_last) {
             bf16x8 kf[2][QK_STEPS];
 #pragma unroll
@@ -383,8 +406,8 @@ attention_prefill_lds_kernel(const bf16* __restrict__ q, int64_t q_stride, const
             float mx[QB];
 #pragma unroll
             for (int qb = 0; qb < QB; ++qb)
-                mx[qb] = fmaxf(fmaxf(fmaxf(s[qb][0][0], s[qb][0][1]), fmaxf(s[qb][0][2], s[qb][0][3])),
-                               fmaxf(fmaxf(s[qb][1][0], s[qb][1][1]), fmaxf(s[qb][1][2], s[qb][1][3])));
+                mx[qb] = max3(max3(s[qb][0][0], s[qb][0][1], s[qb][0][2]), max3(s[qb][0][3], s[qb][1][0], s[qb][1][1]),
+                              max2(s[qb][1][2], s[qb][1][3]));
 #pragma unroll
             for (int qb = 0; qb < QB; ++qb) mx[qb] = group_max(mx[qb]) * scale_log2;   // scale > 0 commutes with max
             float corr[QB], sum[QB];
@@ -392,7 +415,7 @@ attention_prefill_lds_kernel(const bf16* __restrict__ q, int64_t q_stride, const
             bool rescale = false;
 #pragma unroll
             for (int qb = 0; qb < QB; ++qb) {
-                const float m_new = fmaxf(m_run[qb], mx[qb]);
+                const float m_new = max2(m_run[qb], mx[qb]);
                 const float m_use = m_new == -INFINITY ? 0.f : m_new;     // nothing visible yet: weights stay 0
                 corr[qb] = __builtin_amdgcn_exp2f(m_run[qb] - m_use);
                 rescale = rescale || m_new != m_run[qb];
@@ -431,8 +454,13 @@ attention_prefill_lds_kernel(const bf16* __restrict__ q, int64_t q_stride, const
                     acc[qb][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[qb], acc[qb][dt], 0, 0, 0);
             }
         }
-        if (more) stash(buf ^ 1);
+        if (more) stash(knext, vnext, buf ^ 1);
         __syncthreads();
+    };
+    for (int j0 = j_begin; j0 <= wg_last; j0 += 64) {
+        step(j0, 0, kregs[1], vregs[1], kregs[0], vregs[0]);
+        if (j0 + 32 > wg_last) break;
+        step(j0 + 32, 1, kregs[0], vregs[0], kregs[1], vregs[1]);
     }
 
     if (!active) return;
@@ -525,7 +553,7 @@ extern "C" int somi_attention_prefill(const void* q, int64_t q_stride, const voi
     // head sizes 32..128 stage keys and values through LDS; the others (LDS would not hold two tiles, or a
     // tile is smaller than the workgroup's loads) keep them in registers per wavefront, and so do page sizes
     // that are no power of two and block tables too wide for the LDS copy of a request's pages
-    const bool lds_ok = (page_size & (page_size - 1)) == 0 && max_blocks <= PREFILL_LDS_PAGES;
+    const bool lds_ok = (page_size & (page_size - 1)) == 0 && max_blocks + 8 <= PREFILL_LDS_PAGES;   // + a tile's overhang
     switch (D / 16) {
         SOMI_PREFILL(1, 4); SOMI_PREFILL_LDS(2); SOMI_PREFILL_LDS(3); SOMI_PREFILL_LDS(4); SOMI_PREFILL_LDS(5);
         SOMI_PREFILL_LDS(6); SOMI_PREFILL_LDS(7); SOMI_PREFILL_LDS(8); SOMI_PREFILL(9, 2); SOMI_PREFILL(10, 2);
