@@ -463,13 +463,19 @@ static int64_t mid_workspace_floats(int M, int N, int strips, int splits) {
 // pieces of at least 8 chunks, within the workspace.  Chosen by whole decode steps of 64 requests at 7B
 // layer sizes (7.7 ms with this rule: down in 8 splits, gate_up in 2; 8.0 ms with at most 5 or 3 splits,
 // 7.9 ms with twice as many); timing the kernel alone in a loop ranks the shapes differently.
+#ifndef MID_TARGET_WORKGROUPS
+#define MID_TARGET_WORKGROUPS 448             // K is split until about this many workgroups run
+#endif
+#ifndef MID_MIN_CHUNKS
+#define MID_MIN_CHUNKS 8                      // chunks of K a split holds at least
+#endif
 static void mid_shape(int M, int N, int K, bool swiglu, int64_t workspace_floats, int* strips, int* splits) {
     const int chunks = ceil_div(K, MID_CK);
     int ns = (swiglu || ceil_div(N, 128) >= 256) ? 2 : 1;
     int tiles = ceil_div(N, 64 * ns);
     int ks = 1;
     if (tiles < 384) {
-        ks = min(ceil_div(448, tiles), max(1, chunks / 8));
+        ks = min(ceil_div(MID_TARGET_WORKGROUPS, tiles), max(1, chunks / MID_MIN_CHUNKS));
         const int per = ceil_div(chunks, ks);
         ks = ceil_div(chunks, per);                  // no empty split
     }

@@ -12,12 +12,13 @@ SKINNY_ROWS = 64       # up to here it beats the library product at 7B layer siz
 
 
 def _mid_is_faster(m: int, n: int, k: int) -> bool:
-    """Measured at 7B layer sizes: the kernel that shares x inside a workgroup and splits K over workgroups
-    wins from 17 rows on where K is long and the columns are few (down: 31 us against 38 at 32 rows, 38
-    against 53 at 64), and above 32 rows where there are very many columns (gate_up: 71 us against 79)."""
+    """Measured inside decode steps at 7B layer sizes: from 17 rows on, the kernel that shares x inside a
+    workgroup and splits K over workgroups wins where K is long and the columns are few (down: 26 + 5 us
+    against 38 at 32 rows, 34 + 5 against 53 at 64) and where there are very many columns (gate_up: steps of
+    20 to 32 requests 1.7 % shorter, 58 + 8 us against 79 at 64 rows)."""
     if m <= 16:
         return False
-    return (k >= 8192 and n <= 8192) or (m > 32 and n >= 16384)
+    return (k >= 8192 and n <= 8192) or n >= 16384
 
 
 def linear_swiglu(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
