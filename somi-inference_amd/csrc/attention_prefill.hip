@@ -218,9 +218,12 @@ attention_prefill_kernel(const bf16* __restrict__ q, int64_t q_stride, const bf1
 //   K tile in LDS: [32 keys][D + 8] (rows padded by 16 bytes: the 16 rows a 16-byte read touches fall into
 //   different banks); V tile: [D channels][32 + 8 keys] (a row is 20 dwords: the 32 lanes that an 8-byte
 //   read serves at once, 16 channels x 2 key groups, fall into different banks).
-#define PREFILL_LDS_PAGES 2048     // block-table entries of the visible range kept in LDS (else read from memory)
+#define PREFILL_LDS_PAGES 28672    // block-table entries of the visible range that LDS holds at most (112 KB beside the tiles)
 #ifndef PREFILL_WIDE_GROUPS
 #define PREFILL_WIDE_GROUPS 768    // from this many 128-query groups on, workgroups take 128 queries, else 64
+#endif
+#ifndef PREFILL_WIDE_GROUPS_CACHED
+#define PREFILL_WIDE_GROUPS_CACHED 256   // the same where at least half of the keys were cached before the step
 #endif
 template <int DT, int QB>
 __global__ void __launch_bounds__(256, 2)
@@ -239,7 +242,7 @@ attention_prefill_lds_kernel(const bf16* __restrict__ q, int64_t q_stride, const
                                                                         // channels tid / 8 + 32 i
     __shared__ __attribute__((aligned(16))) bf16 ks[2][32 * KROW];
     __shared__ __attribute__((aligned(16))) bf16 vs[2][D * VROW];
-    __shared__ int pages[PREFILL_LDS_PAGES];
+    extern __shared__ int pages[];                          // the launcher sizes it for the widest visible range
 
     // Workgroups are handed out in the order of blockIdx.x, then y, then z: heads vary fastest (the query
     // heads of one key/value head run side by side and share its tiles in L2) and the query groups go from
@@ -262,7 +265,7 @@ attention_prefill_lds_kernel(const bf16* __restrict__ q, int64_t q_stride, const
 
     // The pages of the visible range go to LDS once, so that a tile's addresses do not wait for a
     // table read from memory before its own loads can start.
-    // (power-of-two page size and at most PREFILL_LDS_PAGES pages in reach: the launcher's duty.  A read of
+    // (power-of-two page size and a list that fits LDS: the launcher's duty.  A read of
     // the table from memory inside the loop would make every tile wait for all loads issued before it.)
     // The list covers the 32-key tiles whole: before the first visible key the table's own entries (pages that
     // a window has released read as page 0), past the last one the last page again.  So every key of a tile
@@ -479,23 +482,45 @@ attention_prefill_lds_kernel(const bf16* __restrict__ q, int64_t q_stride, const
     }
 }
 
+// Block-table entries a workgroup of the LDS kernel may list: the pages of its visible range (everything
+// before its last query, or a window and the workgroup's 128 queries) and a 32-key tile's overhang.
+static int prefill_page_entries(int max_blocks, int page_size, int window) {
+    int entries = max_blocks + 8;
+    if (window > 0) entries = min(entries, (window + 128 + 64) / page_size + 8);
+    return entries;
+}
+
 template <int DT>
 static int launch_prefill_lds(const void* q, int64_t q_stride, const void* kc, const void* vc, const int* block_table,
                               int max_blocks, const int* entry_start, const int* entry_first_pos, int n_entries,
-                              int max_entry_len, int nq, int nkv, int page_size, int window, float scale, void* out,
-                              hipStream_t stream) {
+                              int max_entry_len, int max_context, int nq, int nkv, int page_size, int window,
+                              float scale, void* out, hipStream_t stream) {
     // 128 queries per workgroup read every key and value tile half as often as 64 do, but the longest
     // workgroup sets the time: with few workgroups the smaller ones spread better over the compute units.
-    const bool wide = (int64_t)ceil_div(max_entry_len, 128) * n_entries * nq >= PREFILL_WIDE_GROUPS;
+    // Where most keys were cached before the step (max_context, the caller's hint of the longest context a
+    // portion ends at, is several portions long) all workgroups are long and the wide ones win earlier.
+    const int64_t wide_groups = (int64_t)ceil_div(max_entry_len, 128) * n_entries * nq;
+    int reach = max_context;
+    if (window > 0 && reach > window + max_entry_len) reach = window + max_entry_len;
+    const bool wide = wide_groups >= PREFILL_WIDE_GROUPS ||
+                      (wide_groups >= PREFILL_WIDE_GROUPS_CACHED && reach >= 2 * max_entry_len);
     const dim3 grid(nq, n_entries, ceil_div(max_entry_len, wide ? 128 : 64));
-    if (wide)
-        hipLaunchKernelGGL((attention_prefill_lds_kernel<DT, 2>), grid, dim3(256), 0, stream, (const bf16*)q, q_stride,
-                           (const bf16*)kc, (const bf16*)vc, block_table, max_blocks, entry_start, entry_first_pos, nq,
-                           nkv, page_size, window, scale * 1.44269504088896341f, (bf16*)out);
-    else
-        hipLaunchKernelGGL((attention_prefill_lds_kernel<DT, 1>), grid, dim3(256), 0, stream, (const bf16*)q, q_stride,
-                           (const bf16*)kc, (const bf16*)vc, block_table, max_blocks, entry_start, entry_first_pos, nq,
-                           nkv, page_size, window, scale * 1.44269504088896341f, (bf16*)out);
+    const size_t page_list = (size_t)prefill_page_entries(max_blocks, page_size, window) * sizeof(int);
+    if (wide) {
+        if (page_list > 16 * 1024)                       // with the tiles beyond the default limit of LDS
+            (void)hipFuncSetAttribute((const void*)attention_prefill_lds_kernel<DT, 2>,
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)page_list);
+        hipLaunchKernelGGL((attention_prefill_lds_kernel<DT, 2>), grid, dim3(256), page_list, stream, (const bf16*)q,
+                           q_stride, (const bf16*)kc, (const bf16*)vc, block_table, max_blocks, entry_start,
+                           entry_first_pos, nq, nkv, page_size, window, scale * 1.44269504088896341f, (bf16*)out);
+    } else {
+        if (page_list > 16 * 1024)
+            (void)hipFuncSetAttribute((const void*)attention_prefill_lds_kernel<DT, 1>,
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)page_list);
+        hipLaunchKernelGGL((attention_prefill_lds_kernel<DT, 1>), grid, dim3(256), page_list, stream, (const bf16*)q,
+                           q_stride, (const bf16*)kc, (const bf16*)vc, block_table, max_blocks, entry_start,
+                           entry_first_pos, nq, nkv, page_size, window, scale * 1.44269504088896341f, (bf16*)out);
+    }
     SOMI_LAUNCH_CHECK("attention_prefill_lds");
     return 0;
 }
@@ -519,11 +544,12 @@ static int launch_prefill(const void* q, int64_t q_stride, const void* kc, const
 // offsets of the portions in the flat token batch; entry_first_pos: [n_entries] position of each portion's
 // first token; max_entry_len: the longest portion (sizes the grid).  bfloat16 only; head_dim a multiple of 16
 // up to 256; page_size a multiple of 4.  k_cache [pages, nkv, page_size, D], v_cache [pages, nkv, D, page_size];
-// out: [n_tokens, nq * D].
+// out: [n_tokens, nq * D].  max_context: the longest context a portion ends at (a hint for the launch shape; 0: unknown).
 extern "C" int somi_attention_prefill(const void* q, int64_t q_stride, const void* k_cache, const void* v_cache,
                                       const int* block_table, int max_blocks, const int* entry_start,
-                                      const int* entry_first_pos, int n_entries, int max_entry_len, int nq, int nkv,
-                                      int D, int page_size, int window, float scale, void* out, hipStream_t stream) {
+                                      const int* entry_first_pos, int n_entries, int max_entry_len, int max_context,
+                                      int nq, int nkv, int D, int page_size, int window, float scale, void* out,
+                                      hipStream_t stream) {
     SOMI_REQUIRE(n_entries >= 0 && max_entry_len >= 0 && nq > 0 && nkv > 0 && max_blocks > 0,
                  "attention_prefill: bad sizes");
     SOMI_REQUIRE(nq % nkv == 0, "attention_prefill: num_q_heads (%d) must be divisible by num_kv_heads (%d)", nq, nkv);
@@ -548,12 +574,12 @@ extern "C" int somi_attention_prefill(const void* q, int64_t q_stride, const voi
                                          entry_first_pos, n_entries, max_entry_len, nq, nkv, page_size, window,    \
                                          scale, out, stream);                                                      \
         return launch_prefill_lds<DT>(q, q_stride, k_cache, v_cache, block_table, max_blocks, entry_start,         \
-                                      entry_first_pos, n_entries, max_entry_len, nq, nkv, page_size, window, scale, \
-                                      out, stream)
+                                      entry_first_pos, n_entries, max_entry_len, max_context, nq, nkv, page_size,   \
+                                      window, scale, out, stream)
     // head sizes 32..128 stage keys and values through LDS; the others (LDS would not hold two tiles, or a
     // tile is smaller than the workgroup's loads) keep them in registers per wavefront, and so do page sizes
     // that are no power of two and block tables too wide for the LDS copy of a request's pages
-    const bool lds_ok = (page_size & (page_size - 1)) == 0 && max_blocks + 8 <= PREFILL_LDS_PAGES;   // + a tile's overhang
+    const bool lds_ok = (page_size & (page_size - 1)) == 0 && prefill_page_entries(max_blocks, page_size, window) <= PREFILL_LDS_PAGES;
     switch (D / 16) {
         SOMI_PREFILL(1, 4); SOMI_PREFILL_LDS(2); SOMI_PREFILL_LDS(3); SOMI_PREFILL_LDS(4); SOMI_PREFILL_LDS(5);
         SOMI_PREFILL_LDS(6); SOMI_PREFILL_LDS(7); SOMI_PREFILL_LDS(8); SOMI_PREFILL(9, 2); SOMI_PREFILL(10, 2);

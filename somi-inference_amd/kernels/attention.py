@@ -47,7 +47,8 @@ def paged_attention(qkv: torch.Tensor, num_heads: int, k_cache: torch.Tensor, v_
         # portions of prompts: query tiles against key tiles (single tokens in the same batch ride along
         # as portions of one)
         ops.attention_prefill(qkv, qkv.shape[1], k_cache, v_cache, block_table, step.entry_start,
-                              step.entry_first_position, step.max_entry_len, num_heads, window, scale, out)
+                              step.entry_first_position, step.max_entry_len, num_heads, window, scale, out,
+                              max_context=step.max_context)
         return out
     split_len, num_splits = decode_splits(step.num_tokens, groups, step.max_context)
     ops.attention_decode(qkv, qkv.shape[1], k_cache, v_cache, block_table, step.token_entry, step.positions,

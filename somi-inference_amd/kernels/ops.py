@@ -240,10 +240,12 @@ def attention_decode(q: torch.Tensor, q_stride: int, k_cache: torch.Tensor, v_ca
 
 def attention_prefill(q: torch.Tensor, q_stride: int, k_cache: torch.Tensor, v_cache: torch.Tensor,
                       block_table: torch.Tensor, entry_start: torch.Tensor, entry_first_position: torch.Tensor,
-                      max_entry_len: int, nq: int, window: int, scale: float, out: torch.Tensor) -> None:
+                      max_entry_len: int, nq: int, window: int, scale: float, out: torch.Tensor,
+                      max_context: int = 0) -> None:
     """MFMA causal attention of every token of every portion over its request's pages, into ``out``
     ([N, nq * D] bfloat16).  entry_start: [E + 1] int32 offsets of the portions in the flat batch;
-    entry_first_position: [E] int32."""
+    entry_first_position: [E] int32.  ``max_context``: the longest context a portion ends at, a hint for the
+    launch shape (0: unknown)."""
     _need(q, "q", torch.bfloat16)
     n = q.shape[0]
     _need(k_cache, "k cache", torch.bfloat16)
@@ -262,8 +264,8 @@ def attention_prefill(q: torch.Tensor, q_stride: int, k_cache: torch.Tensor, v_c
         raise KernelError(f"attention_prefill: longest portion {max_entry_len} does not fit {n} tokens")
     _check(library().somi_attention_prefill(
         _ptr(q), ctypes.c_int64(q_stride), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), block_table.shape[1],
-        _ptr(entry_start), _ptr(entry_first_position), entries, max_entry_len, nq, nkv, head_dim, page_size, window,
-        ctypes.c_float(scale), _ptr(out), _stream()))
+        _ptr(entry_start), _ptr(entry_first_position), entries, max_entry_len, max(0, int(max_context)), nq, nkv,
+        head_dim, page_size, window, ctypes.c_float(scale), _ptr(out), _stream()))
 
 
 def silu_mul(gate_up: torch.Tensor, block: int = 0) -> torch.Tensor:
