@@ -18,6 +18,9 @@
 // One workgroup per (token, group of heads): cos and sin of the token's angles are computed once into LDS
 // and serve every head of the group; the group's (head, channel pair) items are dealt to the threads.
 template <typename T>
+struct __attribute__((aligned(16))) Pack8 { T v[8]; };      // eight bfloat16: one 16-byte access
+
+template <typename T, bool VEC8>
 __global__ void __launch_bounds__(ROPE_THREADS)
 rope_kv_store_kernel(T* __restrict__ qkv, int64_t row_stride, const int* __restrict__ positions,
                      const int* __restrict__ slots, const float* __restrict__ inv_freq, int rot_half,
@@ -42,7 +45,30 @@ rope_kv_store_kernel(T* __restrict__ qkv, int64_t row_stride, const int* __restr
 
     // q (in place) and k (into its page): rotate the pairs (j, j + rot_half)
     const int rot0 = h0, rot1 = min(h1, nq + nkv);
-    if (rot_half > 0)
+    if (VEC8 && rot_half > 0) {
+        // eight neighbouring pairs per thread: 16-byte loads and stores (the launcher checked the alignment)
+        const int groups = rot_half / 8;
+        for (int item = tid; item < (rot1 - rot0) * groups; item += ROPE_THREADS) {
+            const int hh = rot0 + item / groups, j = (item % groups) * 8;
+            const T* src = row + (int64_t)hh * D + j;
+            T* dst = row + (int64_t)hh * D + j;
+            if (hh >= nq) {
+                if (slot < 0) continue;
+                dst = kc + ((page * nkv + (hh - nq)) * page_size + off) * D + j;
+            }
+            Pack8<T> lo = *reinterpret_cast<const Pack8<T>*>(src), hi = *reinterpret_cast<const Pack8<T>*>(src + rot_half);
+            Pack8<T> first, second;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const float x1 = to_float(lo.v[i]), x2 = to_float(hi.v[i]);
+                const float c = cs[0][j + i], sn = cs[1][j + i];
+                first.v[i] = from_float<T>(x1 * c - x2 * sn);
+                second.v[i] = from_float<T>(x2 * c + x1 * sn);
+            }
+            *reinterpret_cast<Pack8<T>*>(dst) = first;
+            *reinterpret_cast<Pack8<T>*>(dst + rot_half) = second;
+        }
+    } else if (rot_half > 0)
         for (int item = tid; item < (rot1 - rot0) * rot_half; item += ROPE_THREADS) {
             const int hh = rot0 + item / rot_half, j = item % rot_half;
             const T* src = row + (int64_t)hh * D;
@@ -94,12 +120,19 @@ extern "C" int somi_rope_kv_store(void* qkv, int dtype, int64_t row_stride, cons
     const int heads_per_block = max(1, min(heads, (int)(((int64_t)n_tokens * heads + 2047) / 2048)));
     const dim3 grid(n_tokens, ceil_div(heads, heads_per_block));
     const int rot_half = inv_freq ? rotary_dim / 2 : 0;
+    // the 16-byte path of bfloat16: every head, half and row starts at a multiple of eight elements
+    const bool vec8 = dtype == SOMI_BF16 && rot_half % 8 == 0 && D % 8 == 0 && row_stride % 8 == 0 &&
+                      (uintptr_t)qkv % 16 == 0 && (nkv == 0 || (uintptr_t)k_cache % 16 == 0);
     if (dtype == SOMI_F32)
-        hipLaunchKernelGGL(rope_kv_store_kernel<float>, grid, dim3(ROPE_THREADS), 0, stream, (float*)qkv, row_stride,
-                           positions, slots, inv_freq, rot_half, nq, nkv, D, (float*)k_cache, (float*)v_cache,
+        hipLaunchKernelGGL((rope_kv_store_kernel<float, false>), grid, dim3(ROPE_THREADS), 0, stream, (float*)qkv,
+                           row_stride, positions, slots, inv_freq, rot_half, nq, nkv, D, (float*)k_cache,
+                           (float*)v_cache, page_size, heads_per_block);
+    else if (dtype == SOMI_BF16 && vec8)
+        hipLaunchKernelGGL((rope_kv_store_kernel<bf16, true>), grid, dim3(ROPE_THREADS), 0, stream, (bf16*)qkv, row_stride,
+                           positions, slots, inv_freq, rot_half, nq, nkv, D, (bf16*)k_cache, (bf16*)v_cache,
                            page_size, heads_per_block);
     else if (dtype == SOMI_BF16)
-        hipLaunchKernelGGL(rope_kv_store_kernel<bf16>, grid, dim3(ROPE_THREADS), 0, stream, (bf16*)qkv, row_stride,
+        hipLaunchKernelGGL((rope_kv_store_kernel<bf16, false>), grid, dim3(ROPE_THREADS), 0, stream, (bf16*)qkv, row_stride,
                            positions, slots, inv_freq, rot_half, nq, nkv, D, (bf16*)k_cache, (bf16*)v_cache,
                            page_size, heads_per_block);
     else
