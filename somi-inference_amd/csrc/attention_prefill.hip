@@ -216,8 +216,9 @@ attention_prefill_kernel(const bf16* __restrict__ q, int64_t q_stride, const bf1
 // from LDS, then store it into the other LDS buffer; one barrier per step.  Every key and value is read
 // from L2/HBM once per 128 queries instead of once per wavefront.
 //   K tile in LDS: [32 keys][D + 8] (rows padded by 16 bytes: the 16 rows a 16-byte read touches fall into
-//   different banks); V tile: [D channels][32 + 8 keys] (a row is 20 dwords: the 32 lanes that an 8-byte
-//   read serves at once, 16 channels x 2 key groups, fall into different banks).
+//   different banks); V tile: [D channels][32 + 4 keys] (a row is 18 dwords: the 16 channels that an 8-byte
+//   read serves at once fall into different pairs of the 32 banks; with 20 dwords a row the counters showed
+//   twice the conflicts).
 #define PREFILL_LDS_PAGES 28672    // block-table entries of the visible range that LDS holds at most (112 KB beside the tiles)
 #ifndef PREFILL_WIDE_GROUPS
 #define PREFILL_WIDE_GROUPS 768    // from this many 128-query groups on, workgroups take 128 queries, else 64
@@ -234,7 +235,7 @@ attention_prefill_lds_kernel(const bf16* __restrict__ q, int64_t q_stride, const
     constexpr int D = DT * 16;
     constexpr int QK_STEPS = (DT + 1) / 2;
     constexpr int QW = QB * 16, WAVES = 4, QG = WAVES * QW;             // 64 or 128 queries per workgroup
-    constexpr int KROW = D + 8, VROW = 32 + 8;                          // padded LDS rows, in elements
+    constexpr int KROW = D + 8, VROW = 32 + 4;                          // padded LDS rows, in elements
     constexpr int K_CHUNKS = 32 * D / 8;                                // 16-byte pieces of a key tile
     constexpr int K_PER_THREAD = (K_CHUNKS + 255) / 256;
     constexpr int V_PER_THREAD = (D + 31) / 32;                         // 8-byte pieces (4 keys of a channel): a
