@@ -180,11 +180,23 @@ attention_decode_kernel(const bf16* __restrict__ q, int64_t q_stride, const bf16
 // scores and the softmax of the 32 keys (a few products), then applies the weights to its own quarter of
 // the head's channels, so the output needs no merge across wavefronts.
 typedef __attribute__((ext_vector_type(2))) unsigned u32x2;
+// Maxima of scores, which are never NaN (keys that must not be seen are -inf): the bare instructions, without
+// the quieting of signalling NaNs that fmaxf adds to each operand.
+__device__ __forceinline__ float max2(float a, float b) {
+    float r;
+    asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+    return r;
+}
+__device__ __forceinline__ float max3(float a, float b, float c) {
+    float r;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
 __device__ __forceinline__ float lanes4_max(float v) {       // over lanes l, l ^ 16, l ^ 32, l ^ 48
     u32x2 a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
-    v = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+    v = max2(__uint_as_float(a[0]), __uint_as_float(a[1]));
     u32x2 b = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
-    return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+    return max2(__uint_as_float(b[0]), __uint_as_float(b[1]));
 }
 __device__ __forceinline__ float lanes4_sum(float v) {
     u32x2 a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
@@ -248,10 +260,17 @@ attention_decode_lds_kernel(const bf16* __restrict__ q, int64_t q_stride, const 
         // for every tile load issued before it.
         const int shift = __builtin_ctz(page_size);
         auto page_offset = [&](int pos) { return pos & (page_size - 1); };
-        const int page_lo = begin >> shift, page_count = (end >> shift) - page_lo + 1;
-        for (int i = tid; i < page_count; i += 256) pages[i] = table[page_lo + i];
+        // The list covers the 32-key tiles whole (before the first visible key the table's own entries, past the
+        // last one the last page again): every key of a tile has an address that may be read, and the keys
+        // outside the split are masked.
+        const int page_lo = (begin & ~31) >> shift, page_last = end >> shift;
+        const int page_count = ((end | 31) >> shift) - page_lo + 1;
+        for (int i = tid; i < page_count; i += 256) pages[i] = table[min(page_lo + i, page_last)];
         __syncthreads();
         auto page_of = [&](int pos) -> int64_t { return pages[(pos >> shift) - page_lo]; };
+        const int64_t page_stride = (int64_t)nkv * page_size * D;      // elements from one page to the next
+        const bf16* k_head = kc + (int64_t)kvh * page_size * D;
+        const bf16* v_head = vc + (int64_t)kvh * page_size * D;
         // two register sets: the tiles two and three steps ahead are in flight while one is computed
         bf16x8 kreg_a[K_PER_THREAD], kreg_b[K_PER_THREAD];
         short4_t vreg_a[V_PER_THREAD], vreg_b[V_PER_THREAD];
@@ -261,15 +280,14 @@ attention_decode_lds_kernel(const bf16* __restrict__ q, int64_t q_stride, const 
                 const int c = tid + i * 256;
                 if (K_CHUNKS % 256 == 0 || c < K_CHUNKS) {
                     const int row = c / (D / 8), col = c % (D / 8);
-                    int pos = j0 + row;
-                    pos = pos < begin ? begin : (pos > end ? end : pos);
-                    kreg[i] = ld8(kc + ((page_of(pos) * nkv + kvh) * page_size + page_offset(pos)) * (int64_t)D + col * 8);
+                    const int pos = j0 + row;
+                    kreg[i] = ld8(k_head + page_of(pos) * page_stride + (page_offset(pos) * D + col * 8));
                 }
             }
             const int kg = tid & 7;
             int vpos = j0 + kg * 4;
             vpos = vpos < vlo ? vlo : (vpos > vhi ? vhi : vpos);
-            const bf16* vbase = vc + (page_of(vpos) * nkv + kvh) * (int64_t)D * page_size + page_offset(vpos);
+            const bf16* vbase = v_head + page_of(vpos) * page_stride + page_offset(vpos);
 #pragma unroll
             for (int i = 0; i < V_PER_THREAD; ++i) {
                 const int d = (tid >> 3) + 32 * i;
@@ -320,11 +338,10 @@ attention_decode_lds_kernel(const bf16* __restrict__ q, int64_t q_stride, const 
                         if (key < begin || key > end) s[half][i] = -INFINITY;
                     }
             }
-            float mx = fmaxf(fmaxf(fmaxf(s[0][0], s[0][1]), fmaxf(s[0][2], s[0][3])),
-                             fmaxf(fmaxf(s[1][0], s[1][1]), fmaxf(s[1][2], s[1][3])));
+            float mx = max3(max3(s[0][0], s[0][1], s[0][2]), max3(s[0][3], s[1][0], s[1][1]), max2(s[1][2], s[1][3]));
             mx = lanes4_max(mx) * scale_log2;                // scale > 0: the maximum commutes with it
             // running maximum and weights in base 2: weight = 2^(s * scale * log2(e) - m)
-            const float m_new = fmaxf(m_run, mx);            // finite: every 32-key step holds a visible key
+            const float m_new = max2(m_run, mx);             // finite: every 32-key step holds a visible key
             const float corr = __builtin_amdgcn_exp2f(m_run - m_new);
             float pr[2][4], sum = 0.f;
 #pragma unroll
@@ -455,7 +472,7 @@ static int launch_decode(const void* q, int64_t q_stride, const void* kc, const 
     const int G = nq / nkv, HB = (G + 15) / 16;
     const size_t smem = (size_t)(waves * DT * 256 + waves * 32) * sizeof(float);
     const bool pow2_pages = (page_size & (page_size - 1)) == 0;
-    if (DT >= 2 && DT <= 8 && pow2_pages && split_len / page_size + 2 <= DECODE_LDS_PAGES)
+    if (DT >= 2 && DT <= 8 && pow2_pages && split_len / page_size + 2 + 8 <= DECODE_LDS_PAGES)   // + a tile's overhang
         // head sizes 32..128: keys and values staged through LDS (two tiles fit)
         hipLaunchKernelGGL((attention_decode_lds_kernel<(DT >= 2 && DT <= 8 ? DT : 2)>), dim3(n_list, nkv * HB, num_splits),
                            dim3(256), 0, stream, (const bf16*)q, q_stride, (const bf16*)kc, (const bf16*)vc, block_table,
