@@ -441,8 +441,12 @@ static int mid_launch(const void* x, const void* w, const float* bias, void* out
 // A program that measures other shapes (chunk sizes, depths) can include this file with SOMI_MID_NO_ENTRY_POINTS
 // defined and instantiate the launchers above itself; the library builds what follows.
 #ifndef SOMI_MID_NO_ENTRY_POINTS
+#ifndef MID_CK
 #define MID_CK 64                                // K values per chunk and chunks in flight of the shapes that are built
+#endif
+#ifndef MID_DEPTH
 #define MID_DEPTH 2
+#endif
 
 template <int MT, typename TO, int FUSE>
 static int mid_strips(const void* x, const void* w, const float* bias, void* out, int M, int N, int K, int strips,
