@@ -175,20 +175,21 @@ def test_step_contract_errors(model_folders):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_captured_decode_steps_replay_like_eager_steps(dtype, model_folders):
-    """Decode steps are captured as HIP graphs per batch size.  Batches of 3 and of 40 requests (the larger
-    one takes the library matrix product inside the graph) are replayed several times, with eager work and
-    synchronisations in between, and every replay is compared with the same step run without graphs."""
+    """Decode steps are captured as HIP graphs per batch size.  Batches of 3, 40 and 70 requests (the largest
+    takes the library matrix product inside the graph, the others the kernels that fuse norm, rotation and
+    residual add into the products) are replayed several times, with eager work and synchronisations in
+    between, and every replay is compared with the same step run without graphs."""
     from somi_inference_amd.models import load_model, make_runner
     from somi_inference_amd.engine import ModelRunner
     from somi_inference_amd.cache import CacheManager
     vocab, bs = TINY["B"]["config"].vocab_size, TINY["B"]["block_size"]
     model, _ = load_model(model_folders["B"], dtype=dtype)
-    graphed = make_runner(model, block_size=bs, num_blocks=256, max_requests=48)
-    eager_cache = CacheManager(model.cache_needs(), block_size=bs, num_blocks=256, max_requests=48,
+    graphed = make_runner(model, block_size=bs, num_blocks=512, max_requests=80)
+    eager_cache = CacheManager(model.cache_needs(), block_size=bs, num_blocks=512, max_requests=80,
                                dtype=model.runtime.dtype, device=model.runtime.device)
     eager = ModelRunner(model, eager_cache, decode_graphs=False)
     assert graphed.decode_graphs and not eager.decode_graphs
-    for batch in (3, 40):
+    for batch in (3, 40, 70):
         ids = [f"g{batch}_{i}" for i in range(batch)]
         prompts = [token_ids(vocab, 5 + (i * 7) % 23, 300 + i) for i in range(batch)]
         for runner in (graphed, eager):
@@ -212,7 +213,7 @@ def test_captured_decode_steps_replay_like_eager_steps(dtype, model_folders):
         for runner in (graphed, eager):
             for rid in ids:
                 runner.end(rid)
-    assert graphed.graph_replays >= 24
+    assert graphed.graph_replays >= 36
 
 
 REAL_SIZES = {
