@@ -221,7 +221,7 @@ attention_prefill_kernel(const bf16* __restrict__ q, int64_t q_stride, const bf1
 //   twice the conflicts).
 #define PREFILL_LDS_PAGES 28672    // block-table entries of the visible range that LDS holds at most (112 KB beside the tiles)
 #ifndef PREFILL_WIDE_GROUPS
-#define PREFILL_WIDE_GROUPS 768    // from this many 128-query groups on, workgroups take 128 queries, else 64
+#define PREFILL_WIDE_GROUPS 600    // from this many 128-query groups on, workgroups take 128 queries, else 64 (measured: 448 groups 72 against 82 us with 64 queries, 672 groups 136 against 119)
 #endif
 #ifndef PREFILL_WIDE_GROUPS_CACHED
 #define PREFILL_WIDE_GROUPS_CACHED 256   // the same where at least half of the keys were cached before the step
