@@ -223,11 +223,27 @@ attention_prefill_kernel(const bf16* __restrict__ q, int64_t q_stride, const bf1
 #ifndef PREFILL_WIDE_GROUPS
 #define PREFILL_WIDE_GROUPS 600    // from this many 128-query groups on, workgroups take 128 queries, else 64 (measured: 448 groups 72 against 82 us with 64 queries, 672 groups 136 against 119)
 #endif
+// The launch shapes of the LDS kernel; a caller may ask for one (tests do, to reach each at small sizes).
+#define PREFILL_SHAPE_AUTO 0
+#define PREFILL_SHAPE_NARROW 1     // 64 queries a workgroup
+#define PREFILL_SHAPE_SPLIT 2      // 64 queries, two wavefronts share a query block's keys
+#define PREFILL_SHAPE_WIDE 3       // 128 queries
+#ifndef PREFILL_KEY_SPLIT_BELOW
+#define PREFILL_KEY_SPLIT_BELOW 896   // below this many 64-query workgroups two wavefronts share a query block's keys
+                                      // (measured at 7B head counts: 448 workgroups 29 against 33 us, 512 tokens after
+                                      // 3,584 cached 83 against 108; 896 workgroups the same; 1,120 workgroups 94 against 89)
+#endif
+#ifndef PREFILL_KEY_SPLIT_REACH
+#define PREFILL_KEY_SPLIT_REACH 1024  // and only where the longest workgroup walks at least this many keys (32 tiles)
+#endif
 #ifndef PREFILL_WIDE_GROUPS_CACHED
 #define PREFILL_WIDE_GROUPS_CACHED 256   // the same where at least half of the keys were cached before the step
 #endif
-template <int DT, int QB>
-__global__ void __launch_bounds__(256, 2)
+// KS = 2: twice the wavefronts; each query block is owned by KS of them, which take the 32-key tiles in turn
+// (tile index modulo KS, by absolute position) and join their sums, maxima and outputs through LDS at the
+// end.  The longest workgroup, which sets the time of a short prompt, has half as many steps to walk.
+template <int DT, int QB, int KS>
+__global__ void __launch_bounds__(256 * KS, 2 * KS)     // the second figure: wavefronts per SIMD to leave room for
 attention_prefill_lds_kernel(const bf16* __restrict__ q, int64_t q_stride, const bf16* __restrict__ kc,
                              const bf16* __restrict__ vc, const int* __restrict__ block_table, int max_blocks,
                              const int* __restrict__ entry_start, const int* __restrict__ entry_first_pos, int nq,
@@ -241,8 +257,9 @@ attention_prefill_lds_kernel(const bf16* __restrict__ q, int64_t q_stride, const
     constexpr int V_PER_THREAD = (D + 31) / 32;                         // 8-byte pieces (4 keys of a channel): a
                                                                         // thread takes key group tid % 8 of
                                                                         // channels tid / 8 + 32 i
-    __shared__ __attribute__((aligned(16))) bf16 ks[2][32 * KROW];
-    __shared__ __attribute__((aligned(16))) bf16 vs[2][D * VROW];
+    constexpr int THREADS = 256 * KS, STEP = 32 * KS;                   // keys a step of the workgroup covers
+    __shared__ __attribute__((aligned(16))) bf16 ks[2][KS][32 * KROW];
+    __shared__ __attribute__((aligned(16))) bf16 vs[2][KS][D * VROW];
     extern __shared__ int pages[];                          // the launcher sizes it for the widest visible range
 
     // Workgroups are handed out in the order of blockIdx.x, then y, then z: heads vary fastest (the query
@@ -251,7 +268,10 @@ attention_prefill_lds_kernel(const bf16* __restrict__ q, int64_t q_stride, const
     // workgroups first and the short ones land beside them.
     const int h = blockIdx.x, e = blockIdx.y;
     const int kvh = h / (nq / nkv);
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, r = lane & 15, g = lane >> 4;
+    const int tid = threadIdx.x, lane = tid & 63, r = lane & 15, g = lane >> 4;
+    const int wave = (tid >> 6) & 3;                        // the query block of this wavefront
+    const int kh = tid >> 8;                                // which of a step's KS tiles it computes and fetches
+    const int tid256 = tid & 255;
     const int start = entry_start[e];
     const int len = entry_start[e + 1] - start;
     const int group = gridDim.z - 1 - blockIdx.z;
@@ -268,14 +288,14 @@ attention_prefill_lds_kernel(const bf16* __restrict__ q, int64_t q_stride, const
     // table read from memory before its own loads can start.
     // (power-of-two page size and a list that fits LDS: the launcher's duty.  A read of
     // the table from memory inside the loop would make every tile wait for all loads issued before it.)
-    // The list covers the 32-key tiles whole: before the first visible key the table's own entries (pages that
+    // The list covers the steps' tiles whole: before the first visible key the table's own entries (pages that
     // a window has released read as page 0), past the last one the last page again.  So every key of a tile
     // has an address that may be read, and keys outside the visible range need no clamp: their scores are
     // masked.
     const int shift = __builtin_ctz(page_size);
-    const int page_lo = (lo & ~31) >> shift, page_last = wg_last >> shift;
-    const int page_count = (((wg_last | 31) >> shift) - page_lo) + 1;
-    for (int i = tid; i < page_count; i += 256) pages[i] = table[min(page_lo + i, page_last)];
+    const int page_lo = (lo & ~(STEP - 1)) >> shift, page_last = wg_last >> shift;
+    const int page_count = (((wg_last | (STEP - 1)) >> shift) - page_lo) + 1;
+    for (int i = tid; i < page_count; i += THREADS) pages[i] = table[min(page_lo + i, page_last)];
     __syncthreads();
     auto page_of = [&](int pos) -> int64_t { return pages[(pos >> shift) - page_lo]; };
     auto page_offset = [&](int pos) { return pos & (page_size - 1); };
@@ -314,10 +334,11 @@ attention_prefill_lds_kernel(const bf16* __restrict__ q, int64_t q_stride, const
     // their latency has two steps of arithmetic to hide behind
     bf16x8 kregs[2][K_PER_THREAD];
     short4_t vregs[2][V_PER_THREAD];
-    auto fetch = [&](bf16x8 (&kreg)[K_PER_THREAD], short4_t (&vreg)[V_PER_THREAD], int j0) {
+    auto fetch = [&](bf16x8 (&kreg)[K_PER_THREAD], short4_t (&vreg)[V_PER_THREAD], int j_step) {
+        const int j0 = j_step + 32 * kh;                     // this thread's tile of the step
 #pragma unroll
         for (int i = 0; i < K_PER_THREAD; ++i) {
-            const int c = tid + i * 256;
+            const int c = tid256 + i * 256;
             if (K_CHUNKS % 256 == 0 || c < K_CHUNKS) {
                 const int row = c / (D / 8), col = c % (D / 8);
                 const int pos = j0 + row;
@@ -325,13 +346,13 @@ attention_prefill_lds_kernel(const bf16* __restrict__ q, int64_t q_stride, const
             }
         }
         {
-            const int kg = tid & 7;
+            const int kg = tid256 & 7;
             int vpos = j0 + kg * 4;
             vpos = vpos < vlo ? vlo : (vpos > vhi ? vhi : vpos);
             const bf16* vbase = v_head + page_of(vpos) * page_stride + page_offset(vpos);
 #pragma unroll
             for (int i = 0; i < V_PER_THREAD; ++i) {
-                const int d = (tid >> 3) + 32 * i;
+                const int d = (tid256 >> 3) + 32 * i;
                 if (D % 32 == 0 || d < D) vreg[i] = pld4(vbase + (int64_t)d * page_size);
             }
         }
@@ -339,38 +360,39 @@ attention_prefill_lds_kernel(const bf16* __restrict__ q, int64_t q_stride, const
     auto stash = [&](const bf16x8 (&kreg)[K_PER_THREAD], const short4_t (&vreg)[V_PER_THREAD], int buf) {
 #pragma unroll
         for (int i = 0; i < K_PER_THREAD; ++i) {
-            const int c = tid + i * 256;
+            const int c = tid256 + i * 256;
             if (K_CHUNKS % 256 == 0 || c < K_CHUNKS) {
                 const int row = c / (D / 8), col = c % (D / 8);
-                *reinterpret_cast<bf16x8*>(&ks[buf][row * KROW + col * 8]) = kreg[i];
+                *reinterpret_cast<bf16x8*>(&ks[buf][kh][row * KROW + col * 8]) = kreg[i];
             }
         }
         {
-            const int kg = tid & 7;
+            const int kg = tid256 & 7;
 #pragma unroll
             for (int i = 0; i < V_PER_THREAD; ++i) {
-                const int d = (tid >> 3) + 32 * i;
-                if (D % 32 == 0 || d < D) *reinterpret_cast<short4_t*>(&vs[buf][d * VROW + kg * 4]) = vreg[i];
+                const int d = (tid256 >> 3) + 32 * i;
+                if (D % 32 == 0 || d < D) *reinterpret_cast<short4_t*>(&vs[buf][kh][d * VROW + kg * 4]) = vreg[i];
             }
         }
     };
 
-    const int j_begin = lo & ~31;
+    const int j_begin = lo & ~(STEP - 1);
     fetch(kregs[0], vregs[0], j_begin);
-    if (j_begin + 32 <= wg_last) fetch(kregs[1], vregs[1], j_begin + 32);
+    if (j_begin + STEP <= wg_last) fetch(kregs[1], vregs[1], j_begin + STEP);
     stash(kregs[0], vregs[0], 0);
     __syncthreads();
-    // one step: the tile at j0 is in LDS buffer `buf`, the next one is on its way into register set `next`,
-    // and the set that was stored last takes the loads of the tile after that
-    auto step = [&](int j0, int buf, bf16x8 (&knext)[K_PER_THREAD], short4_t (&vnext)[V_PER_THREAD],
+    // one step: the tiles from j_step on are in LDS buffer `buf`, the next ones are on their way into register
+    // set `next`, and the set that was stored last takes the loads of the tiles after those
+    auto step = [&](int j_step, int buf, bf16x8 (&knext)[K_PER_THREAD], short4_t (&vnext)[V_PER_THREAD],
                     bf16x8 (&kfree)[K_PER_THREAD], short4_t (&vfree)[V_PER_THREAD]) {
-        const bool more = j0 + 32 <= wg_last;
-        if (j0 + 64 <= wg_last) fetch(kfree, vfree, j0 + 64);
+        const bool more = j_step + STEP <= wg_last;
+        if (j_step + 2 * STEP <= wg_last) fetch(kfree, vfree, j_step + 2 * STEP);
+        const int j0 = j_step + 32 * kh;                     // this wavefront's tile of the step
         if (active && j0 <= w_last) {
             bf16x8 kf[2][QK_STEPS];
 #pragma unroll
             for (int half = 0; half < 2; ++half) {
-                const bf16* krow = &ks[buf][(half * 16 + r) * KROW];
+                const bf16* krow = &ks[buf][kh][(half * 16 + r) * KROW];
 #pragma unroll
                 for (int c = 0; c < DT / 2; ++c) kf[half][c] = *reinterpret_cast<const bf16x8*>(krow + c * 32 + g * 8);
                 if (DT & 1) {
@@ -450,7 +472,7 @@ attention_prefill_lds_kernel(const bf16* __restrict__ q, int64_t q_stride, const
             }
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) {
-                const bf16* vrow = &vs[buf][(dt * 16 + r) * VROW];
+                const bf16* vrow = &vs[buf][kh][(dt * 16 + r) * VROW];
                 const bf16x8 vf = pjoin(*reinterpret_cast<const short4_t*>(vrow + g * 4),
                                         *reinterpret_cast<const short4_t*>(vrow + 16 + g * 4));
 #pragma unroll
@@ -461,12 +483,46 @@ attention_prefill_lds_kernel(const bf16* __restrict__ q, int64_t q_stride, const
         if (more) stash(knext, vnext, buf ^ 1);
         __syncthreads();
     };
-    for (int j0 = j_begin; j0 <= wg_last; j0 += 64) {
+    for (int j0 = j_begin; j0 <= wg_last; j0 += 2 * STEP) {
         step(j0, 0, kregs[1], vregs[1], kregs[0], vregs[0]);
-        if (j0 + 32 > wg_last) break;
-        step(j0 + 32, 1, kregs[0], vregs[0], kregs[1], vregs[1]);
+        if (j0 + STEP > wg_last) break;
+        step(j0 + STEP, 1, kregs[0], vregs[0], kregs[1], vregs[1]);
     }
 
+    if constexpr (KS == 2) {
+        // the wavefronts of the odd tiles hand their maxima, sums and outputs to those of the even tiles (every
+        // wavefront has passed the last step's barrier: the key tiles are done with)
+        constexpr int ITEMS = QB * (DT * 4 + 2);
+        float* hand = reinterpret_cast<float*>(&ks[0][0][0]) + wave * ITEMS * 64 + lane;
+        static_assert(sizeof(ks) >= sizeof(float) * 4 * ITEMS * 64, "the key tiles hold what the wavefronts hand over");
+        if (kh == 1) {
+#pragma unroll
+            for (int qb = 0; qb < QB; ++qb) {
+                float* to = hand + qb * (DT * 4 + 2) * 64;
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) to[(dt * 4 + i) * 64] = acc[qb][dt][i];
+                to[DT * 4 * 64] = m_run[qb];
+                to[(DT * 4 + 1) * 64] = l_run[qb];
+            }
+        }
+        __syncthreads();
+        if (kh == 1) return;
+#pragma unroll
+        for (int qb = 0; qb < QB; ++qb) {
+            const float* from = hand + qb * (DT * 4 + 2) * 64;
+            const float m_other = from[DT * 4 * 64], l_other = from[(DT * 4 + 1) * 64];
+            const float m_new = max2(m_run[qb], m_other);
+            const float m_use = m_new == -INFINITY ? 0.f : m_new;
+            const float mine = __builtin_amdgcn_exp2f(m_run[qb] - m_use), theirs = __builtin_amdgcn_exp2f(m_other - m_use);
+            l_run[qb] = l_run[qb] * mine + l_other * theirs;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) acc[qb][dt][i] = acc[qb][dt][i] * mine + from[(dt * 4 + i) * 64] * theirs;
+        }
+    }
     if (!active) return;
 #pragma unroll
     for (int qb = 0; qb < QB; ++qb) {
@@ -486,16 +542,16 @@ attention_prefill_lds_kernel(const bf16* __restrict__ q, int64_t q_stride, const
 // Block-table entries a workgroup of the LDS kernel may list: the pages of its visible range (everything
 // before its last query, or a window and the workgroup's 128 queries) and a 32-key tile's overhang.
 static int prefill_page_entries(int max_blocks, int page_size, int window) {
-    int entries = max_blocks + 8;
-    if (window > 0) entries = min(entries, (window + 128 + 64) / page_size + 8);
+    int entries = max_blocks + 16;                   // + the overhang of a step of two 32-key tiles, pages of 4 keys
+    if (window > 0) entries = min(entries, (window + 128 + 128) / page_size + 16);
     return entries;
 }
 
 template <int DT>
 static int launch_prefill_lds(const void* q, int64_t q_stride, const void* kc, const void* vc, const int* block_table,
                               int max_blocks, const int* entry_start, const int* entry_first_pos, int n_entries,
-                              int max_entry_len, int max_context, int nq, int nkv, int page_size, int window,
-                              float scale, void* out, hipStream_t stream) {
+                              int max_entry_len, int max_context, int shape, int nq, int nkv, int page_size,
+                              int window, float scale, void* out, hipStream_t stream) {
     // 128 queries per workgroup read every key and value tile half as often as 64 do, but the longest
     // workgroup sets the time: with few workgroups the smaller ones spread better over the compute units.
     // Where most keys were cached before the step (max_context, the caller's hint of the longest context a
@@ -503,22 +559,33 @@ static int launch_prefill_lds(const void* q, int64_t q_stride, const void* kc, c
     const int64_t wide_groups = (int64_t)ceil_div(max_entry_len, 128) * n_entries * nq;
     int reach = max_context;
     if (window > 0 && reach > window + max_entry_len) reach = window + max_entry_len;
-    const bool wide = wide_groups >= PREFILL_WIDE_GROUPS ||
-                      (wide_groups >= PREFILL_WIDE_GROUPS_CACHED && reach >= 2 * max_entry_len);
+    bool wide = wide_groups >= PREFILL_WIDE_GROUPS ||
+                (wide_groups >= PREFILL_WIDE_GROUPS_CACHED && reach >= 2 * max_entry_len);
+    if (shape != PREFILL_SHAPE_AUTO) wide = shape == PREFILL_SHAPE_WIDE;
     const dim3 grid(nq, n_entries, ceil_div(max_entry_len, wide ? 128 : 64));
     const size_t page_list = (size_t)prefill_page_entries(max_blocks, page_size, window) * sizeof(int);
     if (wide) {
         if (page_list > 16 * 1024)                       // with the tiles beyond the default limit of LDS
-            (void)hipFuncSetAttribute((const void*)attention_prefill_lds_kernel<DT, 2>,
+            (void)hipFuncSetAttribute((const void*)attention_prefill_lds_kernel<DT, 2, 1>,
                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)page_list);
-        hipLaunchKernelGGL((attention_prefill_lds_kernel<DT, 2>), grid, dim3(256), page_list, stream, (const bf16*)q,
+        hipLaunchKernelGGL((attention_prefill_lds_kernel<DT, 2, 1>), grid, dim3(256), page_list, stream, (const bf16*)q,
+                           q_stride, (const bf16*)kc, (const bf16*)vc, block_table, max_blocks, entry_start,
+                           entry_first_pos, nq, nkv, page_size, window, scale * 1.44269504088896341f, (bf16*)out);
+    } else if (shape == PREFILL_SHAPE_AUTO
+                   ? (int64_t)grid.x * grid.y * grid.z < PREFILL_KEY_SPLIT_BELOW && reach >= PREFILL_KEY_SPLIT_REACH
+                   : shape == PREFILL_SHAPE_SPLIT) {
+        // few workgroups with many tiles each: the keys of a query block are split over two wavefronts
+        if (page_list > 16 * 1024)
+            (void)hipFuncSetAttribute((const void*)attention_prefill_lds_kernel<DT, 1, 2>,
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)page_list);
+        hipLaunchKernelGGL((attention_prefill_lds_kernel<DT, 1, 2>), grid, dim3(512), page_list, stream, (const bf16*)q,
                            q_stride, (const bf16*)kc, (const bf16*)vc, block_table, max_blocks, entry_start,
                            entry_first_pos, nq, nkv, page_size, window, scale * 1.44269504088896341f, (bf16*)out);
     } else {
         if (page_list > 16 * 1024)
-            (void)hipFuncSetAttribute((const void*)attention_prefill_lds_kernel<DT, 1>,
+            (void)hipFuncSetAttribute((const void*)attention_prefill_lds_kernel<DT, 1, 1>,
                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)page_list);
-        hipLaunchKernelGGL((attention_prefill_lds_kernel<DT, 1>), grid, dim3(256), page_list, stream, (const bf16*)q,
+        hipLaunchKernelGGL((attention_prefill_lds_kernel<DT, 1, 1>), grid, dim3(256), page_list, stream, (const bf16*)q,
                            q_stride, (const bf16*)kc, (const bf16*)vc, block_table, max_blocks, entry_start,
                            entry_first_pos, nq, nkv, page_size, window, scale * 1.44269504088896341f, (bf16*)out);
     }
@@ -546,17 +613,19 @@ static int launch_prefill(const void* q, int64_t q_stride, const void* kc, const
 // first token; max_entry_len: the longest portion (sizes the grid).  bfloat16 only; head_dim a multiple of 16
 // up to 256; page_size a multiple of 4.  k_cache [pages, nkv, page_size, D], v_cache [pages, nkv, D, page_size];
 // out: [n_tokens, nq * D].  max_context: the longest context a portion ends at (a hint for the launch shape; 0: unknown).
+// shape: 0 lets the launcher choose; 1..3 ask for a launch shape of the LDS kernel (PREFILL_SHAPE_*).
 extern "C" int somi_attention_prefill(const void* q, int64_t q_stride, const void* k_cache, const void* v_cache,
                                       const int* block_table, int max_blocks, const int* entry_start,
                                       const int* entry_first_pos, int n_entries, int max_entry_len, int max_context,
-                                      int nq, int nkv, int D, int page_size, int window, float scale, void* out,
-                                      hipStream_t stream) {
+                                      int shape, int nq, int nkv, int D, int page_size, int window, float scale,
+                                      void* out, hipStream_t stream) {
     SOMI_REQUIRE(n_entries >= 0 && max_entry_len >= 0 && nq > 0 && nkv > 0 && max_blocks > 0,
                  "attention_prefill: bad sizes");
     SOMI_REQUIRE(nq % nkv == 0, "attention_prefill: num_q_heads (%d) must be divisible by num_kv_heads (%d)", nq, nkv);
     SOMI_REQUIRE(D % 16 == 0 && D >= 16 && D <= 256, "attention_prefill: head_dim %d must be a multiple of 16 up to 256", D);
     SOMI_REQUIRE(page_size > 0 && page_size % 4 == 0, "attention_prefill: page size %d must be a multiple of 4", page_size);
     SOMI_REQUIRE(window >= 0, "attention_prefill: window must be >= 0");
+    SOMI_REQUIRE(shape >= PREFILL_SHAPE_AUTO && shape <= PREFILL_SHAPE_WIDE, "attention_prefill: unknown launch shape %d", shape);
     SOMI_REQUIRE(n_entries <= 65535 && nq <= 65535, "attention_prefill: too many entries or heads");
     SOMI_REQUIRE(max_entry_len <= 65535 * 128, "attention_prefill: a portion of %d tokens is too long", max_entry_len);
     SOMI_REQUIRE((uintptr_t)q % 16 == 0 && (q_stride * 2) % 16 == 0 && (uintptr_t)k_cache % 16 == 0 &&
@@ -575,8 +644,8 @@ extern "C" int somi_attention_prefill(const void* q, int64_t q_stride, const voi
                                          entry_first_pos, n_entries, max_entry_len, nq, nkv, page_size, window,    \
                                          scale, out, stream);                                                      \
         return launch_prefill_lds<DT>(q, q_stride, k_cache, v_cache, block_table, max_blocks, entry_start,         \
-                                      entry_first_pos, n_entries, max_entry_len, max_context, nq, nkv, page_size,   \
-                                      window, scale, out, stream)
+                                      entry_first_pos, n_entries, max_entry_len, max_context, shape, nq, nkv,      \
+                                      page_size, window, scale, out, stream)
     // head sizes 32..128 stage keys and values through LDS; the others (LDS would not hold two tiles, or a
     // tile is smaller than the workgroup's loads) keep them in registers per wavefront, and so do page sizes
     // that are no power of two and block tables too wide for the LDS copy of a request's pages

@@ -241,11 +241,12 @@ def attention_decode(q: torch.Tensor, q_stride: int, k_cache: torch.Tensor, v_ca
 def attention_prefill(q: torch.Tensor, q_stride: int, k_cache: torch.Tensor, v_cache: torch.Tensor,
                       block_table: torch.Tensor, entry_start: torch.Tensor, entry_first_position: torch.Tensor,
                       max_entry_len: int, nq: int, window: int, scale: float, out: torch.Tensor,
-                      max_context: int = 0) -> None:
+                      max_context: int = 0, shape: int = 0) -> None:
     """MFMA causal attention of every token of every portion over its request's pages, into ``out``
     ([N, nq * D] bfloat16).  entry_start: [E + 1] int32 offsets of the portions in the flat batch;
     entry_first_position: [E] int32.  ``max_context``: the longest context a portion ends at, a hint for the
-    launch shape (0: unknown)."""
+    launch shape (0: unknown).  ``shape``: 0 lets the launcher choose; 1 (64 queries a workgroup), 2 (the same
+    with a query block's keys split over two wavefronts) or 3 (128 queries) asks for that shape of the LDS kernel."""
     _need(q, "q", torch.bfloat16)
     n = q.shape[0]
     _need(k_cache, "k cache", torch.bfloat16)
@@ -264,7 +265,7 @@ def attention_prefill(q: torch.Tensor, q_stride: int, k_cache: torch.Tensor, v_c
         raise KernelError(f"attention_prefill: longest portion {max_entry_len} does not fit {n} tokens")
     _check(library().somi_attention_prefill(
         _ptr(q), ctypes.c_int64(q_stride), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), block_table.shape[1],
-        _ptr(entry_start), _ptr(entry_first_position), entries, max_entry_len, max(0, int(max_context)), nq, nkv,
+        _ptr(entry_start), _ptr(entry_first_position), entries, max_entry_len, max(0, int(max_context)), int(shape), nq, nkv,
         head_dim, page_size, window, ctypes.c_float(scale), _ptr(out), _stream()))
 
 

@@ -316,9 +316,11 @@ def test_attention_decode_refuses_what_it_cannot_do():
 @pytest.mark.parametrize("nq, nkv, d, page, window", [
     (8, 4, 32, 4, 0), (12, 2, 64, 16, 0), (8, 1, 48, 8, 0), (6, 3, 128, 16, 37), (28, 4, 128, 16, 0),
     (4, 2, 16, 8, 0), (14, 2, 256, 16, 0), (5, 5, 80, 4, 5), (7, 1, 112, 32, 100), (3, 1, 208, 16, 0)])
-def test_attention_prefill_mfma_against_dense_softmax(nq, nkv, d, page, window):
+@pytest.mark.parametrize("shape", [0, 1, 2, 3], ids=["auto", "narrow", "split", "wide"])
+def test_attention_prefill_mfma_against_dense_softmax(nq, nkv, d, page, window, shape):
     """Portions of several requests in one launch: a long one that starts at position 0, one that continues
-    after 150 cached tokens, a portion of two tokens, single tokens after 77 and after 0 cached ones."""
+    after 150 cached tokens, a portion of two tokens, single tokens after 77 and after 0 cached ones.  Each
+    launch shape of the kernel that stages tiles through LDS is asked for in turn."""
     cached, new = [0, 150, 30, 77, 0], [203, 130, 2, 1, 1]
     total = [c + n for c, n in zip(cached, new)]
     n_pages = sum((t + page - 1) // page for t in total) + 3
@@ -347,7 +349,8 @@ def test_attention_prefill_mfma_against_dense_softmax(nq, nkv, d, page, window):
         starts.append(starts[-1] + k)
     scale = d ** -0.5
     out = torch.full((n, nq * d), float("nan"), dtype=torch.bfloat16, device=DEV)
-    ops.attention_prefill(q, nq * d, kc, vc, block_table, i32(starts), i32(cached), max(new), nq, window, scale, out)
+    ops.attention_prefill(q, nq * d, kc, vc, block_table, i32(starts), i32(cached), max(new), nq, window, scale, out,
+                          shape=shape)
     qh = q.float().view(n, nq, d).cpu()
     want, at = [], 0
     for e, k in enumerate(new):
