@@ -15,6 +15,7 @@ import ctypes
 import hashlib
 import os
 import shutil
+import stat
 import subprocess
 import sys
 import tempfile
@@ -67,9 +68,22 @@ def _candidate_dirs() -> list[str]:
     return dirs
 
 
+def _own_private(path: str) -> bool:
+    """A build folder under the shared temporary folder counts only if it is ours and closed to others."""
+    if os.path.dirname(path) == CSRC or not hasattr(os, "getuid"):
+        return True
+    try:
+        info = os.lstat(path)
+    except OSError:
+        return False
+    return stat.S_ISDIR(info.st_mode) and info.st_uid == os.getuid() and not (info.st_mode & 0o022)
+
+
 def _writable(path: str) -> bool:
     try:
-        os.makedirs(path, exist_ok=True)
+        os.makedirs(path, mode=0o700, exist_ok=True)
+        if not _own_private(path):
+            return False
         probe = os.path.join(path, f".probe_{os.getpid()}")
         with open(probe, "w"):
             pass
@@ -84,18 +98,10 @@ def built_library() -> str | None:
     want = source_digest()
     for folder in _candidate_dirs():
         lib, stamp = os.path.join(folder, LIB_NAME), os.path.join(folder, "digest.txt")
-        if os.path.isfile(lib) and os.path.isfile(stamp):
+        if _own_private(folder) and os.path.isfile(lib) and os.path.isfile(stamp):
             with open(stamp, "r", encoding="utf-8") as handle:
                 if handle.read().strip() == want:
                     return lib
-    return None
-
-
-def any_library() -> str | None:
-    for folder in _candidate_dirs():
-        lib = os.path.join(folder, LIB_NAME)
-        if os.path.isfile(lib):
-            return lib
     return None
 
 
