@@ -453,3 +453,30 @@ def repetition_penalty(logits_row: torch.Tensor, ids: torch.Tensor, penalty: flo
     _need(ids, "penalised ids", torch.int32)
     _check(library().somi_repetition_penalty(_ptr(logits_row), logits_row.numel(), _ptr(ids), ids.numel(),
                                              ctypes.c_float(penalty), _stream()))
+
+
+def repetition_penalty_rows(logits: torch.Tensor, offsets: torch.Tensor, ids: torch.Tensor, penalties: torch.Tensor,
+                            most_ids: int) -> None:
+    """In place on [rows, vocab] float32 logits: row r's distinct ids are ids[offsets[r]:offsets[r + 1]], its
+    penalty penalties[r] (1 leaves the row alone).  ``most_ids``: the largest number of ids a row has."""
+    _need(logits, "logits", torch.float32)
+    rows, vocab = logits.shape
+    _need(offsets, "penalty offsets", torch.int32, (rows + 1,))
+    _need(ids, "penalised ids", torch.int32)
+    _need(penalties, "penalties", torch.float32, (rows,))
+    if most_ids < 0 or most_ids > ids.numel():
+        raise KernelError(f"repetition_penalty_rows: most_ids={most_ids} does not fit {ids.numel()} ids")
+    _check(library().somi_repetition_penalty_rows(_ptr(logits), rows, vocab, _ptr(offsets), _ptr(ids), _ptr(penalties),
+                                                  int(most_ids), _stream()))
+
+
+def sample_filter(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor) -> None:
+    """Top-k, then top-p on softmax(logits / T), in place on [rows, vocab] float32 logits: what a rule removes
+    becomes -inf.  top_k: int32 (-1: off), top_p: float32 (1: off); rows with temperature 0 are left alone."""
+    _need(logits, "logits", torch.float32)
+    rows, vocab = logits.shape
+    _need(temperature, "temperature", torch.float32, (rows,))
+    _need(top_k, "top_k", torch.int32, (rows,))
+    _need(top_p, "top_p", torch.float32, (rows,))
+    _check(library().somi_sample_filter(_ptr(logits), rows, vocab, _ptr(temperature), _ptr(top_k), _ptr(top_p),
+                                        _stream()))

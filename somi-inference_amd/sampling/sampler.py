@@ -3,8 +3,8 @@
 Reference: ``Sampler.sample`` (somi_inference/core/sampler.py:31-55): clone,
 repetition penalty, temperature, top-k, top-p, then argmax (temperature 0) or a
 draw from the float32 softmax (:159-176).  The order and every rule are kept.
-Penalty, the temperature scaling, the softmax and the pick run in HIP kernels;
-the top-k and top-p masks use the library's ``topk``/``sort`` on the device.
+Penalty, top-k, top-p, the temperature scaling, the softmax and the pick run in
+HIP kernels (top-k and top-p by a radix search for the cut value, without a sort).
 The draw is by inverse CDF from the request's own counter-based uniform number
 instead of ``torch.multinomial`` on the global generator, so the distribution is
 the reference's and the stream is the request's own.
@@ -36,29 +36,40 @@ class Sampler:
 
     def __init__(self) -> None:
         self._greedy_inputs: dict[tuple[int, torch.device], torch.Tensor] = {}
-        self._host_rings: dict[tuple[int, torch.dtype], tuple[list[torch.Tensor], list[int]]] = {}
+        self._host_rings: dict[tuple[str, int, torch.dtype], tuple[list[torch.Tensor], list[int]]] = {}
 
-    def _host_buffer(self, size: int, dtype: torch.dtype) -> torch.Tensor:
-        """Pinned host memory, a few buffers per size in turn: copies to and from it do not wait for the device."""
+    def _host_buffer(self, purpose: str, size: int, dtype: torch.dtype) -> torch.Tensor:
+        """Pinned host memory, a few buffers per purpose and size in turn: copies to and from it do not wait for
+        the device."""
         ring, turn = self._host_rings.setdefault(
-            (size, dtype), ([torch.empty(size, dtype=dtype).pin_memory() for _ in range(self.RING)], [0]))
+            (purpose, size, dtype), ([torch.empty(size, dtype=dtype).pin_memory() for _ in range(self.RING)], [0]))
         turn[0] = (turn[0] + 1) % self.RING
         return ring[turn[0]]
 
-    def _pick_inputs(self, plist: list[SamplingParams], seeds: list[int], counters: list[int],
-                     device: torch.device) -> tuple[torch.Tensor, torch.Tensor]:
-        """Temperatures and uniform draws of the rows on the device, in one transfer (none for all-greedy rows)."""
+    def _staged(self, values: list, dtype: torch.dtype, device: torch.device) -> torch.Tensor:
+        """``values`` on the device through pinned memory (buffers come in power-of-two sizes, so that a few serve
+        every length)."""
+        capacity = 64
+        while capacity < len(values):
+            capacity *= 2
+        staged = self._host_buffer("in", capacity, dtype)
+        staged[:len(values)].copy_(torch.tensor(values, dtype=dtype))
+        return staged.to(device, non_blocking=True)[:len(values)]
+
+    def _row_inputs(self, plist: list[SamplingParams], seeds: list[int], counters: list[int],
+                    device: torch.device) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+        """Temperatures, uniform draws, top-p values and penalties of the rows on the device, in one transfer (none
+        for all-greedy rows, which read neither of the last three)."""
         rows = len(plist)
-        if all(p.temperature == 0.0 for p in plist):
+        if all(p.temperature == 0.0 and p.repetition_penalty == 1.0 for p in plist):
             held = self._greedy_inputs.get((rows, device))
             if held is None:
-                held = self._greedy_inputs[(rows, device)] = torch.zeros(2 * rows, dtype=torch.float32, device=device)
+                held = self._greedy_inputs[(rows, device)] = torch.zeros(4 * rows, dtype=torch.float32, device=device)
         else:
-            staged = self._host_buffer(2 * rows, torch.float32)
-            staged.copy_(torch.tensor([p.temperature for p in plist] + [uniform(s, c) for s, c in zip(seeds, counters)],
-                                      dtype=torch.float32))
-            held = staged.to(device, non_blocking=True)
-        return held[:rows], held[rows:]
+            held = self._staged([p.temperature for p in plist] + [uniform(s, c) for s, c in zip(seeds, counters)]
+                                + [p.top_p for p in plist] + [p.repetition_penalty for p in plist],
+                                torch.float32, device)
+        return held[:rows], held[rows:2 * rows], held[2 * rows:3 * rows], held[3 * rows:]
 
     def sample(self, logits: torch.Tensor, params: SamplingParams | list[SamplingParams],
                token_histories: list[list[int]] | None = None,
@@ -97,29 +108,24 @@ class Sampler:
             work = work.float()
         work = work.contiguous()
 
-        for row, (p, history) in enumerate(zip(plist, histories)):
+        temperature, draws, top_p, penalties = self._row_inputs(plist, seeds, counters, work.device)
+        filters = any(p.temperature > 0.0 and (p.top_k != -1 or p.top_p != 1.0) for p in plist)
+        # the rows' integers in one transfer: top-k values, then where each row's penalised ids start, then the ids
+        offsets, ids, most = [0], [], 0
+        for p, history in zip(plist, histories):
             if p.repetition_penalty != 1.0 and history:
-                ids = torch.tensor(sorted(set(int(t) for t in history)), dtype=torch.int32, device=work.device)
-                ops.repetition_penalty(work[row], ids, p.repetition_penalty)
-        for row, p in enumerate(plist):
-            if p.temperature == 0.0:
-                continue                    # greedy ignores top-k / top-p (sampler.py:123, 142)
-            if p.top_k != -1:
-                keep = torch.topk(work[row], k=min(p.top_k, vocab)).indices
-                masked = torch.full_like(work[row], float("-inf"))
-                masked[keep] = work[row][keep]
-                work[row] = masked
-            if p.top_p != 1.0:
-                ordered, order = torch.sort(work[row] / p.temperature, descending=True)
-                cumulative = torch.cumsum(torch.softmax(ordered, dim=-1, dtype=torch.float32), dim=-1)
-                remove = cumulative > p.top_p
-                remove[1:] = remove[:-1].clone()     # the entry that crosses p stays (sampler.py:151-153)
-                remove[0] = False
-                work[row, order[remove]] = float("-inf")
-
-        temperature, draws = self._pick_inputs(plist, seeds, counters, work.device)
+                distinct = set(history)
+                ids.extend(distinct)
+                most = max(most, len(distinct))
+            offsets.append(len(ids))
+        if filters or most:
+            ints = self._staged([p.top_k for p in plist] + offsets + ids, torch.int32, work.device)
+            if most:
+                ops.repetition_penalty_rows(work, ints[rows:2 * rows + 1], ints[2 * rows + 1:], penalties, most)
+            if filters:
+                ops.sample_filter(work, temperature, ints[:rows], top_p)
         picked = ops.sample(work, temperature, draws)
-        host = self._host_buffer(rows, torch.int32)
+        host = self._host_buffer("out", rows, torch.int32)
         host.copy_(picked, non_blocking=True)
         copied = torch.cuda.Event()
         copied.record()

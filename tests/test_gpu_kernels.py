@@ -219,6 +219,84 @@ def test_repetition_penalty_rule():
         ops.repetition_penalty(row, i32([0]), 0.0)
 
 
+def test_repetition_penalty_of_several_rows_in_one_launch():
+    logits = rnd(4, 777, seed=21, scale=3.0)
+    histories = [[5, 5, 9, 700], [], list(range(0, 777, 3)), [776, 0]]
+    penalties = [2.0, 1.7, 0.5, 1.0]                       # row 1 has no ids, row 3 a penalty of 1: both stay
+    offsets, ids = [0], []
+    for history in histories:
+        ids += sorted(set(history))
+        offsets.append(len(ids))
+    work = logits.clone()
+    ops.repetition_penalty_rows(work, i32(offsets), i32(ids), torch.tensor(penalties, device=DEV),
+                                max(len(set(h)) for h in histories))
+    for row in range(4):
+        want = plain.penalize_repetition(logits[row].cpu(), histories[row], penalties[row])
+        assert torch.equal(work[row].cpu(), want), f"row {row}"
+
+
+def _midpoint_p(z: torch.Tensor, rank: int) -> float:
+    """A top-p value halfway between the cumulative probabilities of the entries of rank ``rank`` and ``rank + 1`` of
+    softmax(z), so that rounding in a cumulative sum cannot move the cut."""
+    cumulative = torch.cumsum(torch.softmax(torch.sort(z.double(), descending=True).values, dim=-1), dim=-1)
+    return float((cumulative[rank] + cumulative[rank + 1]) / 2)
+
+
+@pytest.mark.parametrize("vocab", [5, 1237, 152064 // 8 + 5, 152064])
+def test_top_k_and_top_p_masks_against_the_sorted_rule(vocab):
+    """Rows of one launch with different rules: greedy (untouched), top-k, top-p, both, neither."""
+    logits = rnd(6, vocab, seed=30 + vocab % 7, scale=2.0)
+    temps = [0.0, 0.8, 1.3, 0.7, 1.0, 0.9]
+    ks = [2, min(50, vocab - 1), -1, min(300, vocab - 1), vocab + 5, 1]
+    host = logits.cpu()
+    ps = [0.3, 1.0, _midpoint_p(host[2] / temps[2], min(40, vocab - 2)), 0.0, 1.0, 0.5]
+    # row 3: the p sits between two entries of what top-k left
+    ps[3] = _midpoint_p(plain.keep_top_k(host[3] / temps[3], ks[3]), min(17, vocab - 2))
+    work = logits.clone()
+    ops.sample_filter(work, torch.tensor(temps, device=DEV), i32(ks), torch.tensor(ps, device=DEV))
+    got = work.cpu()
+    for row in range(6):
+        if temps[row] == 0.0:
+            want = host[row]
+        else:
+            scaled = plain.keep_top_p(plain.keep_top_k(host[row] / temps[row], ks[row]), ps[row])
+            want = torch.where(torch.isinf(scaled), scaled, host[row])
+        assert torch.equal(got[row], want), (
+            f"row {row}: kept {int((~torch.isinf(got[row])).sum())}, expected {int((~torch.isinf(want)).sum())}")
+    # the masked rows go on into the draw: it lands on a kept entry
+    picks = ops.sample(work, torch.tensor(temps, device=DEV), torch.full((6,), 0.999, device=DEV)).tolist()
+    assert all(not math.isinf(got[row, picks[row]]) for row in range(6))
+
+
+def test_top_k_and_top_p_masks_with_equal_entries():
+    # reference test_sampler.py:96-106: exactly k survive also where the k-th value is shared
+    row = torch.tensor([[5.0, 4.0, 4.0, 1.0]], device=DEV)
+    one = torch.ones(1, device=DEV)
+    work = row.clone()
+    ops.sample_filter(work, one, i32([2]), one)
+    assert work[0].tolist() == [5.0, 4.0, -math.inf, -math.inf]          # of equal entries the earlier ones stay
+    # :108-128: softmax of 4, 3, 2, 1 is 0.64, 0.24, ...: p = 0.5 keeps the first entry only, p = 0.7 the first two
+    for p, kept in [(0.5, 1), (0.7, 2), (0.9, 3), (0.99, 4)]:
+        work = torch.tensor([[4.0, 3.0, 2.0, 1.0]], device=DEV)
+        ops.sample_filter(work, one, i32([-1]), torch.tensor([p], device=DEV))
+        assert int((~torch.isinf(work)).sum()) == kept, p
+    # many shared values (logits in steps of 0.5, negative ones and both zeros among them): the number kept and the
+    # values kept are those of the sorted rule, whichever of the equal entries a sort would have put first
+    gen = torch.Generator().manual_seed(5)
+    coarse = (torch.randn(3, 6000, generator=gen) * 2.0 / 0.5).round() * 0.5
+    coarse[0, 17] = -0.0
+    temps = torch.tensor([1.0, 0.5, 2.0], device=DEV)
+    for ks, ps in [([40, 700, 5999], [1.0, 1.0, 1.0]), ([-1, -1, -1], [0.35, 0.8, 0.97]), ([100, 2000, 30], [0.6, 0.9, 0.2])]:
+        work = coarse.to(DEV)
+        ops.sample_filter(work, temps, i32(ks), torch.tensor(ps, device=DEV))
+        for r in range(3):
+            scaled = coarse[r] / temps[r].item()
+            want = plain.keep_top_p(plain.keep_top_k(scaled, ks[r]), ps[r])
+            kept_got = torch.sort(scaled[~torch.isinf(work[r].cpu())]).values
+            kept_want = torch.sort(want[~torch.isinf(want)]).values
+            assert kept_got.shape == kept_want.shape and torch.equal(kept_got, kept_want), (r, ks, ps)
+
+
 @pytest.mark.parametrize("m, n, k", [(1, 503, 192), (7, 64, 72), (16, 130, 200), (17, 33, 1000), (48, 3584 + 16, 3584),
                                      (64, 70, 18944), (8, 152064 // 16 + 3, 512), (2, 32768 + 16, 128), (20, 65536 + 48, 64)])
 def test_linear_skinny_mfma_against_float32(m, n, k):
