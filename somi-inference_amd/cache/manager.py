@@ -97,6 +97,13 @@ class CacheManager:
         self._requests: dict[Hashable, RequestCache] = {}
         self._free_slots = list(range(self.max_requests - 1, -1, -1))
 
+    @staticmethod
+    def page_bytes(needs: list, block_size: int, dtype: torch.dtype) -> int:
+        """Bytes of device memory that one more page per group costs: keys and values of every run that writes."""
+        item = torch.empty((), dtype=dtype).element_size()
+        return sum(2 * need.num_kv_heads * need.head_dim * int(block_size) * item
+                   for need in needs if isinstance(need, PagedKVSpec))
+
     # --------------------------------------------------------------- requests
     def has(self, request_id: Hashable) -> bool:
         return request_id in self._requests

@@ -26,7 +26,10 @@ def parse_args(argv: list[str] | None = None) -> argparse.Namespace:
     parser.add_argument("--config-json", type=str, default=None,
                         help="A config.json to make random weights for (with --write-random-model).")
     parser.add_argument("--random-seed", type=int, default=0, help="Seed of the random weights.")
-    parser.add_argument("--num-blocks", type=int, default=256, help="Total KV cache blocks.")
+    parser.add_argument("--num-blocks", type=int, default=256,
+                        help="Total KV cache blocks. 0: as many as fit into --memory-fraction of the free memory.")
+    parser.add_argument("--memory-fraction", type=float, default=0.9,
+                        help="Share of the free device memory that --num-blocks 0 fills with cache blocks.")
     parser.add_argument("--block-size", type=int, default=16, help="KV cache block size.")
     parser.add_argument("--max-concurrent", type=int, default=16, help="Scheduler max concurrent sequences.")
     parser.add_argument("--max-num-batched-tokens", type=int, default=2048, help="Token budget of one step.")
@@ -70,7 +73,8 @@ def main(argv: list[str] | None = None) -> int:
     if not model_dir:
         return _usage_error("give --model-name (or --write-random-model with --config-json)")
     from .llm import LLM
-    llm = LLM(model_dir, num_blocks=args.num_blocks, block_size=args.block_size,
+    llm = LLM(model_dir, num_blocks=args.num_blocks or None, memory_fraction=args.memory_fraction,
+              block_size=args.block_size,
               max_concurrent=args.max_concurrent, device=args.device, dtype=args.dtype,
               max_num_batched_tokens=args.max_num_batched_tokens, max_chunk=args.max_chunk, seed=args.seed)
     if args.warm_up:

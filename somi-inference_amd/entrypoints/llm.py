@@ -14,6 +14,7 @@ from __future__ import annotations
 
 import os
 from collections import deque
+from dataclasses import replace
 from typing import Iterator, Sequence
 
 import torch
@@ -37,7 +38,7 @@ class LLM:
         self,
         model_name: str | ModelConfig,
         *,
-        num_blocks: int = DEFAULT_NUM_BLOCKS,
+        num_blocks: int | None = DEFAULT_NUM_BLOCKS,
         block_size: int = DEFAULT_BLOCK_SIZE,
         max_concurrent: int = DEFAULT_MAX_CONCURRENT,
         device: torch.device | str | None = None,
@@ -47,14 +48,17 @@ class LLM:
         seed: int = 0,
         random_seed: int | None = None,
         eos_token_id: int | None = None,
+        memory_fraction: float = 0.9,
     ) -> None:
         """``model_name``: a model folder (config.json + model.safetensors), or a typed
-        configuration together with ``random_seed`` for seeded random weights."""
+        configuration together with ``random_seed`` for seeded random weights.  ``num_blocks=None``
+        (not in the reference): as many cache pages as fit into ``memory_fraction`` of the device memory that
+        is free once the weights are loaded."""
         device = torch.device(device) if device is not None else torch.device("cuda:0")
         if device.type == "cuda" and device.index is None:
             device = torch.device("cuda:0")
         self.options = EngineConfig(dtype=str(dtype).replace("torch.", ""), block_size=block_size,
-                                    num_blocks=num_blocks, max_concurrent=max_concurrent,
+                                    num_blocks=1 if num_blocks is None else num_blocks, max_concurrent=max_concurrent,
                                     max_num_batched_tokens=max_num_batched_tokens, max_chunk=max_chunk,
                                     device=str(device))
         self.device, self.dtype, self.seed = device, self.options.dtype, int(seed)
@@ -70,7 +74,9 @@ class LLM:
             if has_tokenizer_files(model_dir):
                 self.tokenizer = Tokenizer(model_dir)
         self.runner = make_runner(self.model, block_size=block_size, num_blocks=num_blocks,
-                                  max_requests=max_concurrent)
+                                  max_requests=max_concurrent, memory_fraction=memory_fraction)
+        if num_blocks is None:
+            self.options = replace(self.options, num_blocks=self.runner.cache.num_blocks)
         self.kv_manager = self.runner.cache
         self.sampler = Sampler()
         self.scheduler = Scheduler(self.runner.cache, max_concurrent=max_concurrent,

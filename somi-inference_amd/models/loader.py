@@ -53,7 +53,26 @@ def random_model(config: ModelConfig, seed: int, dtype: object = "bfloat16",
     return model
 
 
-def make_runner(model: DecoderModel, *, block_size: int, num_blocks: int, max_requests: int) -> ModelRunner:
+def pages_that_fit(model: DecoderModel, block_size: int, memory_fraction: float = 0.9) -> int:
+    """How many cache pages per group fit into ``memory_fraction`` of the device memory that is free now (after
+    the weights): the pool of a GPU with hundreds of gigabytes is sized by its memory, not by a constant."""
+    if not 0.0 < memory_fraction <= 1.0:
+        raise ValueError(f"memory_fraction must be in (0, 1], got {memory_fraction}")
+    per_page = CacheManager.page_bytes(model.cache_needs(), block_size, model.runtime.dtype)
+    if per_page == 0:
+        return 1
+    free, _ = torch.cuda.mem_get_info(model.runtime.device)
+    pages = int(free * memory_fraction) // per_page
+    if pages < 1:
+        raise RuntimeError(f"no cache page of {per_page} bytes fits into {memory_fraction:.2f} of the {free} free bytes")
+    return pages
+
+
+def make_runner(model: DecoderModel, *, block_size: int, num_blocks: int | None, max_requests: int,
+                memory_fraction: float = 0.9) -> ModelRunner:
+    """``num_blocks=None``: as many pages as fit into ``memory_fraction`` of the free device memory."""
+    if num_blocks is None:
+        num_blocks = pages_that_fit(model, block_size, memory_fraction)
     cache = CacheManager(model.cache_needs(), block_size=block_size, num_blocks=num_blocks,
                          max_requests=max_requests, dtype=model.runtime.dtype, device=model.runtime.device)
     return ModelRunner(model, cache)

@@ -104,6 +104,22 @@ def test_entry_point_options_and_errors(model_folders):
         LLM(model_folders["A"], device="cpu")
 
 
+def test_page_pool_sized_by_the_free_memory(model_folders):
+    from somi_inference_amd.cache import CacheManager
+    fixed = LLM(model_folders["B"], dtype="bfloat16", num_blocks=64, block_size=8)
+    free, _ = torch.cuda.mem_get_info()
+    sized = LLM(model_folders["B"], dtype="bfloat16", num_blocks=None, memory_fraction=0.001, block_size=8)
+    per_page = CacheManager.page_bytes(sized.model.cache_needs(), 8, torch.bfloat16)
+    cfg = TINY["B"]["config"]
+    assert per_page == cfg.num_hidden_layers * 2 * cfg.num_key_value_heads * cfg.head_dim * 8 * 2
+    pages = sized.kv_manager.num_blocks
+    assert pages == sized.options.num_blocks and 0.5 * free * 0.001 / per_page < pages <= free * 0.001 / per_page
+    prompts = [token_ids(cfg.vocab_size, n, 70 + n) for n in (9, 40)]
+    assert sized.generate(prompts, max_new_tokens=6, temperature=0.0) == fixed.generate(prompts, max_new_tokens=6, temperature=0.0)
+    with pytest.raises(ValueError, match="memory_fraction"):
+        LLM(model_folders["B"], dtype="bfloat16", num_blocks=None, memory_fraction=0.0)
+
+
 def test_sampler_rules_on_the_gpu():
     sampler, dev = Sampler(), "cuda:0"
     t = lambda rows: torch.tensor(rows, dtype=torch.float32, device=dev)

@@ -123,6 +123,19 @@ def test_mixed_batches_with_so_few_pages_that_they_are_used_again(name, dtype, p
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+def test_pages_beyond_two_to_the_31_elements_of_a_cache_tensor(dtype, peaky_folders, oracle):
+    """A pool sized for a large GPU: the pool hands out its highest pages first, so the first request's keys
+    and values lie past 2^31 elements of their tensors, where a 32-bit offset would wrap."""
+    config, bs = TINY["A"]["config"], TINY["A"]["block_size"]
+    per_page = config.num_key_value_heads * config.head_dim * bs
+    pages = (1 << 31) // per_page + 64
+    runner, _ = make_engine(peaky_folders["A"], dtype, bs, pages)
+    tokens = token_ids(config.vocab_size, 120, 9)
+    got = run_portions(runner, "far", tokens, [70, 9, 9] + [1] * 32)
+    assert_close(got, oracle("peaky", "A", tokens), dtype, f"A {dtype} in the highest pages of {pages}")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("name", ["B", "C"])
 def test_long_decoding_from_a_short_prompt(name, dtype, peaky_folders, oracle):
     vocab, bs = TINY[name]["config"].vocab_size, TINY[name]["block_size"]
