@@ -6,7 +6,8 @@ import torch
 
 from . import ops
 
-TARGET_WORKGROUPS = 512         # about two per compute unit (measured best at 8 requests x 4,096 keys)
+TARGET_WORKGROUPS = 256         # one per compute unit (whole decode steps at 4,096 keys, 7B sizes: 8 / 16 / 32 / 64 requests
+                                # 3.42 / 3.99 / 5.27 / 7.20 ms against 3.43 / 4.05 / 5.39 / 7.29 with 512; 192 and 128 are slower)
 MIN_SPLIT = 64                  # keys per split at least (a multiple of the 16-key tile)
 MAX_SPLITS = 1024               # what the merge kernel holds
 DECODE_PORTION = 8              # batches whose longest portion is at most this take the decode kernel
