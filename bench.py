@@ -185,6 +185,8 @@ def main() -> int:
                                      new_tokens, greedy, seed=i)) for i, n in enumerate(lengths))
         if tuned:
             runner.tune_library_products(512)
+        # as LLM.warm_up() does it: the decode graphs that the requests will replay are captured before they arrive
+        captured = runner.capture_decode_graphs(concurrent, 2048 + new_tokens)
         sync()
         start = time.perf_counter()
         done = engine.run(arrivals)
@@ -195,7 +197,7 @@ def main() -> int:
                    "seconds": round(seconds, 3), "generated_tok_s": round(generated / seconds, 1),
                    "total_tok_s": round((generated + sum(lengths)) / seconds, 1), "steps": engine.num_steps,
                    "steps_run_ahead": engine.steps_run_ahead, "max_concurrent": concurrent,
-                   "preemptions": sum(r.num_preemptions for r in done)}
+                   "preemptions": sum(r.num_preemptions for r in done), "graphs_captured_ahead": captured}
 
     line = {
         "metric": f"decode tok/s at batch {args.batch}, Qwen2.5-{args.sizes.upper()} layer sizes "

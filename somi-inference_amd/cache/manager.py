@@ -85,7 +85,8 @@ class CacheManager:
             elif isinstance(need, FixedStateSpec):
                 state = None
                 if allocate_tensors:
-                    state = torch.zeros((self.max_requests, *need.shape), dtype=need.dtype, device=self.device)
+                    # one row more than there are requests: the slot that padding entries of a step use
+                    state = torch.zeros((self.max_requests + 1, *need.shape), dtype=need.dtype, device=self.device)
                 self.layer_caches[run] = LayerCache(need, -1, state=state)
         for run, need in enumerate(needs):          # runs that read an earlier run's cache
             if isinstance(need, int) and not isinstance(need, bool):
@@ -96,6 +97,7 @@ class CacheManager:
                                                     state=source.state, writes=False)
         self._requests: dict[Hashable, RequestCache] = {}
         self._free_slots = list(range(self.max_requests - 1, -1, -1))
+        self.padding_state_slot = self.max_requests       # never handed to a request
 
     @staticmethod
     def page_bytes(needs: list, block_size: int, dtype: torch.dtype) -> int:

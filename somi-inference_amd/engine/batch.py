@@ -66,9 +66,21 @@ class StepBatch:
     block_size: int
 
 
-def _layout(entries: list[StepEntry], cache: CacheManager, table_widths: list[int] | None):
+class _Padding:
+    def __repr__(self) -> str:
+        return "<padding>"
+
+
+PADDING = _Padding()      # request id of a padding entry
+
+
+def _layout(entries: list[StepEntry], cache: CacheManager, table_widths: list[int] | None, pad_to: int = 0):
     """The step as host arrays: (sections, infos, widths).  ``table_widths`` fixes the block tables'
-    widths (a captured graph needs the same layout at every replay); None = as narrow as possible."""
+    widths (a captured graph needs the same layout at every replay); None = as narrow as possible.
+
+    ``pad_to``: entries are added until there are this many.  A padding entry is one token (id 0, position 0)
+    of no request: it stores nothing (slot -1), reads page 0 through a table row of zeros, uses the state
+    slot that no request gets, and its logits are computed and dropped by the caller."""
     infos: list[EntryInfo] = []
     token_ids: list[int] = []
     positions: list[int] = []
@@ -82,10 +94,17 @@ def _layout(entries: list[StepEntry], cache: CacheManager, table_widths: list[in
         token_ids.extend(entry.tokens)
         positions.extend(range(first, first + len(entry.tokens)))
         token_entry.extend([index] * len(entry.tokens))
-    n, e = len(token_ids), len(entries)
+    for index in range(len(entries), pad_to):
+        infos.append(EntryInfo(PADDING, len(token_ids), 1, 0, cache.padding_state_slot))
+        logit_rows.append(len(token_ids))
+        token_ids.append(0)
+        positions.append(0)
+        token_entry.append(index)
+    n, e = len(token_ids), len(infos)
+    nothing = np.zeros(0, dtype=np.int32)
     tables, slot_maps, widths = [], [], []
     for g in range(len(cache.groups)):
-        rows = [cache.table_row(g, info.request_id) for info in infos]
+        rows = [cache.table_row(g, info.request_id) if info.request_id is not PADDING else nothing for info in infos]
         width = max(1, max((r.size for r in rows), default=1))
         if table_widths is not None:
             if width > table_widths[g]:
@@ -96,7 +115,10 @@ def _layout(entries: list[StepEntry], cache: CacheManager, table_widths: list[in
             table[r, :pages.size] = pages                # released pages read as page 0 there
         slots: list[int] = []
         for info in infos:
-            slots.extend(cache.slots(g, info.request_id, info.first_position, info.length))
+            if info.request_id is PADDING:
+                slots.append(-1)
+            else:
+                slots.extend(cache.slots(g, info.request_id, info.first_position, info.length))
         tables.append(table)
         slot_maps.append(np.asarray(slots, dtype=np.int32))
         widths.append(width)
@@ -150,9 +172,10 @@ class StaticStep:
     whose device arrays stay in place, so that a captured HIP graph can be replayed on new contents."""
 
     def __init__(self, entries: list[StepEntry], cache: CacheManager, device: torch.device,
-                 table_widths: list[int]) -> None:
+                 table_widths: list[int], pad_to: int = 0) -> None:
         self.table_widths = list(table_widths)
-        sections, infos, widths = _layout(entries, cache, self.table_widths)
+        self.pad_to = int(pad_to)
+        sections, infos, widths = _layout(entries, cache, self.table_widths, self.pad_to)
         self.sizes = [s.size for s in sections]
         # Staging in pinned memory, several buffers in turn: the copy to the device is asynchronous, so the
         # host can lay out the next step while the device still runs this one.  A buffer is written again
@@ -180,7 +203,7 @@ class StaticStep:
         self.batch.entries = infos
 
     def update(self, entries: list[StepEntry], cache: CacheManager) -> StepBatch:
-        sections, infos, _ = _layout(entries, cache, self.table_widths)
+        sections, infos, _ = _layout(entries, cache, self.table_widths, self.pad_to)
         if [s.size for s in sections] != self.sizes:
             raise ValueError("the entries do not fit the shape this step was laid out for")
         self._fill(sections, infos)

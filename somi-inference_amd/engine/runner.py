@@ -33,6 +33,19 @@ class _DecodeGraph:
         self.static, self.graph, self.logits = static, graph, logits
 
 
+def graph_rows(entries: int) -> int:
+    """How many rows the captured step for this many single-token entries has: the next power of two up to
+    16, then the next multiple of 16 (the row tile of the matrix products, which cost the same for 17 as for 32
+    rows), so that a batch that shrinks request by request replays a handful of graphs instead of capturing
+    one per size.  The rows beyond the entries are padding."""
+    if entries <= 16:
+        rows = 1
+        while rows < entries:
+            rows *= 2
+        return rows
+    return (entries + 15) // 16 * 16
+
+
 class ModelRunner:
     accepts_device_tokens = True      # step() may take its tokens from a device tensor the host has not read
 
@@ -136,11 +149,49 @@ class ModelRunner:
         return rows
 
     # ------------------------------------------------------------- HIP graphs
+    def _capture(self, entries: list[StepEntry], rows: int, widths: list[int],
+                 device_tokens: torch.Tensor | None = None) -> _DecodeGraph:
+        """Capture the decode step of ``rows`` rows and these table widths, laid out for ``entries`` (none: all
+        rows are padding, which is how graphs are captured ahead of any request)."""
+        static = StaticStep(entries, self.cache, self.device, widths, pad_to=rows)
+        if device_tokens is not None:
+            static.batch.token_ids[:len(entries)].copy_(device_tokens)
+        # once outside a capture: lazy initialisation (library handles, first allocations) must
+        # not happen while the stream is being recorded; the step's writes are simply redone
+        self.model.forward(static.batch, self.cache.layer_caches)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            logits = self.model.forward(static.batch, self.cache.layer_caches)
+        held = self._graphs[(rows, tuple(widths))] = _DecodeGraph(static, graph, logits)
+        return held
+
+    def capture_decode_graphs(self, max_entries: int, max_context: int) -> int:
+        """Capture ahead of time the decode graphs that up to ``max_entries`` requests with contexts of up to
+        ``max_context`` tokens will replay (every row count of :func:`graph_rows`, every power-of-two table
+        width), so that serving does not stop to capture when a batch changes its size or outgrows its
+        tables.  Returns how many graphs were captured."""
+        if not self.decode_graphs or max_entries < 1:
+            return 0
+        pages = (max(1, max_context) + self.cache.block_size - 1) // self.cache.block_size
+        widths = [16]
+        while widths[-1] < pages:
+            widths.append(widths[-1] * 2)
+        captured = 0
+        for rows in sorted({graph_rows(n) for n in range(1, max_entries + 1)}):
+            for width in widths:
+                per_group = [width] * len(self.cache.groups)
+                if (rows, tuple(per_group)) not in self._graphs:
+                    self._capture([], rows, per_group)
+                    captured += 1
+        return captured
+
     def _decode_with_graph(self, entries: list[StepEntry], device_tokens: torch.Tensor | None = None) -> torch.Tensor:
         """Replay (or first capture) the graph for this many single-token entries.
 
         The block tables of a captured step have a fixed width, the next power of two of pages that
-        holds the longest request, so a graph serves until a request outgrows it.  The returned logits
+        holds the longest request, so a graph serves until a request outgrows it; its rows are
+        ``graph_rows(entries)``, the ones beyond the entries being padding.  The returned logits
         are the graph's own output tensor: they are overwritten by the next replay of the same graph.
         """
         widths = []
@@ -150,24 +201,15 @@ class ModelRunner:
             while width < longest:
                 width *= 2
             widths.append(width)
-        key = (len(entries), tuple(widths))
+        real, rows = len(entries), graph_rows(len(entries))
+        key = (rows, tuple(widths))
         held = self._graphs.get(key)
         if held is None:
-            static = StaticStep(entries, self.cache, self.device, widths)
-            if device_tokens is not None:
-                static.batch.token_ids.copy_(device_tokens)
-            # once outside a capture: lazy initialisation (library handles, first allocations) must
-            # not happen while the stream is being recorded; the step's writes are simply redone
-            self.model.forward(static.batch, self.cache.layer_caches)
-            torch.cuda.synchronize()
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph):
-                logits = self.model.forward(static.batch, self.cache.layer_caches)
-            held = self._graphs[key] = _DecodeGraph(static, graph, logits)
+            held = self._capture(entries, rows, widths, device_tokens)
         else:
             held.static.update(entries, self.cache)
             if device_tokens is not None:
-                held.static.batch.token_ids.copy_(device_tokens)      # on the stream, after the arrays' own copy
+                held.static.batch.token_ids[:real].copy_(device_tokens)   # on the stream, after the arrays' own copy
         held.graph.replay()
         self.graph_replays += 1
-        return held.logits
+        return held.logits[:real]

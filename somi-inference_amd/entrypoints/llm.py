@@ -87,12 +87,17 @@ class LLM:
         self._next_seq_id = 0
 
     # ----------------------------------------------------------------- warm-up
-    def warm_up(self) -> int:
-        """Optional: lets the library time its solutions for the matrix products of a full prompt portion.
+    def warm_up(self, max_context: int | None = None) -> int:
+        """Optional work before requests are served; not in the reference.
 
-        Not in the reference.  Worth a few seconds before long prompts are served in bfloat16 (the
-        float32 engine has no library products); returns the portion length that was tuned.
+        In bfloat16 the library times its solutions for the matrix products of a full prompt portion (the
+        float32 engine has no library products), and the decode steps of up to ``max_concurrent`` requests
+        with contexts of up to ``max_context`` tokens (default: 4,096, or what the pool holds if that is less)
+        are captured as graphs, so that serving never stops to capture one.  Returns the portion length that
+        was tuned.
         """
+        pool_tokens = self.options.num_blocks * self.options.block_size
+        self.runner.capture_decode_graphs(self.options.max_concurrent, min(max_context or 4096, pool_tokens))
         if self.dtype != "bfloat16":
             return 0
         return self.runner.tune_library_products(min(self.options.chunk, self.options.max_num_batched_tokens))

@@ -116,7 +116,8 @@ def test_state_slots_and_cache_sharing_runs():
     m = CacheManager(needs, block_size=4, num_blocks=4, max_requests=2, dtype=torch.float32, device="cpu")
     assert m.layer_caches[3] is None
     assert m.layer_caches[2].k is m.layer_caches[1].k and m.layer_caches[2].writes is False
-    assert m.layer_caches[0].state.shape == (2, 3)
+    assert m.layer_caches[0].state.shape == (2 + 1, 3)         # a row per request and the one padding entries use
+    assert m.padding_state_slot == 2
     m.register("a")
     m.layer_caches[0].state[m.state_slot("a")] = 5.0
     m.register("b")

@@ -177,12 +177,16 @@ def test_warm_up_tunes_library_products_without_changing_results(model_folders, 
               eos_token_id=-1)
     free_before = llm.kv_manager.free_pages()
     assert llm.warm_up() == 96
+    # and the decode graphs of up to 4 requests (1, 2 and 4 rows) with tables of 16, 32 and 64 pages (the pool's 512
+    # tokens) are captured before any request came
+    assert sorted(llm.runner._graphs) == [(rows, (width,)) for rows in (1, 2, 4) for width in (16, 32, 64)]
     assert llm.kv_manager.free_pages() == free_before
     llm.kv_manager.check_invariants()
     prompts = [token_ids(TINY["B"]["config"].vocab_size, 96, 3)]
     want, cfg, weights = plain_greedy(folder, prompts, 6)
     got = llm.generate(prompts, max_new_tokens=6, temperature=0.0)
     assert_greedy_matches(got, want, prompts, cfg, weights, exact=False)
+    assert len(llm.runner._graphs) == 9 and llm.runner.graph_replays > 0, "generation captured a graph of its own"
     assert list(tmp_path.iterdir()) == []
     assert LLM(folder, dtype="float32", num_blocks=64, block_size=8).warm_up() == 0
 

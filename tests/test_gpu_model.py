@@ -188,7 +188,8 @@ def test_step_contract_errors(model_folders):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_captured_decode_steps_replay_like_eager_steps(dtype, model_folders):
-    """Decode steps are captured as HIP graphs per batch size.  Batches of 3, 40 and 70 requests (the largest
+    """Decode steps are captured as HIP graphs per number of rows (4, 48 and 80 here, the entries padded up to
+    them).  Batches of 3, 40 and 70 requests (the largest
     takes the library matrix product inside the graph, the others the kernels that fuse norm, rotation and
     residual add into the products) are replayed several times, with eager work and synchronisations in
     between, and every replay is compared with the same step run without graphs."""
@@ -211,6 +212,14 @@ def test_captured_decode_steps_replay_like_eager_steps(dtype, model_folders):
                 runner.step([StepEntry(rid, prompt, [])])
         last = [p[-1] for p in prompts]
         for step in range(12):
+            if batch == 40 and step == 6:
+                # five requests end: 35 entries replay the graph of 48 rows that served 40 (rows beyond the entries
+                # are padding), no new capture
+                captured = len(graphed._graphs)
+                for runner in (graphed, eager):
+                    for rid in ids[35:]:
+                        runner.end(rid)
+                ids, last = ids[:35], last[:35]
             entries = [StepEntry(rid, [tok], [0]) for rid, tok in zip(ids, last)]
             want = eager.step(entries).clone()
             got = graphed.step(entries).clone()
@@ -223,6 +232,8 @@ def test_captured_decode_steps_replay_like_eager_steps(dtype, model_folders):
                 assert (got - want).abs().max() < 2e-2, f"batch {batch}, replay {step}"
             last = want.argmax(dim=-1).tolist()
             _ = torch.randn(64, 64, device="cuda:0") @ torch.randn(64, 64, device="cuda:0")   # eager work in between
+        if batch == 40:
+            assert len(graphed._graphs) == captured, "a batch that shrank within its row bucket was captured again"
         for runner in (graphed, eager):
             for rid in ids:
                 runner.end(rid)

@@ -96,7 +96,7 @@ def test_toy_mixer_is_registered_built_and_stepped(toy_registered, dtype):
     needs = model.cache_needs()
     assert isinstance(needs[0], FixedStateSpec) and isinstance(needs[2], FixedStateSpec)
     runner = make_runner(model, block_size=4, num_blocks=32, max_requests=3)
-    assert runner.cache.layer_caches[0].state.shape == (3, 24)
+    assert runner.cache.layer_caches[0].state.shape == (3 + 1, 24)      # three requests and the padding slot
     gen = torch.Generator().manual_seed(0)
     a = torch.randint(0, 50, (23,), generator=gen).tolist()
     b = torch.randint(0, 50, (9,), generator=gen).tolist()
