@@ -28,11 +28,13 @@ HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E bandwidth
 PEAK_FLOPS = {"bfloat16": 2.5e15, "float32": 157.3e12}   # dense MFMA peaks
 
 
-# layer sizes of the Qwen2.5 family: (layers, hidden, heads, kv heads, head_dim, intermediate, rms_norm_eps)
+# layer sizes of the Qwen2.5 family: (layers, hidden, heads, kv heads, head_dim, intermediate, rms_norm_eps,
+# vocabulary, tied LM head).  0.5b is the model the reference's own published figures are measured on.
 LAYER_SIZES = {
-    "7b": (28, 3584, 28, 4, 128, 18944, 1e-6),
-    "14b": (48, 5120, 40, 8, 128, 13824, 1e-5),
-    "32b": (64, 5120, 40, 8, 128, 27648, 1e-6),
+    "0.5b": (24, 896, 14, 2, 64, 4864, 1e-6, 151936, True),
+    "7b": (28, 3584, 28, 4, 128, 18944, 1e-6, 152064, False),
+    "14b": (48, 5120, 40, 8, 128, 13824, 1e-5, 152064, False),
+    "32b": (64, 5120, 40, 8, 128, 27648, 1e-6, 152064, False),
 }
 
 
@@ -44,7 +46,8 @@ def parse_args() -> argparse.Namespace:
     p.add_argument("--batch", type=int, default=8)
     p.add_argument("--context", type=int, default=4096, help="context length the timed decode steps end at")
     p.add_argument("--sizes", default="7b", choices=sorted(LAYER_SIZES),
-                   help="layer sizes: Qwen2.5-7B (the default and the headline), -14B or -32B")
+                   help="layer sizes: Qwen2.5-7B (the default and the headline), -14B, -32B, or -0.5B (the model of the "
+                        "reference's own published figures)")
     p.add_argument("--layers", type=int, default=None, help="run fewer layers than the configuration has")
     p.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     p.add_argument("--block-size", type=int, default=16)
@@ -75,11 +78,11 @@ def main() -> int:
     from somi_inference_amd.models import make_runner, random_model
     from somi_inference_amd.sampling import Sampler, SamplingParams
 
-    full_layers, hidden, heads, kv_heads, head_dim, intermediate, eps = LAYER_SIZES[args.sizes]
+    full_layers, hidden, heads, kv_heads, head_dim, intermediate, eps, vocab, tied = LAYER_SIZES[args.sizes]
     layers = args.layers or full_layers
-    config = Qwen2Config(vocab_size=152064, hidden_size=hidden, intermediate_size=intermediate,
+    config = Qwen2Config(vocab_size=vocab, hidden_size=hidden, intermediate_size=intermediate,
                          num_hidden_layers=layers, num_attention_heads=heads, num_key_value_heads=kv_heads,
-                         head_dim=head_dim, rope_theta=1e6, rms_norm_eps=eps, tie_word_embeddings=False,
+                         head_dim=head_dim, rope_theta=1e6, rms_norm_eps=eps, tie_word_embeddings=tied,
                          max_position_embeddings=32768)
     torch.manual_seed(args.seed)
     model = random_model(config, seed=args.seed, dtype=args.dtype)
@@ -212,7 +215,7 @@ def main() -> int:
                    "layers_of_config": full_layers, "hidden_size": config.hidden_size,
                    "intermediate_size": config.intermediate_size, "num_attention_heads": config.num_attention_heads,
                    "num_key_value_heads": config.num_key_value_heads, "head_dim": config.head_dim,
-                   "vocab_size": config.vocab_size, "tie_word_embeddings": False, "block_size": args.block_size,
+                   "vocab_size": config.vocab_size, "tie_word_embeddings": tied, "block_size": args.block_size,
                    "context_at_end": args.context, "library_gemm_tuned": tuned > 0},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4)},
