@@ -534,7 +534,7 @@ def test_products_fused_with_the_residual_add_and_the_norm(m, hidden, n_out, int
 
 @pytest.mark.parametrize("scaled", [True, False], ids=["normed", "as-is"])
 @pytest.mark.parametrize("m, nq, nkv, d, hidden, page", [(1, 4, 2, 32, 64, 16), (9, 12, 2, 64, 200, 8), (16, 3, 3, 128, 520, 4),
-                                                         (37, 5, 1, 96, 1000, 16), (64, 28, 4, 128, 3584, 16)])
+                                                         (24, 6, 2, 96, 264, 8), (37, 5, 1, 96, 1000, 16), (64, 28, 4, 128, 3584, 16)])
 def test_qkv_product_with_the_rotation_and_the_cache_store(m, nq, nkv, d, hidden, page, scaled):
     """q/k/v projection, rotary encoding and cache write in one kernel: against the float32 formulas (norm as a
     row scale, product, rotation) and against the three separate kernels."""
