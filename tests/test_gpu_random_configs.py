@@ -17,17 +17,20 @@ from somi_inference_amd.weights import write_random_model
 pytestmark = pytest.mark.gpu
 
 
-def random_case(seed: int):
-    rng = random.Random(seed)
+def random_case(seed: int, odd: bool = False):
+    """``odd``: widths that are no multiple of 8 and head sizes that are no multiple of 16 or beyond 128, which
+    take the plain kernels in places."""
+    rng = random.Random(seed + (1000 if odd else 0))
     nkv = rng.choice([1, 2, 3, 4, 5])
     nq = nkv * rng.choice([1, 2, 3, 4, 7, 8])
     layers = rng.choice([1, 2, 3])
     window = rng.random() < 0.4
     config = Qwen2Config(
-        vocab_size=rng.choice([97, 256, 301, 503, 1000]), hidden_size=rng.choice([40, 64, 72, 120, 136, 200]),
-        intermediate_size=rng.choice([48, 96, 160, 200, 272, 520]), num_hidden_layers=layers,
-        num_attention_heads=nq, num_key_value_heads=nkv,
-        head_dim=rng.choice([16, 32, 48, 64, 80, 96, 112, 128, 24, 40]),
+        vocab_size=rng.choice([97, 256, 301, 503, 1000]),
+        hidden_size=rng.choice([36, 50, 66, 100, 44, 68] if odd else [40, 64, 72, 120, 136, 200]),
+        intermediate_size=rng.choice([50, 70, 100, 36, 132] if odd else [48, 96, 160, 200, 272, 520]),
+        num_hidden_layers=layers, num_attention_heads=nq, num_key_value_heads=nkv,
+        head_dim=rng.choice([6, 10, 18, 24, 40, 144, 160, 256] if odd else [16, 32, 48, 64, 80, 96, 112, 128, 24, 40]),
         rope_theta=rng.choice([1e4, 5e4, 1e6]), rms_norm_eps=rng.choice([1e-6, 1e-5, 3e-6]),
         tie_word_embeddings=rng.random() < 0.5, attention_bias=rng.random() < 0.8,
         use_sliding_window=window, sliding_window=rng.choice([5, 20, 33, 64]) if window else None,
@@ -36,9 +39,10 @@ def random_case(seed: int):
     return rng, config, block_size
 
 
+@pytest.mark.parametrize("odd", [False, True], ids=["even", "odd"])
 @pytest.mark.parametrize("seed", range(16))
-def test_random_configuration_under_a_random_mixed_trace(seed, tmp_path):
-    rng, config, block_size = random_case(seed)
+def test_random_configuration_under_a_random_mixed_trace(seed, odd, tmp_path):
+    rng, config, block_size = random_case(seed, odd)
     base = write_random_model(str(tmp_path / "model"), config, seed=rng.randrange(1000))
     folder = peaky_folder(base, str(tmp_path / "peaky"), factor=rng.choice([1.0, 3.0, 4.0]))
     plain_config, weights = plain.read_model(folder)
