@@ -14,15 +14,24 @@ from __future__ import annotations
 
 import contextlib
 import os
+import stat
 import tempfile
 
 import torch
 
 
 def _results_file() -> str:
+    """A file in a folder of the user's own under the temporary folder (a folder of that name that someone else
+    made, or that others may write, is not used: a fresh one is made instead)."""
     uid = os.getuid() if hasattr(os, "getuid") else 0
     folder = os.path.join(tempfile.gettempdir(), f"somi_inference_amd_tuning_{uid}")
-    os.makedirs(folder, exist_ok=True)
+    try:
+        os.makedirs(folder, mode=0o700, exist_ok=True)
+        info = os.lstat(folder)
+        if not stat.S_ISDIR(info.st_mode) or (hasattr(os, "getuid") and info.st_uid != uid) or info.st_mode & 0o022:
+            raise OSError("not a private folder")
+    except OSError:
+        folder = tempfile.mkdtemp(prefix="somi_inference_amd_tuning_")
     return os.path.join(folder, "library_products.csv")
 
 
