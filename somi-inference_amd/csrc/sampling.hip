@@ -6,6 +6,9 @@
 // number that the host derives from the request's own seed and token count, so a request's tokens do not
 // depend on what else is in the batch.
 #include "common.h"
+#include "no_alloc.h"
+
+#include <mutex>
 
 // The vocabulary is cut into chunks of SAMPLE_CHUNK entries; one workgroup per (row, chunk) finds the
 // chunk's maximum, its first index and (for a draw) the chunk's softmax mass relative to that maximum.  A
@@ -161,6 +164,53 @@ extern "C" int somi_sample(const float* logits, int rows, int vocab, const float
                        uniform, workspace, out);
     SOMI_LAUNCH_CHECK("sample_pick");
     return 0;
+}
+
+// The workspace of somi_sample_no_alloc: one array per GPU, held until the process ends.  In host code the
+// array's name is only a handle for hipGetSymbolAddress; the address it yields differs from GPU to GPU and is
+// what the kernels get.
+static __device__ __align__(256) float scratch[SOMI_SAMPLE_SCRATCH_FLOATS];
+
+#define SOMI_MAX_DEVICES 64
+static float* g_scratch_ptr[SOMI_MAX_DEVICES];      // the array's address on each device, once asked for
+static std::mutex g_scratch_mutex;
+
+// The address of `scratch` on the current device (asked for once per device, with that device current).
+static int scratch_on_current_device(float** ptr) {
+    int device = -1;
+    hipError_t err = hipGetDevice(&device);
+    SOMI_REQUIRE(err == hipSuccess, "sample_no_alloc: hipGetDevice: %s", hipGetErrorString(err));
+    SOMI_REQUIRE(device >= 0 && device < SOMI_MAX_DEVICES, "sample_no_alloc: device %d is beyond the %d this library "
+                 "keeps a workspace for", device, SOMI_MAX_DEVICES);
+    std::lock_guard<std::mutex> hold(g_scratch_mutex);
+    if (g_scratch_ptr[device] == nullptr) {
+        float* found = nullptr;
+        err = hipGetSymbolAddress((void**)&found, HIP_SYMBOL(scratch));
+        SOMI_REQUIRE(err == hipSuccess && found != nullptr, "sample_no_alloc: hipGetSymbolAddress on device %d: %s",
+                     device, hipGetErrorString(err));
+        g_scratch_ptr[device] = found;
+    }
+    *ptr = g_scratch_ptr[device];
+    return 0;
+}
+
+extern "C" int somi_sample_no_alloc_capacity() { return SOMI_SAMPLE_SCRATCH_FLOATS; }
+
+extern "C" int somi_sample_no_alloc(const float* logits, int rows, int vocab, const float* temperature,
+                                    const float* uniform, int* out, hipStream_t stream) {
+    SOMI_REQUIRE(rows >= 0 && vocab > 0, "sample_no_alloc: bad sizes rows=%d vocab=%d", rows, vocab);
+    SOMI_REQUIRE(rows <= 65535, "sample_no_alloc: too many rows");
+    if (rows == 0) return 0;
+    SOMI_REQUIRE(logits && temperature && uniform && out, "sample_no_alloc: a null pointer among the arguments");
+    const int64_t need = (int64_t)rows * ceil_div(vocab, SAMPLE_CHUNK) * 3;
+    SOMI_REQUIRE(need <= SOMI_SAMPLE_SCRATCH_FLOATS,
+                 "sample_no_alloc: %d rows of %d logits need %lld floats of workspace, the fixed one holds %d "
+                 "(rows * ceil(vocab / %d) * 3 must not exceed it); use somi_sample with a workspace of your own",
+                 rows, vocab, (long long)need, SOMI_SAMPLE_SCRATCH_FLOATS, SAMPLE_CHUNK);
+    float* workspace = nullptr;
+    if (scratch_on_current_device(&workspace) != 0) return 1;
+    // every (row, chunk) triple that the second kernel reads is written by the first: nothing to clear
+    return somi_sample(logits, rows, vocab, temperature, uniform, out, workspace, stream);
 }
 
 // logits[row, id] = logit > 0 ? logit / penalty : logit * penalty for each listed id (ids must be distinct).
