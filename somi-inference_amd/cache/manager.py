@@ -183,6 +183,17 @@ class CacheManager:
                 pages.append(group.pool.allocate())
                 record.note_page(g, len(pages) - 1, pages[-1])
 
+    def rollback(self, request_id: Hashable) -> None:
+        """Give back the pages that were reserved beyond the committed tokens (a step that failed after
+        ``reserve`` and before ``commit``); what the committed tokens hold stays."""
+        record = self._get(request_id)
+        keep = self._pages_for(record.num_tokens)
+        for group, pages in zip(self.groups, record.pages):
+            while len(pages) > keep:
+                page = pages.pop()
+                if page != RELEASED:
+                    group.pool.release(page)
+
     def commit(self, request_id: Hashable, new_tokens: int) -> None:
         """Count the tokens a step wrote, and give back pages a window has passed."""
         record = self._get(request_id)

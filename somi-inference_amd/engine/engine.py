@@ -136,16 +136,33 @@ class Engine:
     def run(self, requests: deque[tuple[int, Request]] | None = None) -> list[Request]:
         """Run until every request has finished; ``requests`` holds (arrival_step, request) in
         arrival order, as the reference's ``run`` takes them (continuous_batching.py:179-205).
-        Returns the requests in the order they finished."""
+        Returns the requests in the order they finished.  A request that can never run (too long for the pool
+        or the model, a token id outside the vocabulary) raises before anything is queued; if a step raises,
+        the call's requests are aborted and what they held is free again, so the next call starts clean."""
         requests = requests if requests is not None else deque()
+        mine = [request for _, request in requests]
+        for request in mine:
+            self.scheduler.check_request(request)      # all of them before any is queued: a refusal leaves nothing behind
         finished: list[Request] = []
         self.scheduler.drain_finished()
         step = 0
-        while requests or self.scheduler.has_unfinished():
-            while requests and requests[0][0] <= step:
-                self.add_request(requests.popleft()[1])
-            finished.extend(self.step())
-            step += 1
-        self._read_unread()
+        try:
+            while requests or self.scheduler.has_unfinished():
+                while requests and requests[0][0] <= step:
+                    self.add_request(requests.popleft()[1])
+                finished.extend(self.step())
+                step += 1
+            self._read_unread()
+        except BaseException:
+            self.abort(mine)
+            raise
         finished.extend(self.scheduler.drain_finished())
         return finished
+
+    def abort(self, requests: list[Request]) -> None:
+        """Take these requests out of the queues and give back their pages and state slots, whatever state a
+        failed step left them in; tokens that were drawn but not read are dropped."""
+        self._unread = None
+        for request in requests:
+            self.scheduler.abort(request)
+        self.scheduler.drain_finished()

@@ -101,7 +101,8 @@ class ModelRunner:
         """Run the entries as one batch; float32 logits ``[sum(len(want)), vocab]`` in entry order.
 
         Raises :class:`OutOfPages` before anything changes if the pages for
-        all entries are not free.
+        all entries are not free.  If the forward pass raises, the pages the step
+        reserved are given back and the requests' token counts stay as they were.
 
         ``device_tokens``: the entries' (single) tokens as an int32 tensor that is still on the device,
         typically what the sampler drew from the previous step's logits and the host has not read yet;
@@ -114,13 +115,19 @@ class ModelRunner:
             raise OutOfPages(f"the step needs more pages than are free ({self.cache.free_pages()} free)")
         for request_id, count in portions:
             self.cache.reserve(request_id, count)
-        if self.decode_graphs and all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries):
-            logits = self._decode_with_graph(entries, device_tokens)
-        else:
-            batch = build_step(entries, self.cache, self.device)
-            if device_tokens is not None:
-                batch.token_ids.copy_(device_tokens)
-            logits = self.model.forward(batch, self.cache.layer_caches)
+        try:
+            if self.decode_graphs and all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries):
+                logits = self._decode_with_graph(entries, device_tokens)
+            else:
+                batch = build_step(entries, self.cache, self.device)
+                if device_tokens is not None:
+                    batch.token_ids.copy_(device_tokens)
+                logits = self.model.forward(batch, self.cache.layer_caches)
+        except BaseException:
+            # nothing of the step counts: the pages it took go back, the requests stand where they stood
+            for request_id, _ in portions:
+                self.cache.rollback(request_id)
+            raise
         for request_id, count in portions:
             self.cache.commit(request_id, count)
         self.steps_run += 1

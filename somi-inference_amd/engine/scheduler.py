@@ -57,27 +57,73 @@ class SchedulerOutput:
 
 class Scheduler:
     def __init__(self, cache: CacheManager, *, max_concurrent: int, max_num_batched_tokens: int,
-                 chunk: int | None = None) -> None:
+                 chunk: int | None = None, vocab_size: int | None = None, max_positions: int | None = None,
+                 granule: int = 1) -> None:
+        """``vocab_size``: token ids must lie below it (None: not checked here).  ``max_positions``: the longest
+        sequence the model's position encoding covers (None: unbounded).  ``granule``: a prompt portion that
+        does not end its prompt holds a multiple of this many tokens (a mixer that works on blocks of tokens
+        says so through ``portion_granule``)."""
         if max_concurrent < 1 or max_num_batched_tokens < 1:
             raise SchedulerError("max_concurrent and max_num_batched_tokens must be >= 1")
+        if granule < 1 or granule > max_num_batched_tokens:
+            raise SchedulerError(f"the portion granule {granule} must lie in [1, max_num_batched_tokens = "
+                                 f"{max_num_batched_tokens}]")
         self.cache = cache
         self.max_concurrent = int(max_concurrent)
         self.max_num_batched_tokens = int(max_num_batched_tokens)
+        self.granule = int(granule)
         self.chunk = int(min(chunk or max_num_batched_tokens, max_num_batched_tokens))
+        if self.chunk < self.granule:
+            raise SchedulerError(f"portions of at most {self.chunk} tokens cannot hold the granule of {self.granule}")
+        self.chunk -= self.chunk % self.granule
+        self.vocab_size = int(vocab_size) if vocab_size is not None else None
+        self.max_positions = int(max_positions) if max_positions is not None else None
         self.waiting: deque[Request] = deque()
         self.running: list[Request] = []          # in admission order
         self.finished: list[Request] = []
 
     # -------------------------------------------------------------- requests
-    def add_request(self, request: Request) -> None:
+    def check_request(self, request: Request) -> None:
+        """Raises :class:`SchedulerError` if the request can never run; changes nothing."""
         pages = (request.max_cached_tokens + self.cache.block_size - 1) // self.cache.block_size
         if pages > self.cache.num_blocks:
             raise SchedulerError(
                 f"request {request.request_id!r} needs {pages} pages for {request.max_cached_tokens} tokens "
                 f"(prompt {len(request.prompt_tokens)} + max_new_tokens {request.max_new_tokens} - 1), "
                 f"the cache has {self.cache.num_blocks}")
+        if self.max_positions is not None and request.max_cached_tokens > self.max_positions:
+            # the reference's rotary table ends at max_position_embeddings and a lookup beyond it fails
+            # (somi_inference/models/qwen2.py:72-81, 89-90)
+            raise SchedulerError(
+                f"request {request.request_id!r} reaches position {request.max_cached_tokens - 1} "
+                f"(prompt {len(request.prompt_tokens)} + max_new_tokens {request.max_new_tokens} - 1 tokens), beyond "
+                f"the model's max_position_embeddings = {self.max_positions}")
+        if self.vocab_size is not None:
+            for token in request.prompt_tokens:
+                if not 0 <= int(token) < self.vocab_size:
+                    raise SchedulerError(f"request {request.request_id!r}: token id {token} is outside "
+                                         f"[0, {self.vocab_size})")
+
+    def add_request(self, request: Request) -> None:
+        self.check_request(request)
         request.status = RequestStatus.WAITING
         self.waiting.append(request)
+
+    def abort(self, request: Request) -> None:
+        """Take a request out wherever it stands and give back what it holds (no-op for one that is finished
+        or unknown)."""
+        if request in self.running:
+            self.running.remove(request)
+        else:
+            try:
+                self.waiting.remove(request)
+            except ValueError:
+                pass
+        if self.cache.has(request.request_id):
+            self.cache.free(request.request_id)
+        if request.status is not RequestStatus.FINISHED:
+            request.status = RequestStatus.FINISHED
+            request.finish_reason = "aborted"
 
     def has_unfinished(self) -> bool:
         return bool(self.waiting) or bool(self.running)
@@ -106,10 +152,16 @@ class Scheduler:
         output.portions = [p for p in output.portions if p.request is not victim]
         return victim
 
+    def _whole(self, request: Request, count: int) -> int:
+        """``count`` cut down to a multiple of the granule, unless it ends what the request has pending."""
+        if self.granule == 1 or count >= request.num_pending:
+            return count
+        return count - count % self.granule
+
     def _fit(self, request: Request, want: int, taken: list[int]) -> int:
         """Largest portion <= want whose pages are free after what this step already took."""
         free = [f - t for f, t in zip(self.cache.free_pages(), taken)]
-        count = want
+        count = self._whole(request, want)
         while count > 0:
             need = self.cache.pages_needed(request.request_id, count)
             if all(n <= f for n, f in zip(need, free)):
@@ -118,7 +170,7 @@ class Scheduler:
             cached = self.cache.num_tokens(request.request_id)
             pages_ok = min(len(self.cache.page_list(g, request.request_id)) + free[g]
                            for g in range(len(free)))
-            count = min(count - 1, pages_ok * self.cache.block_size - cached)
+            count = self._whole(request, min(count - 1, pages_ok * self.cache.block_size - cached))
         return 0
 
     def schedule(self) -> SchedulerOutput:
@@ -142,7 +194,9 @@ class Scheduler:
         for request in order:
             if request not in self.running or budget <= 0:
                 continue
-            want = min(request.num_pending, self.chunk, budget)
+            want = self._whole(request, min(request.num_pending, self.chunk, budget))
+            if want == 0:
+                continue                     # what is left of the budget does not hold a granule: next step
             while True:
                 count = self._fit(request, want, taken)
                 if count > 0:
@@ -165,8 +219,10 @@ class Scheduler:
         # 2. admissions, first come first served; the head of the queue blocks the rest
         while self.waiting and len(self.running) < self.max_concurrent and budget > 0 and not output.preempted:
             request = self.waiting[0]
+            want = self._whole(request, min(request.num_pending, self.chunk, budget))
+            if want == 0:
+                break
             self.cache.register(request.request_id)
-            want = min(request.num_pending, self.chunk, budget)
             count = self._fit(request, want, taken)
             if count < want:
                 self.cache.free(request.request_id)     # the pages of its first portion are not free: wait

@@ -80,7 +80,9 @@ class LLM:
         self.kv_manager = self.runner.cache
         self.sampler = Sampler()
         self.scheduler = Scheduler(self.runner.cache, max_concurrent=max_concurrent,
-                                   max_num_batched_tokens=max_num_batched_tokens, chunk=self.options.chunk)
+                                   max_num_batched_tokens=max_num_batched_tokens, chunk=self.options.chunk,
+                                   vocab_size=self.model.vocab_size, max_positions=self.model.plan.max_positions,
+                                   granule=self.model.portion_granule())
         if eos_token_id is None:
             eos_token_id = self.tokenizer.eos_token_id if self.tokenizer else getattr(self.config, "eos_token_id", None)
         self.engine = Engine(self.runner, self.scheduler, self.sampler, eos_token_id)
@@ -139,7 +141,8 @@ class LLM:
             requests.append(Request(self._next_seq_id, tokens, max_new_tokens, params, seed=request_seed))
             self._next_seq_id += 1
         finished = self.engine.run(deque((0, r) for r in requests))
-        assert len(finished) == len(requests), "generate expects every request to finish"
+        if len(finished) != len(requests):
+            raise RuntimeError(f"{len(requests)} requests were run and {len(finished)} finished")
         results = []
         for request, is_text in zip(requests, as_text):
             results.append(self.tokenizer.decode(request.output_tokens) if is_text else list(request.output_tokens))

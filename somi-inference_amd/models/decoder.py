@@ -76,6 +76,11 @@ class DecoderModel:
             parts.extend(layer.parts())
         return all(getattr(part, "graph_safe", False) for part in parts)
 
+    def portion_granule(self) -> int:
+        """The least common multiple of what the mixers ask of the scheduler's prompt portions."""
+        import math
+        return math.lcm(*[int(getattr(layer.mixer, "portion_granule", 1)) for layer in self.layers] or [1])
+
     # -------------------------------------------------------------------- cache
     def cache_needs(self) -> list[PagedKVSpec | FixedStateSpec | int | None]:
         """For each run of a layer: the cache its mixer needs, the index of the earlier

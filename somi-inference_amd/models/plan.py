@@ -37,6 +37,7 @@ class ModelPlan:
     vocab_size: int = 0
     embedding_position: PartSpec | None = None       # a position encoding applied to the embedded tokens
     embedding_position_prefix: str = ""
+    max_positions: int | None = None                 # longest sequence the position encoding covers; None = no bound
 
     def run_order(self) -> tuple[int, ...]:
         return self.order if self.order else tuple(range(len(self.layers)))

@@ -50,6 +50,8 @@ def qwen2_plan(config: Qwen2Config) -> ModelPlan:
         head_prefix="lm_head",
         ignore_weights=tuple(ignore),
         vocab_size=config.vocab_size,
+        # the reference's rotary table has max_position_embeddings rows (qwen2_adapter.py:222, qwen2.py:72-81)
+        max_positions=config.max_position_embeddings,
     )
 
 

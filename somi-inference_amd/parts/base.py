@@ -148,6 +148,7 @@ class Mixer(Part):
         return None
 
     takes_normed_rows = False      # True: x may arrive as parts.linear.NormedRows (rows still to be normed)
+    portion_granule = 1            # a prompt portion that does not end its prompt holds a multiple of this many tokens
 
     def forward(self, x: torch.Tensor, step: Any, cache: LayerCache | None) -> torch.Tensor:
         """x: [N, H] compute dtype -> [N, H] compute dtype, or a parts.linear.DeferredProduct of that shape

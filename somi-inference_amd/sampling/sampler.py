@@ -36,15 +36,19 @@ class Sampler:
 
     def __init__(self) -> None:
         self._greedy_inputs: dict[tuple[int, torch.device], torch.Tensor] = {}
-        self._host_rings: dict[tuple[str, int, torch.dtype], tuple[list[torch.Tensor], list[int]]] = {}
+        self._host_rings: dict[tuple[str, int, torch.dtype], tuple[list[torch.Tensor], list, list[int]]] = {}
 
-    def _host_buffer(self, purpose: str, size: int, dtype: torch.dtype) -> torch.Tensor:
+    def _host_buffer(self, purpose: str, size: int, dtype: torch.dtype) -> tuple[torch.Tensor, list, int]:
         """Pinned host memory, a few buffers per purpose and size in turn: copies to and from it do not wait for
-        the device."""
-        ring, turn = self._host_rings.setdefault(
-            (purpose, size, dtype), ([torch.empty(size, dtype=dtype).pin_memory() for _ in range(self.RING)], [0]))
+        the device.  Returns (buffer, events, turn): the caller records ``events[turn]`` after the copy it
+        starts on the buffer; a buffer is handed out again only once that copy has finished."""
+        ring, events, turn = self._host_rings.setdefault(
+            (purpose, size, dtype), ([torch.empty(size, dtype=dtype).pin_memory() for _ in range(self.RING)],
+                                     [None] * self.RING, [0]))
         turn[0] = (turn[0] + 1) % self.RING
-        return ring[turn[0]]
+        if events[turn[0]] is not None:
+            events[turn[0]].synchronize()
+        return ring[turn[0]], events, turn[0]
 
     def _staged(self, values: list, dtype: torch.dtype, device: torch.device) -> torch.Tensor:
         """``values`` on the device through pinned memory (buffers come in power-of-two sizes, so that a few serve
@@ -52,9 +56,12 @@ class Sampler:
         capacity = 64
         while capacity < len(values):
             capacity *= 2
-        staged = self._host_buffer("in", capacity, dtype)
+        staged, events, turn = self._host_buffer("in", capacity, dtype)
         staged[:len(values)].copy_(torch.tensor(values, dtype=dtype))
-        return staged.to(device, non_blocking=True)[:len(values)]
+        on_device = staged.to(device, non_blocking=True)
+        events[turn] = torch.cuda.Event()
+        events[turn].record()
+        return on_device[:len(values)]
 
     def _row_inputs(self, plist: list[SamplingParams], seeds: list[int], counters: list[int],
                     device: torch.device) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
@@ -125,8 +132,8 @@ class Sampler:
             if filters:
                 ops.sample_filter(work, temperature, ints[:rows], top_p)
         picked = ops.sample(work, temperature, draws)
-        host = self._host_buffer("out", rows, torch.int32)
+        host, events, turn = self._host_buffer("out", rows, torch.int32)
         host.copy_(picked, non_blocking=True)
-        copied = torch.cuda.Event()
+        copied = events[turn] = torch.cuda.Event()
         copied.record()
         return PendingTokens(picked, host, copied)

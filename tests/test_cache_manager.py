@@ -187,3 +187,24 @@ def test_step_arrays_for_a_mixed_batch():
     assert step.paged[0].slot_mapping.tolist() == m.slots(0, "p", 0, 6) + m.slots(0, "d", 5, 1)
     assert step.max_entry_len == 6 and step.max_context == 6
     assert all(t.dtype == torch.int32 for t in (step.token_ids, step.positions, table, step.logit_rows))
+
+
+def test_rollback_gives_back_what_a_failed_step_reserved_and_nothing_else():
+    cache = CacheManager([PagedKVSpec(1, 8), PagedKVSpec(1, 8, window=6)], block_size=4, num_blocks=8,
+                         max_requests=2, dtype=torch.float32, device="cpu", allocate_tensors=False)
+    cache.register("a")
+    cache.reserve("a", 10)
+    cache.commit("a", 10)                       # the window of 6 has passed page 0 of the second group
+    held = cache.free_pages()
+    cache.reserve("a", 7)                       # 17 tokens: two more pages in each group
+    assert cache.free_pages() == [held[0] - 2, held[1] - 2]
+    cache.rollback("a")
+    assert cache.free_pages() == held and cache.num_tokens("a") == 10
+    cache.check_invariants()
+    cache.rollback("a")                         # nothing reserved: nothing happens
+    assert cache.free_pages() == held
+    cache.reserve("a", 1)
+    cache.commit("a", 1)
+    cache.free("a")
+    assert cache.free_pages() == [8, 8]
+    cache.check_invariants()

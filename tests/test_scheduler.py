@@ -285,3 +285,75 @@ def test_running_ahead_is_left_alone_when_a_sampling_rule_reads_the_history():
     done = engine.run(deque([(0, request(0, 5, 4, sampling_params=SamplingParams(repetition_penalty=1.3)))]))
     assert done[0].output_tokens == [30, 31, 32, 33] and engine.steps_run_ahead == 0
     assert "launch ahead" not in runner.log
+
+
+def test_a_refused_request_leaves_nothing_behind_for_the_next_call():
+    """A list whose second request can never fit is refused before the first is queued, so the next call runs
+    its own requests only."""
+    cache = make_cache(num_blocks=4, block_size=4)
+    engine, scheduler, _, _ = make_engine(cache, {0: [1, 2], 1: [3], 2: [4, 5]})
+    with pytest.raises(SchedulerError, match="pages"):
+        engine.run(deque([(0, request(0, 3, 2)), (0, request(1, 30, 1))]))
+    assert not scheduler.waiting and not scheduler.running and cache.free_pages() == [4]
+    done = engine.run(deque([(0, request(2, 3, 2))]))
+    assert [(r.request_id, r.output_tokens) for r in done] == [(2, [4, 5])]
+
+
+def test_token_ids_and_positions_are_checked_before_anything_is_queued():
+    cache = make_cache(num_blocks=16)
+    scheduler = Scheduler(cache, max_concurrent=4, max_num_batched_tokens=64, vocab_size=50, max_positions=12)
+    engine = Engine(ScriptedRunner(cache), scheduler, ScriptedSampler({0: [1, 2], 1: [3, 4, 5]}), None)
+    good = Request(0, [1, 2, 3], 2, seed=0)
+    with pytest.raises(SchedulerError, match=r"token id 50 is outside \[0, 50\)"):
+        engine.run(deque([(0, good), (0, Request(1, [4, 50], 1, seed=1))]))
+    with pytest.raises(SchedulerError, match="max_position_embeddings = 12"):
+        engine.run(deque([(0, Request(1, list(range(10)), 4, seed=1))]))       # 13 cached tokens
+    assert not scheduler.waiting and not scheduler.running and not cache.live_requests()
+    done = engine.run(deque([(0, good), (0, Request(1, list(range(10)), 3, seed=1))]))   # 12 tokens: the last position
+    assert sorted(r.request_id for r in done) == [0, 1]
+
+
+class FailingRunner(ScriptedRunner):
+    """Raises in a chosen step after it has reserved pages, as a kernel that refuses its arguments would."""
+
+    def __init__(self, cache, fail_at):
+        super().__init__(cache)
+        self.fail_at = fail_at
+
+    def step(self, entries):
+        if len(self.calls) == self.fail_at:
+            self.fail_at = -1
+            for e in entries:
+                self.cache.reserve(e.request_id, len(e.tokens))
+            raise RuntimeError("the step failed")
+        return super().step(entries)
+
+
+def test_a_step_that_raises_aborts_the_calls_requests_and_the_next_call_runs():
+    cache = make_cache(num_blocks=8, block_size=4)
+    scheduler = Scheduler(cache, max_concurrent=4, max_num_batched_tokens=64)
+    runner = FailingRunner(cache, fail_at=2)
+    engine = Engine(runner, scheduler, ScriptedSampler({0: [1] * 6, 1: [2] * 6, 2: [7, 8]}), None)
+    first, second = request(0, 5, 6), request(1, 6, 6)
+    with pytest.raises(RuntimeError, match="the step failed"):
+        engine.run(deque([(0, first), (0, second)]))
+    assert first.finish_reason == second.finish_reason == "aborted"
+    assert not scheduler.waiting and not scheduler.running and not cache.live_requests()
+    assert cache.free_pages() == [8]
+    cache.check_invariants()
+    done = engine.run(deque([(0, request(2, 3, 2))]))
+    assert [(r.request_id, r.output_tokens) for r in done] == [(2, [7, 8])]
+
+
+def test_portions_come_in_multiples_of_the_granule_except_the_one_that_ends_the_prompt():
+    cache = make_cache(num_blocks=32)
+    scheduler = Scheduler(cache, max_concurrent=4, max_num_batched_tokens=11, chunk=10, granule=4)
+    runner = ScriptedRunner(cache)
+    engine = Engine(runner, scheduler, ScriptedSampler({0: [1, 2, 3], 1: [5, 6]}), None)
+    done = engine.run(deque([(0, request(0, 3, 3)), (1, request(1, 18, 2))]))
+    assert {r.request_id: r.output_tokens for r in done} == {0: [1, 2, 3], 1: [5, 6]}
+    portions = [n for call in runner.calls for rid, tokens, _ in call if rid == 1 for n in [len(tokens)]]
+    # chunk 10 becomes 8; beside a decoding request 10 tokens of budget are left: 8 again; the rest ends the prompt
+    assert portions[:3] == [8, 8, 2] and all(n == 1 for n in portions[3:])
+    with pytest.raises(SchedulerError, match="granule"):
+        Scheduler(cache, max_concurrent=1, max_num_batched_tokens=8, chunk=3, granule=4)
