@@ -81,6 +81,7 @@ class Scheduler:
         self.waiting: deque[Request] = deque()
         self.running: list[Request] = []          # in admission order
         self.finished: list[Request] = []
+        self.preemptions = 0                      # how often a running request had to give its pages back
 
     # -------------------------------------------------------------- requests
     def check_request(self, request: Request) -> None:
@@ -147,6 +148,7 @@ class Scheduler:
         victim.status = RequestStatus.WAITING
         victim.num_computed = 0
         victim.num_preemptions += 1
+        self.preemptions += 1
         self.waiting.appendleft(victim)
         output.preempted.append(victim)
         output.portions = [p for p in output.portions if p.request is not victim]

@@ -69,15 +69,119 @@ def test_prompts_in_portions_of_seven_beside_decoding(dtype, model_folders):
     assert llm.generate(prompts, max_new_tokens=12, temperature=0.8, seed=5) == sampled
 
 
-def test_running_out_of_pages_preempts_and_still_gives_the_same_tokens(model_folders):
+def assert_sampled_matches(got, want, prompts, cfg, weights, temperature, seed, exact):
+    """Tokens drawn with a temperature by two runs that cut or batch the work differently.  The float32 engine
+    must give the same tokens.  In bfloat16 the two runs' logits differ by rounding, so a draw may fall on the
+    other side of an edge of the cumulative distribution: at the first difference, both tokens must lie within
+    2 % of probability mass of the request's uniform number in the plain implementation's distribution."""
+    for index, (prompt, tokens, expected) in enumerate(zip(prompts, got, want)):
+        if tokens == expected:
+            continue
+        assert not exact, f"float32 tokens {tokens} differ from {expected}"
+        first = next(i for i, (a, b) in enumerate(zip(tokens, expected)) if a != b)
+        logits = plain.model_logits(cfg, weights, prompt + expected[:first])[-1]
+        cdf = torch.cumsum(plain.sampling_distribution(logits, [], temperature).double(), dim=0)
+        u = uniform(seed + index, first)
+        for token in (tokens[first], expected[first]):
+            low = float(cdf[token - 1]) if token > 0 else 0.0
+            assert low - 0.02 <= u <= float(cdf[token]) + 0.02, \
+                f"prompt {index}, token {first}: {token} covers [{low:.4f}, {float(cdf[token]):.4f}], drawn at {u:.4f}"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_running_out_of_pages_preempts_and_still_gives_the_same_tokens(dtype, model_folders):
     vocab = TINY["A"]["config"].vocab_size
     prompts = [token_ids(vocab, n, 30 + n) for n in (30, 28, 25)]
-    roomy = LLM(model_folders["A"], dtype="float32", block_size=16, num_blocks=32, max_concurrent=3, eos_token_id=-1)
+    cfg, weights = plain.read_model(model_folders["A"])
+    roomy = LLM(model_folders["A"], dtype=dtype, block_size=16, num_blocks=32, max_concurrent=3, eos_token_id=-1)
     want = roomy.generate(prompts, max_new_tokens=24, temperature=0.7, seed=1)
-    tight = LLM(model_folders["A"], dtype="float32", block_size=16, num_blocks=7, max_concurrent=3, eos_token_id=-1)
+    tight = LLM(model_folders["A"], dtype=dtype, block_size=16, num_blocks=7, max_concurrent=3, eos_token_id=-1)
     got = tight.generate(prompts, max_new_tokens=24, temperature=0.7, seed=1)
-    assert got == want
+    assert_sampled_matches(got, want, prompts, cfg, weights, 0.7, 1, exact=dtype == "float32")
     assert tight.kv_manager.free_pages() == [7]
+    tight.kv_manager.check_invariants()
+    assert tight.scheduler.preemptions > 0 and roomy.scheduler.preemptions == 0
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_temperature_sampling_does_not_depend_on_the_batch(dtype, model_folders):
+    """A request's draws come from its own seed and token count: alone, or in portions of 7 beside four others,
+    it gets the same tokens (in bfloat16 up to draws that sit on an edge of the distribution)."""
+    vocab = TINY["B"]["config"].vocab_size
+    prompts = [token_ids(vocab, n, 20 + n) for n in (1, 9, 40, 64, 100)]
+    cfg, weights = plain.read_model(model_folders["B"])
+    together = LLM(model_folders["B"], dtype=dtype, block_size=8, num_blocks=64, max_concurrent=5,
+                   max_num_batched_tokens=24, max_chunk=7, eos_token_id=-1)
+    sampled = together.generate(prompts, max_new_tokens=12, temperature=0.8, seed=5)
+    alone = LLM(model_folders["B"], dtype=dtype, block_size=8, num_blocks=64, max_concurrent=1, eos_token_id=-1)
+    single = [alone.generate(prompt, max_new_tokens=12, temperature=0.8, seed=5 + index)
+              for index, prompt in enumerate(prompts)]
+    assert_sampled_matches(sampled, single, prompts, cfg, weights, 0.8, 5, exact=dtype == "float32")
+    # and they are draws from the plain implementation's distribution, not just equal to each other
+    for index, (prompt, tokens) in enumerate(zip(prompts, single)):
+        logits = plain.model_logits(cfg, weights, prompt)[-1]
+        cdf = torch.cumsum(plain.sampling_distribution(logits, [], 0.8).double(), dim=0)
+        u, token = uniform(5 + index, 0), tokens[0]
+        low = float(cdf[token - 1]) if token > 0 else 0.0
+        slack = 1e-5 if dtype == "float32" else 0.02
+        assert low - slack <= u <= float(cdf[token]) + slack
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_generation_of_the_windowed_configuration(dtype, model_folders):
+    """Layers with a window of 20 keys beside layers that see everything: greedy tokens through the entry point
+    (scheduler, captured decode steps, running ahead) against the plain implementation, with prompts shorter and
+    longer than the window and portions that straddle it; the window's pages come back while requests run."""
+    vocab = TINY["C"]["config"].vocab_size
+    prompts = [token_ids(vocab, n, 60 + n) for n in (3, 19, 21, 47, 90)]
+    want, cfg, weights = plain_greedy(model_folders["C"], prompts, 30)
+    llm = LLM(model_folders["C"], dtype=dtype, block_size=16, num_blocks=40, max_concurrent=5,
+              max_num_batched_tokens=40, max_chunk=13, eos_token_id=-1)
+    assert len(llm.kv_manager.groups) == 2
+    got = llm.generate(prompts, max_new_tokens=30, temperature=0.0)
+    assert_greedy_matches(got, want, prompts, cfg, weights, exact=dtype == "float32")
+    assert llm.kv_manager.free_pages() == [40, 40]
+    llm.kv_manager.check_invariants()
+    assert llm.engine.steps_run_ahead > 0
+
+
+def test_a_step_whose_forward_raises_gives_its_pages_back(model_folders):
+    from somi_inference_amd.engine import StepEntry
+    llm = LLM(model_folders["A"], dtype="bfloat16", block_size=16, num_blocks=8, max_concurrent=2, eos_token_id=-1)
+    runner, cache = llm.runner, llm.kv_manager
+    runner.begin("r")
+    runner.step([StepEntry("r", list(range(10)), [9])])
+    free = cache.free_pages()
+    forward = runner.model.forward
+
+    def failing(batch, caches):
+        raise RuntimeError("a kernel refused its arguments")
+    runner.model.forward = failing
+    with pytest.raises(RuntimeError, match="refused"):
+        runner.step([StepEntry("r", list(range(30)), [])])          # two more pages reserved, none committed
+    runner.model.forward = forward
+    assert cache.free_pages() == free and cache.num_tokens("r") == 10
+    cache.check_invariants()
+    again = runner.step([StepEntry("r", list(range(30)), [29])])    # and the request goes on from where it stood
+    assert again.shape[0] == 1 and cache.num_tokens("r") == 40
+    runner.end("r")
+    # through the entry point: the call's requests are aborted, the next call runs
+    calls = {"n": 0}
+
+    def failing_later(batch, caches):
+        calls["n"] += 1
+        if calls["n"] == 3:
+            raise RuntimeError("a kernel refused its arguments")
+        return forward(batch, caches)
+    runner.model.forward = failing_later
+    runner.decode_graphs = False
+    prompts = [list(range(5, 25)), list(range(40, 47))]
+    with pytest.raises(RuntimeError, match="refused"):
+        llm.generate(prompts, max_new_tokens=6, temperature=0.0)
+    runner.model.forward = forward
+    assert cache.free_pages() == [8] and not cache.live_requests()
+    want, cfg, weights = plain_greedy(model_folders["A"], prompts, 6)
+    assert_greedy_matches(llm.generate(prompts, max_new_tokens=6, temperature=0.0), want, prompts, cfg, weights, exact=False)
 
 
 def test_eos_ends_a_request_and_is_kept(model_folders):

@@ -122,6 +122,39 @@ def test_mixed_batches_with_so_few_pages_that_they_are_used_again(name, dtype, p
     assert runner.cache.free_pages() == [pages] * len(runner.cache.groups)
 
 
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_float32_engine_on_weights_stored_in_float32(name, tmp_path):
+    """The other folders hold bfloat16 values, which a product that rounded its operands to bfloat16 would
+    multiply exactly.  Here every tensor is stored in float32 with a full mantissa (and stays so on the device),
+    attention is sharpened, and the float32 engine must still meet the float32 tolerance under every cutting."""
+    from safetensors.torch import load_file
+    from somi_inference_amd.weights import write_random_model
+    config, bs = TINY[name]["config"], TINY[name]["block_size"]
+    base = write_random_model(str(tmp_path / "f32"), config, seed=TINY[name]["seed"], stored=torch.float32)
+    folder = peaky_folder(base, str(tmp_path / "f32_peaky"))
+    stored = load_file(f"{folder}/model.safetensors")
+    assert all(t.dtype == torch.float32 for t in stored.values())
+    some = stored["model.layers.0.mlp.down_proj.weight"]
+    assert not torch.equal(some, some.bfloat16().float()), "the stored values would survive a rounding to bfloat16"
+    cfg, weights = plain.read_model(folder)
+    tokens = token_ids(config.vocab_size, 150, 3)
+    want = plain.model_logits(cfg, weights, tokens)
+    runner, _ = make_engine(folder, "float32", bs, 32)
+    assert runner.model.layers[0].feed_forward.down.weight.dtype == torch.float32
+    whole = run_portions(runner, "w", tokens, [150])
+    assert_close(whole, want, "float32", f"{name} float32 weights: whole prompt")
+    for sizes in ([118] + [1] * 32, [7, 2, 5, 3, 11, 2, 16, 2, 29]):
+        got = run_portions(runner, "c", tokens, sizes)
+        assert_close(got, want, "float32", f"{name} float32 weights: portions {sizes[:4]}")
+        assert torch.equal(got, whole)
+    # the bfloat16 engine rounds these weights once, at load: it agrees with the plain implementation run on the
+    # rounded values
+    lowp, _ = make_engine(folder, "bfloat16", bs, 32)
+    rounded = {k: v.bfloat16().float() if v.dim() == 2 else v for k, v in weights.items()}
+    assert_close(run_portions(lowp, "w", tokens, [150]), plain.model_logits(cfg, rounded, tokens), "bfloat16",
+                 f"{name} float32 weights in the bfloat16 engine")
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_pages_beyond_two_to_the_31_elements_of_a_cache_tensor(dtype, peaky_folders, oracle):
     """A pool sized for a large GPU: the pool hands out its highest pages first, so the first request's keys

@@ -40,7 +40,7 @@ def random_case(seed: int, odd: bool = False):
 
 
 @pytest.mark.parametrize("odd", [False, True], ids=["even", "odd"])
-@pytest.mark.parametrize("seed", range(16))
+@pytest.mark.parametrize("seed", range(40))
 def test_random_configuration_under_a_random_mixed_trace(seed, odd, tmp_path):
     rng, config, block_size = random_case(seed, odd)
     base = write_random_model(str(tmp_path / "model"), config, seed=rng.randrange(1000))

@@ -201,6 +201,87 @@ def test_model_logits_do_not_depend_on_a_shift_of_positions():
                                P.model_logits(cfg, w, ids, first_position=29), atol=1e-9, rtol=1e-9)
 
 
+# ------------------------------------------------------------------------------ projections, head split, final norm
+def test_linear_is_library_linear_with_its_bias():
+    # /root/reference/somi_inference/models/qwen2.py:268-271: nn.Linear, weight [out, in]; a transposed weight or a
+    # dropped bias fails
+    x, w, b = torch.randn(5, 7), torch.randn(3, 7), torch.randn(3)
+    torch.testing.assert_close(P.linear(x, w, b), F.linear(x, w, b))
+    torch.testing.assert_close(P.linear(x, w), F.linear(x, w))
+    assert not torch.allclose(P.linear(x, w, b), F.linear(x, w), atol=1e-3)
+
+
+def _attention_weights(prefix, h, nq, nkv, d, fill):
+    w = {}
+    for name, rows in (("q_proj", nq * d), ("k_proj", nkv * d), ("v_proj", nkv * d)):
+        w[f"{prefix}.{name}.weight"] = fill(rows, h)
+        w[f"{prefix}.{name}.bias"] = fill(rows)
+    w[f"{prefix}.o_proj.weight"] = fill(h, nq * d)
+    return w
+
+
+def test_a_value_bias_alone_comes_out_as_the_output_projection_of_the_bias():
+    """/root/reference/somi_inference/models/qwen2.py:270, 290, 297: v = x . Wv^T + bv.  With every attention
+    tensor zero but the value bias and the output projection, every softmax is uniform over equal values, so
+    each token's output is o_proj(bv repeated for the query heads of its kv head), whatever x is.  A value bias
+    that is dropped (a key bias cancels in the softmax and would not be missed) gives zero instead."""
+    h, nq, nkv, d = 10, 4, 2, 6
+    cfg = dict(num_attention_heads=nq, num_key_value_heads=nkv, head_dim=d, rope_theta=1e4)
+    w = _attention_weights("a", h, nq, nkv, d, lambda *s: torch.zeros(*s))
+    bv = torch.randn(nkv * d)
+    wo = torch.randn(h, nq * d)
+    w["a.v_proj.bias"], w["a.o_proj.weight"] = bv, wo
+    out = P.attention_block(torch.randn(7, h), w, "a", cfg, torch.arange(7), None)
+    merged = bv.view(nkv, d).repeat_interleave(nq // nkv, dim=0).reshape(nq * d)      # query head h reads kv head h // 2
+    torch.testing.assert_close(out, (wo @ merged).expand(7, h))
+    assert out.abs().max() > 1e-2
+
+
+def test_heads_are_contiguous_blocks_of_head_dim_of_a_projection():
+    """/root/reference/somi_inference/models/qwen2.py:292-297, 285: view(.., n_heads, head_dim): head h of a
+    projection is its elements [h D, (h + 1) D), and the heads are merged in the same order before o_proj.
+    Checked against a loop that slices those ranges explicitly and calls the library's attention once per query
+    head; heads interleaved (element i belongs to head i mod n) fail it."""
+    h, nq, nkv, d, t = 12, 4, 2, 8, 6
+    cfg = dict(num_attention_heads=nq, num_key_value_heads=nkv, head_dim=d, rope_theta=1e4)
+    w = _attention_weights("a", h, nq, nkv, d, lambda *s: torch.randn(*s) * 0.5)
+    x, positions = torch.randn(t, h), torch.arange(t)
+    got = P.attention_block(x, w, "a", cfg, positions, None)
+    q = F.linear(x, w["a.q_proj.weight"], w["a.q_proj.bias"])
+    k = F.linear(x, w["a.k_proj.weight"], w["a.k_proj.bias"])
+    v = F.linear(x, w["a.v_proj.weight"], w["a.v_proj.bias"])
+    cos, sin = P.rope_cos_sin(positions, d, 1e4)
+    rotate = lambda block: block * cos + P.rotate_half(block) * sin
+    merged = torch.zeros(t, nq * d)
+    for head in range(nq):
+        kv = head // (nq // nkv)
+        qh = rotate(q[:, head * d:(head + 1) * d])
+        kh = rotate(k[:, kv * d:(kv + 1) * d])
+        vh = v[:, kv * d:(kv + 1) * d]
+        merged[:, head * d:(head + 1) * d] = F.scaled_dot_product_attention(qh[None], kh[None], vh[None], is_causal=True)[0]
+    torch.testing.assert_close(got, F.linear(merged, w["a.o_proj.weight"]), atol=1e-5, rtol=1e-5)
+
+
+def test_final_norm_stands_between_the_last_layer_and_the_head():
+    """/root/reference/somi_inference/models/qwen2.py:378, 386 and qwen2_adapter.py:60-62: logits =
+    head(norm(h)).  The norm's weight scales the logits linearly (a norm applied after the head, or none, does
+    not), and a model without layers has the closed form E . rmsnorm(E[id])."""
+    cfg, w = _tiny_weights(layers=2)
+    ids = [3, 1, 4, 1, 5]
+    base = P.model_logits(cfg, w, ids)
+    doubled = dict(w)
+    doubled["model.norm.weight"] = 2.0 * w["model.norm.weight"]
+    torch.testing.assert_close(P.model_logits(cfg, doubled, ids), 2.0 * base)
+    skewed = dict(w)
+    skewed["model.norm.weight"] = torch.linspace(0.5, 2.0, 8)
+    assert not torch.allclose(P.model_logits(cfg, skewed, ids), base, atol=1e-3)
+    empty = dict(cfg, num_hidden_layers=0)
+    table = w["model.embed_tokens.weight"]
+    rows = table[torch.tensor(ids)]
+    want = (skewed["model.norm.weight"] * rows * torch.rsqrt(rows.pow(2).mean(-1, keepdim=True) + 1e-6)) @ table.t()
+    torch.testing.assert_close(P.model_logits(empty, skewed, ids), want)
+
+
 # ------------------------------------------------------------------------------ sampling rules
 def test_sampling_vectors_of_reference_tests():
     # /root/reference/tests/core/test_sampler.py:58-128
