@@ -1,0 +1,500 @@
+// Linear layer for many rows (prompt portions, decode batches beyond 64 requests):
+// out[m, n] = sum_k x[m, k] * w[n, k], bfloat16 in, float32 accumulation on the matrix cores, with the
+// feed-forward's and the block's element-wise work in the end of the product.
+//
+// Reference: the reference has a kernel of its own for the feed-forward's two products
+// (somi_inference/core/mlp_triton.py:28-108, launched at :162-211, used at models/qwen2.py:231-249); its
+// q/k/v and o products are nn.Linear (models/qwen2.py:268-271).  The forms here:
+//   plain     out = s[m] * (x . w^T) + bias             (bfloat16; s: the row scale of an RMS norm, or 1)
+//   swiglu    out = silu(s g) * (s u), g and u the gate and up products    (models/qwen2.py:226-229)
+//   residual  h += x . w^T + bias in float32, in place (models/qwen2.py:333-339), leaving what the next
+//             norm needs: bfloat16(norm_w * h) and the rows' sums of squares in partial sums
+//
+// How it maps to gfx950:
+//   * a workgroup owns a 256 x 256 or 256 x 128 tile of the output and walks K in stages of 64 (one
+//     128-byte line per row: the L2 serves whole lines, half-used lines cost as much as full ones);
+//   * both operands come by direct-to-LDS loads of 16 bytes a lane into a ring of stages (two for the wide
+//     tile: 2 x 64 KB; three for the narrow one: 3 x 48 KB).  The 16-byte piece c of row r lies at piece
+//     position c ^ ((r >> 1) & 7): the LDS has 64 banks of 4 bytes, so 16 lanes of a 16-byte read must
+//     cover 256 distinct bytes; the permutation is applied on the global side of the load (a lane's LDS
+//     position is fixed by the instruction);
+//   * a wavefront computes 128 x 64 of the tile as 4 x 2 products of 32 x 32 x 16 (128 accumulator
+//     registers); 8 wavefronts (wide) or 4 (narrow).  Two wavefronts on a SIMD matter: within one
+//     wavefront no instruction overlaps its own matrix instruction, so loads and LDS reads of one hide
+//     behind the products of the other;
+//   * fragment reads are software-pipelined one 16-deep sub-step ahead and issued between the products;
+//     the order of instructions in the loop is pinned (the compiler's own schedule waited for each read
+//     right after issuing it);
+//   * products are taken transposed (D[n][m]): a lane then holds 4 consecutive columns of one row, so the
+//     gate and up value of a channel (16 columns apart) meet in one lane, and a row's values are packed
+//     and turned through LDS into stores of whole 128-byte rows;
+//   * workgroups are numbered so that the eight dies (blockIdx % 8) each take a contiguous range of
+//     tiles, the row tiles of one column tile next to each other: a weight tile is read from HBM by
+//     one die only.
+// Measured on an MI355X (2,048 rows): 256 x 128 tiles over K = 18,944 run at 1.2 PFLOP/s; 256 x 256 tiles
+// over K = 3,584 at 1.05 to 1.1 (4.3 GB go from the L2s to the compute units per call; that stream
+// alone takes 390 us and the products alone 310).
+#include "common.h"
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
+
+#define BIG_GLOBAL __attribute__((address_space(1)))
+#define BIG_LDS __attribute__((address_space(3)))
+#define BIG_FENCE() __builtin_amdgcn_sched_barrier(0)
+
+#define BIG_PLAIN 0
+#define BIG_SWIGLU 1
+#define BIG_RESIDUAL 2
+
+#define BIG_BK 64                 // K per stage: one 128-byte line per row
+#define BIG_ROW_BYTES 128
+#define BIG_BM 256
+
+// A stage's pieces past K read from here, so that a K that is no multiple of 64 adds zeros.
+static __device__ __align__(16) unsigned int big_zero_piece[4];
+
+struct BigArgs {
+    const bf16* x; int64_t ldx;       // [M, K], row stride in elements
+    const bf16* w; int64_t ldw;       // [N, K]
+    const float* bias;                // [N] or null
+    int M, N, K;
+    int tiles_m, tiles_n;
+    // plain / swiglu
+    bf16* out;                        // [M, N] or [M, N / 2]
+    const float* stats_in;            // [stats_blocks][stats_width] partial sums of squares of the rows, or null
+    int stats_blocks, stats_width;
+    float eps;
+    // residual
+    float* h;                         // [M, N] float32, in and out
+    const float* norm_w;              // [N] or null
+    bf16* weighted;                   // [M, N] = bfloat16(norm_w * h) or null
+    float* stats_out;                 // [tiles_n * waves along n][stats_width] or null
+};
+
+template <int N> __device__ __forceinline__ void big_wait_vmcnt() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
+
+// One fragment read that the compiler does not track: every register it fills is named by the wait that
+// precedes its first use (so that no use can be moved before the wait).
+#define BIG_DS_READ(dst, addr, off) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(off))
+
+template <int BN, int S, int NW, int EPI, bool KTAIL>
+__global__ void __launch_bounds__(NW * 64, 1)
+linear_big_kernel(const BigArgs p) {
+    extern __shared__ __attribute__((aligned(1024))) char lds[];
+    constexpr int BM = BIG_BM, BK = BIG_BK, ROW_BYTES = BIG_ROW_BYTES;
+    constexpr int A_BYTES = BM * ROW_BYTES, B_BYTES = BN * ROW_BYTES, STAGE = A_BYTES + B_BYTES;
+    constexpr int WAVES_N = NW / 2;                               // wavefronts: 2 along m, NW / 2 along n
+    constexpr int WTM = 4, WTN = 2;                               // 32 x 32 products of a wavefront: 128 x 64
+    static_assert(BM / 2 == WTM * 32 && BN / WAVES_N == WTN * 32, "a wavefront owns 128 x 64 of the tile");
+    constexpr int LA = BM / 8 / NW, LB = BN / 8 / NW, L = LA + LB;  // direct loads a lane issues per stage (8 rows each)
+    constexpr int KK = BK / 16, NM = WTM * WTN, NF = WTM + WTN;
+    constexpr bool TWO = S == 2;
+    static_assert(TWO || L % KK == 0, "loads divisible over the sub-steps");
+    constexpr int LPS = TWO ? 0 : L / KK;
+    constexpr int AHEAD = TWO ? 2 : S - 1;                        // stages issued before the loop
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+    const int M = p.M, N = p.N, K = p.K;
+
+    const int total = p.tiles_m * p.tiles_n, per = (total + 7) / 8;
+    const int logical = (blockIdx.x & 7) * per + (blockIdx.x >> 3);
+    if (logical >= total) return;
+    const int tn = logical / p.tiles_m, tm = logical % p.tiles_m;
+    const int m0 = tm * BM, n0 = tn * BN;
+    const char* xa = (const char*)(p.x + (int64_t)m0 * p.ldx);
+    const char* wb = (const char*)(p.w + (int64_t)n0 * p.ldw);
+    const int mlim = M - m0, nlim = N - n0;
+    const int KT = (K + BK - 1) / BK;
+
+    // ------------------------------------------------------------------ loads: global -> LDS
+    // An instruction covers 8 rows of 128 bytes; lane l writes LDS position l % 8 of row l / 8 and reads the
+    // global piece that belongs there.  Rows past the matrix repeat its last row (never stored).
+    const int lrow = lane >> 3, lpos = lane & 7;
+    uint32_t offa[LA], offb[LB];
+    int piece_a[LA], piece_b[LB];
+#pragma unroll
+    for (int i = 0; i < LA; ++i) {
+        const int row = (wave * LA + i) * 8 + lrow;
+        piece_a[i] = lpos ^ ((row >> 1) & 7);
+        offa[i] = (uint32_t)(row < mlim ? row : mlim - 1) * (uint32_t)p.ldx * 2u + (piece_a[i] << 4);
+    }
+#pragma unroll
+    for (int i = 0; i < LB; ++i) {
+        const int row = (wave * LB + i) * 8 + lrow;
+        piece_b[i] = lpos ^ ((row >> 1) & 7);
+        offb[i] = (uint32_t)(row < nlim ? row : nlim - 1) * (uint32_t)p.ldw * 2u + (piece_b[i] << 4);
+    }
+    auto issue_load = [&](int kt, int buf, int i) {
+        const char* src;
+        char* dst;
+        int piece;
+        if (i < LA) {
+            src = xa + (int64_t)kt * ROW_BYTES + offa[i];
+            dst = lds + buf * STAGE + (wave * LA + i) * 1024;
+            piece = piece_a[i];
+        } else {
+            src = wb + (int64_t)kt * ROW_BYTES + offb[i - LA];
+            dst = lds + buf * STAGE + A_BYTES + (wave * LB + i - LA) * 1024;
+            piece = piece_b[i - LA];
+        }
+        if (KTAIL) {
+            if (kt * BK + piece * 8 >= K) src = (const char*)big_zero_piece;
+        }
+        __builtin_amdgcn_global_load_lds((const BIG_GLOBAL void*)src, (BIG_LDS void*)dst, 16, 0, 0);
+    };
+
+    f32x16 acc[WTM][WTN];
+#pragma unroll
+    for (int i = 0; i < WTM; ++i)
+#pragma unroll
+        for (int j = 0; j < WTN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+    // ------------------------------------------------------------------ fragments: LDS -> registers
+    const int frow = lane & 31, fk = lane >> 5;
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(BIG_LDS char*)lds;
+    uint32_t foffa[KK], foffb[KK];
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+        const uint32_t f = frow * ROW_BYTES + (((kk * 2 + fk) ^ ((frow >> 1) & 7)) << 4);
+        foffa[kk] = lds_base + f + wm * (BM / 2) * ROW_BYTES;
+        foffb[kk] = lds_base + f + A_BYTES + wn * (BN / WAVES_N) * ROW_BYTES;
+    }
+    // read q of a set, in the order the products need them: a[0], every b, then the other a
+    auto read_one = [&](bf16x8 (&a)[WTM], bf16x8 (&b)[WTN], uint32_t aa, uint32_t ab, int q) {
+        if (q == 0) BIG_DS_READ(a[0], aa, 0);
+        else if (q == 1) BIG_DS_READ(b[0], ab, 0);
+        else if (q == 2) BIG_DS_READ(b[1], ab, 32 * ROW_BYTES);
+        else if (q == 3) BIG_DS_READ(a[1], aa, 32 * ROW_BYTES);
+        else if (q == 4) BIG_DS_READ(a[2], aa, 64 * ROW_BYTES);
+        else if (q == 5) BIG_DS_READ(a[3], aa, 96 * ROW_BYTES);
+    };
+    auto wait_frags = [&](bf16x8 (&a)[WTM], bf16x8 (&b)[WTN]) {
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(b[0]), "+v"(b[1]));
+    };
+    auto product = [&](bf16x8 (&a)[WTM], bf16x8 (&b)[WTN], int q) {
+        const int i = q / WTN, j = q % WTN;
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b[j], a[i], acc[i][j], 0, 0, 0);    // D[n][m]
+    };
+
+    // ------------------------------------------------------------------ the ring
+    // Three stages or more: the slot freed one iteration ago is refilled evenly over the sub-steps.  Two: the
+    // stage just read is refilled in a burst after the barrier.
+#pragma unroll
+    for (int st = 0; st < AHEAD; ++st)
+#pragma unroll
+        for (int i = 0; i < L; ++i) issue_load(st < KT ? st : KT - 1, st, i);
+    big_wait_vmcnt<(AHEAD - 1) * L>();
+    __syncthreads();
+
+    bf16x8 a0[WTM], b0[WTN], a1[WTM], b1[WTN];
+#pragma unroll
+    for (int q = 0; q < NF; ++q) read_one(a0, b0, foffa[0], foffb[0], q);
+    int buf = 0, rbuf = TWO ? 0 : S - 1;    // the stage computed on; the slot being refilled
+    constexpr int SYNC_AFTER = 2;           // products of the last sub-step issued before the barrier
+    for (int kt = 0; kt < KT; ++kt) {
+        const int nbuf = buf + 1 == S ? 0 : buf + 1;
+        const int rstage = kt + AHEAD < KT ? kt + AHEAD : KT - 1;      // past the end: a harmless repeat
+        if (TWO) rbuf = buf;
+        BIG_FENCE();
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) {
+            const bool last = kk == KK - 1;
+            const uint32_t aa = (last ? foffa[0] + nbuf * STAGE : foffa[kk + 1 < KK ? kk + 1 : 0] + buf * STAGE);
+            const uint32_t ab = (last ? foffb[0] + nbuf * STAGE : foffb[kk + 1 < KK ? kk + 1 : 0] + buf * STAGE);
+            BIG_FENCE();
+            if (kk & 1) wait_frags(a1, b1); else wait_frags(a0, b0);
+            BIG_FENCE();
+            int reads = 0, loads = 0;
+            constexpr int PER_SLOT = TWO ? (L + NF - 1) / NF : 1;
+#pragma unroll
+            for (int q = 0; q < NM; ++q) {
+                if (last && q == SYNC_AFTER) {
+                    // the next stage has landed and everybody has read this one
+                    big_wait_vmcnt<TWO ? 0 : (S - 3) * L + LPS * (KK - 1)>();
+                    __builtin_amdgcn_s_barrier();
+                    BIG_FENCE();
+                }
+                if (kk & 1) product(a1, b1, q); else product(a0, b0, q);
+                BIG_FENCE();
+                if ((!last || q >= SYNC_AFTER) && reads < NF) {
+                    if (kk & 1) read_one(a0, b0, aa, ab, reads); else read_one(a1, b1, aa, ab, reads);
+                    ++reads;
+                    if (TWO) {
+                        if (last)
+#pragma unroll
+                            for (int e = 0; e < PER_SLOT; ++e)
+                                if (loads < L) { issue_load(rstage, rbuf, loads); ++loads; }
+                    } else if (loads < LPS) { issue_load(rstage, rbuf, kk * LPS + loads); ++loads; }
+                    BIG_FENCE();
+                }
+            }
+        }
+        if (!TWO) rbuf = buf;
+        buf = nbuf;
+    }
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    __syncthreads();                       // the ring is free: its memory serves the epilogue
+
+    // ------------------------------------------------------------------ epilogue
+    // A product holds D[n][m]: lane l has row m = l % 32 and, in registers 4 g .. 4 g + 3, the columns
+    // 8 g + 4 (l / 32) + 0..3 of its 32.  A wavefront turns 32 rows at a time through its own 16 KB of LDS
+    // into whole rows and stores 16 bytes a lane.
+    char* stg = lds + wave * 16384;
+    const int ml = lane & 31, nh = lane >> 5;
+    const int wave_n0 = n0 + wn * (BN / WAVES_N);            // first column of the wavefront
+
+    // the row scale of the norm whose rows x holds (plain and swiglu)
+    float scale[WTM];
+#pragma unroll
+    for (int i = 0; i < WTM; ++i) scale[i] = 1.f;
+    if (EPI != BIG_RESIDUAL && p.stats_in != nullptr) {
+#pragma unroll
+        for (int i = 0; i < WTM; ++i) {
+            const int gm = m0 + wm * (BM / 2) + i * 32 + ml;
+            float sum = 0.f;
+            if (gm < M)
+                for (int b = 0; b < p.stats_blocks; ++b) sum += p.stats_in[(int64_t)b * p.stats_width + gm];
+            scale[i] = rsqrtf(sum / (float)K + p.eps);
+        }
+    }
+
+    if (EPI == BIG_PLAIN || EPI == BIG_SWIGLU) {
+        constexpr int CW = EPI == BIG_SWIGLU ? WTN * 16 : WTN * 32;      // output columns of the wavefront per row
+        constexpr int SROW = CW * 2 + 8;                                   // staged row: 8 bytes of padding spread the banks
+        constexpr int LPR = CW * 2 / 16;                                   // lanes per row when reading back
+        const int out_n = EPI == BIG_SWIGLU ? N / 2 : N;
+        const int out_c0 = EPI == BIG_SWIGLU ? wave_n0 / 2 : wave_n0;
+        const bool aligned = (out_n & 7) == 0 && ((uintptr_t)p.out & 15) == 0;
+#pragma unroll
+        for (int i = 0; i < WTM; ++i) {
+            const float s = scale[i];
+#pragma unroll
+            for (int j = 0; j < WTN; ++j) {
+                const f32x16& t = acc[i][j];
+                if (EPI == BIG_SWIGLU) {
+                    // registers r and r + 8 are gate and up of one channel (columns 16 apart)
+#pragma unroll
+                    for (int g = 0; g < 2; ++g) {
+                        bf16x4 v;
+#pragma unroll
+                        for (int c = 0; c < 4; ++c) {
+                            const float gate = s * t[4 * g + c], up = s * t[4 * g + c + 8];
+                            v[c] = (bf16)(gate / (1.f + expf(-gate)) * up);
+                        }
+                        *(bf16x4*)(stg + ml * SROW + (j * 16 + 8 * g + 4 * nh) * 2) = v;
+                    }
+                } else {
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                        bf16x4 v;
+#pragma unroll
+                        for (int c = 0; c < 4; ++c) {
+                            float val = s * t[4 * g + c];
+                            if (p.bias != nullptr) {
+                                const int gn = wave_n0 + j * 32 + 8 * g + 4 * nh + c;
+                                val += p.bias[gn < N ? gn : N - 1];
+                            }
+                            v[c] = (bf16)val;
+                        }
+                        *(bf16x4*)(stg + ml * SROW + (j * 32 + 8 * g + 4 * nh) * 2) = v;
+                    }
+                }
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+            for (int pass = 0; pass < 32 * LPR / 64; ++pass) {
+                const int row = pass * (64 / LPR) + lane / LPR, piece = lane % LPR;
+                const u32x4 v = *(const u32x4*)(stg + row * SROW + piece * 16);
+                const int gm = m0 + wm * (BM / 2) + i * 32 + row;
+                const int gc = out_c0 + piece * 8;
+                if (gm < M) {
+                    bf16* dst = p.out + (int64_t)gm * out_n + gc;
+                    if (aligned && gc + 8 <= out_n) *(u32x4*)dst = v;
+                    else {
+                        const bf16* e = (const bf16*)&v;
+                        for (int c = 0; c < 8; ++c)
+                            if (gc + c < out_n) dst[c] = e[c];
+                    }
+                }
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        }
+    } else {
+        // h += product (+ bias), 32 rows x 64 columns of float32 at a time; a row is read back by 16 lanes
+        constexpr int CW = WTN * 32;
+        constexpr int SROW = CW * 4 + 16;
+        const bool aligned = (N & 3) == 0 && ((uintptr_t)p.h & 15) == 0 &&
+                             (p.weighted == nullptr || ((uintptr_t)p.weighted & 7) == 0);
+        const int stats_row0 = (tn * WAVES_N + wn);
+#pragma unroll
+        for (int i = 0; i < WTM; ++i) {
+#pragma unroll
+            for (int j = 0; j < WTN; ++j)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const f32x16& t = acc[i][j];
+                    f32x4 v = {t[4 * g], t[4 * g + 1], t[4 * g + 2], t[4 * g + 3]};
+                    *(f32x4*)(stg + ml * SROW + (j * 32 + 8 * g + 4 * nh) * 4) = v;
+                }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+            for (int pass = 0; pass < 8; ++pass) {
+                const int row = pass * 4 + (lane >> 4), piece = lane & 15;
+                f32x4 v = *(const f32x4*)(stg + row * SROW + piece * 16);
+                const int gm = m0 + wm * (BM / 2) + i * 32 + row;
+                const int gn = wave_n0 + piece * 4;
+                float sq = 0.f;
+                if (gm < M && gn < N) {
+                    float* hp = p.h + (int64_t)gm * N + gn;
+                    if (aligned && gn + 4 <= N) {
+                        f32x4 hv = *(const f32x4*)hp;
+#pragma unroll
+                        for (int c = 0; c < 4; ++c) {
+                            hv[c] += v[c] + (p.bias != nullptr ? p.bias[gn + c] : 0.f);
+                            sq += hv[c] * hv[c];
+                        }
+                        *(f32x4*)hp = hv;
+                        if (p.weighted != nullptr) {
+                            bf16x4 wv;
+#pragma unroll
+                            for (int c = 0; c < 4; ++c) wv[c] = (bf16)(p.norm_w[gn + c] * hv[c]);
+                            *(bf16x4*)(p.weighted + (int64_t)gm * N + gn) = wv;
+                        }
+                    } else {
+                        for (int c = 0; c < 4; ++c)
+                            if (gn + c < N) {
+                                const float hv = hp[c] + v[c] + (p.bias != nullptr ? p.bias[gn + c] : 0.f);
+                                hp[c] = hv;
+                                sq += hv * hv;
+                                if (p.weighted != nullptr) p.weighted[(int64_t)gm * N + gn + c] = (bf16)(p.norm_w[gn + c] * hv);
+                            }
+                    }
+                }
+                if (p.stats_out != nullptr) {
+                    // the 16 lanes of a row add their squares in a fixed order
+#pragma unroll
+                    for (int off = 8; off > 0; off >>= 1) sq += __shfl_xor(sq, off, 64);
+                    if (piece == 0 && gm < M) p.stats_out[(int64_t)stats_row0 * p.stats_width + gm] = sq;
+                }
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        }
+    }
+}
+
+// ---------------------------------------------------------------------- host side
+static int big_compute_units() {
+    static int cached[64];
+    int device = 0;
+    if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) return 256;
+    if (cached[device] == 0) {
+        hipDeviceProp_t prop;
+        cached[device] = hipGetDeviceProperties(&prop, device) == hipSuccess && prop.multiProcessorCount > 0
+                             ? prop.multiProcessorCount : 256;
+    }
+    return cached[device];
+}
+
+// The wide tile moves fewer bytes per product and wins where it fills the device; the narrow one has twice the
+// workgroups.  Costs in units of a narrow tile's time: rounds of tiles x the tile's size (the narrow tile is
+// about 8 % less efficient per product).
+static bool big_use_wide(int m, int n) {
+    const int cus = big_compute_units();
+    const int tm = ceil_div(m, BIG_BM);
+    const double wide = (double)ceil_div(tm * ceil_div(n, 256), cus) * 2.0;
+    const double narrow = (double)ceil_div(tm * ceil_div(n, 128), cus) * 1.08;
+    return wide <= narrow;
+}
+
+template <int BN, int S, int NW, int EPI, bool KTAIL>
+static int big_launch_one(const BigArgs& args, hipStream_t stream) {
+    const int lds_bytes = S * (BIG_BM + BN) * BIG_ROW_BYTES;
+    static bool raised[64];
+    int device = 0;
+    hipError_t err = hipGetDevice(&device);
+    if (err != hipSuccess || device < 0 || device >= 64) return somi_fail("linear_big: hipGetDevice failed");
+    if (!raised[device]) {
+        err = hipFuncSetAttribute((const void*)linear_big_kernel<BN, S, NW, EPI, KTAIL>,
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+        if (err != hipSuccess) return somi_fail("linear_big: %d bytes of LDS refused: %s", lds_bytes, hipGetErrorString(err));
+        raised[device] = true;
+    }
+    const int per = ceil_div(args.tiles_m * args.tiles_n, 8);
+    hipLaunchKernelGGL((linear_big_kernel<BN, S, NW, EPI, KTAIL>), dim3(per * 8), dim3(NW * 64), lds_bytes, stream, args);
+    SOMI_LAUNCH_CHECK("linear_big");
+    return 0;
+}
+
+template <int EPI>
+static int big_launch(BigArgs& args, int tile, hipStream_t stream) {
+    const bool wide = tile == 0 ? big_use_wide(args.M, args.N) : tile == 256;
+    args.tiles_m = ceil_div(args.M, BIG_BM);
+    args.tiles_n = ceil_div(args.N, wide ? 256 : 128);
+    const bool ktail = args.K % BIG_BK != 0;
+    if (wide) return ktail ? big_launch_one<256, 2, 8, EPI, true>(args, stream) : big_launch_one<256, 2, 8, EPI, false>(args, stream);
+    return ktail ? big_launch_one<128, 3, 4, EPI, true>(args, stream) : big_launch_one<128, 3, 4, EPI, false>(args, stream);
+}
+
+static int big_check(const char* what, const void* x, int64_t ldx, const void* w, int64_t ldw, int m, int n, int k) {
+    SOMI_REQUIRE(m > 0 && n > 0 && k > 0, "%s: bad sizes m=%d n=%d k=%d", what, m, n, k);
+    SOMI_REQUIRE(k % 8 == 0, "%s: K = %d is no multiple of 8", what, k);
+    SOMI_REQUIRE(ldx >= k && ldw >= k && ldx % 8 == 0 && ldw % 8 == 0, "%s: row strides %lld and %lld must be multiples of 8 and >= K",
+                 what, (long long)ldx, (long long)ldw);
+    SOMI_REQUIRE(((uintptr_t)x & 15) == 0 && ((uintptr_t)w & 15) == 0, "%s: operands must be aligned to 16 bytes", what);
+    // a lane's byte offset inside a tile is 32-bit
+    SOMI_REQUIRE((int64_t)256 * ldx * 2 < ((int64_t)1 << 32) && (int64_t)256 * ldw * 2 < ((int64_t)1 << 32),
+                 "%s: rows too long for 32-bit offsets inside a tile", what);
+    return 0;
+}
+
+// Workgroup columns that write row statistics in the residual form: the first size of stats_out.
+// tile: 0 lets the launcher choose, 128 or 256 asks for that tile width.
+extern "C" int somi_linear_big_stats_blocks(int m, int n, int tile) {
+    const bool wide = tile == 0 ? big_use_wide(m, n) : tile == 256;
+    return wide ? ceil_div(n, 256) * 4 : ceil_div(n, 128) * 2;
+}
+
+// out = s * (x . w^T) + bias -> bfloat16 [M, N]; with swiglu w is [N, K] with gate and up rows interleaved in blocks
+// of 16 and out is [M, N / 2] = silu(s g) * (s u).  stats (or null): [stats_blocks][stats_width] partial sums of
+// squares; s[m] = 1 / sqrt(sum_b stats[b][m] / K + eps).
+extern "C" int somi_linear_big(const void* x, int64_t ldx, const void* w, int64_t ldw, const float* bias, void* out,
+                               int m, int n, int k, const float* stats, int stats_blocks, int stats_width, float eps,
+                               int swiglu, int tile, hipStream_t stream) {
+    if (big_check("linear_big", x, ldx, w, ldw, m, n, k) != 0) return 1;
+    SOMI_REQUIRE(out != nullptr, "linear_big: no output");
+    SOMI_REQUIRE(!swiglu || (n % 32 == 0 && bias == nullptr), "linear_big: the gated form needs N a multiple of 32 and no bias");
+    SOMI_REQUIRE(stats == nullptr || (stats_blocks > 0 && stats_width >= m), "linear_big: row statistics of %d x %d do not cover %d rows",
+                 stats_blocks, stats_width, m);
+    SOMI_REQUIRE(tile == 0 || tile == 128 || tile == 256, "linear_big: tile width %d (0, 128 or 256)", tile);
+    BigArgs args = {};
+    args.x = (const bf16*)x; args.ldx = ldx; args.w = (const bf16*)w; args.ldw = ldw; args.bias = bias;
+    args.M = m; args.N = n; args.K = k; args.out = (bf16*)out;
+    args.stats_in = stats; args.stats_blocks = stats_blocks; args.stats_width = stats_width; args.eps = eps;
+    return swiglu ? big_launch<BIG_SWIGLU>(args, tile, stream) : big_launch<BIG_PLAIN>(args, tile, stream);
+}
+
+// h += x . w^T + bias, float32 in place [M, N].  norm_w / weighted (or null): weighted = bfloat16(norm_w * h);
+// stats_out (or null): [somi_linear_big_stats_blocks(m, n, tile)][stats_width] sums of squares of the new h, each over
+// the 64 columns of one wavefront.
+extern "C" int somi_linear_big_residual(const void* x, int64_t ldx, const void* w, int64_t ldw, const float* bias, float* h,
+                                        const float* norm_w, void* weighted, float* stats_out, int stats_width,
+                                        int m, int n, int k, int tile, hipStream_t stream) {
+    if (big_check("linear_big_residual", x, ldx, w, ldw, m, n, k) != 0) return 1;
+    SOMI_REQUIRE(h != nullptr, "linear_big_residual: no residual stream");
+    SOMI_REQUIRE((weighted == nullptr) == (norm_w == nullptr), "linear_big_residual: the norm's weight and its rows come together");
+    SOMI_REQUIRE(stats_out == nullptr || stats_width >= m, "linear_big_residual: row statistics of width %d do not cover %d rows", stats_width, m);
+    SOMI_REQUIRE(tile == 0 || tile == 128 || tile == 256, "linear_big_residual: tile width %d (0, 128 or 256)", tile);
+    BigArgs args = {};
+    args.x = (const bf16*)x; args.ldx = ldx; args.w = (const bf16*)w; args.ldw = ldw; args.bias = bias;
+    args.M = m; args.N = n; args.K = k; args.h = h; args.norm_w = norm_w; args.weighted = (bf16*)weighted;
+    args.stats_out = stats_out; args.stats_width = stats_width;
+    return big_launch<BIG_RESIDUAL>(args, tile, stream);
+}

@@ -22,10 +22,18 @@ def _mid_is_faster(m: int, n: int, k: int) -> bool:
     return (k >= 8192 and n <= 8192) or n >= 16384
 
 
+# Above SKINNY_ROWS rows the products of the feed-forward run the many-rows kernel (ops.linear_big), also with
+# the norm before them and the residual add after them taken in.  The other products of that size (q/k/v, o,
+# logits of many rows) are plain library GEMMs in the reference; which of the two runs them here:
+BIG_FOR_ALL = True
+
+
 def linear_swiglu(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
-    """silu(x @ gate.T) * (x @ up.T) for at most SKINNY_ROWS bfloat16 rows; weight: [2 I, K], gate and up rows
-    interleaved in blocks of 16."""
+    """silu(x @ gate.T) * (x @ up.T) for bfloat16 rows; weight: [2 I, K], gate and up rows interleaved in blocks
+    of 16."""
     m, k = x.shape
+    if m > SKINNY_ROWS:
+        return ops.linear_big(x, weight, swiglu=True)
     if _mid_is_faster(m, weight.shape[0], k):
         return ops.linear_mid(x, weight, swiglu=True)
     return ops.linear_skinny_swiglu(x, weight)
@@ -35,6 +43,8 @@ def linear_residual(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | 
                     next_norm_weight: torch.Tensor | None = None) -> tuple[torch.Tensor, torch.Tensor | None]:
     """h += x @ weight.T (+ bias) in place, by the kernel that :func:`linear` would take for the sizes; see
     :func:`ops.linear_residual`."""
+    if x.shape[0] > ops.FUSED_MAX_ROWS:
+        return ops.linear_big_residual(x, weight, bias, h, next_norm_weight)
     mid = _mid_is_faster(x.shape[0], weight.shape[0], x.shape[1])
     return ops.linear_residual(x, weight, bias, h, next_norm_weight, mid=mid)
 
@@ -43,6 +53,8 @@ def linear_scaled(x: torch.Tensor, eps: float, stats: torch.Tensor, weight: torc
                   bias: torch.Tensor | None = None, swiglu: bool = False) -> torch.Tensor:
     """The product of rows that are still to be normed, by the kernel that :func:`linear` would take for the
     sizes; see :func:`ops.linear_scaled`."""
+    if x.shape[0] > ops.FUSED_MAX_ROWS:
+        return ops.linear_big(x, weight, bias, swiglu=swiglu, eps=eps, stats=stats)
     mid = _mid_is_faster(x.shape[0], weight.shape[0], x.shape[1])
     return ops.linear_scaled(x, eps, stats, weight, bias, swiglu, mid=mid)
 
@@ -67,6 +79,8 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = No
         if _mid_is_faster(m, weight.shape[0], k):
             return ops.linear_mid(x, weight, bias, out_dtype)
         return ops.linear_skinny(x, weight, bias, out_dtype)
+    if BIG_FOR_ALL and out_dtype == x.dtype and ops.big_supported(x, weight):
+        return ops.linear_big(x, weight, bias)
     if m <= MID_PASSES_ROWS and k >= 8192 and weight.shape[0] <= 8192 and out_dtype == x.dtype:
         # long K and few columns (down): the library's product leaves most of the device idle here (95 us at 65 to
         # 128 rows of the 7B down projection, 111 at 192); the split-K kernel, 64 rows at a time, takes 62 to 67 and 99

@@ -318,6 +318,78 @@ def _stats_width(rows: int) -> int:
     return 16 * ((rows + 15) // 16)
 
 
+def _big_operands(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, what: str) -> tuple[int, int, int]:
+    """Checks what the many-rows kernel assumes of its operands; x may be a view with a row stride of its own."""
+    for t, name in ((x, "input"), (weight, "weight")):
+        if not isinstance(t, torch.Tensor) or not t.is_cuda or t.dtype != torch.bfloat16 or t.dim() != 2 or t.stride(1) != 1:
+            raise KernelError(f"{what}: the {name} must be a bfloat16 matrix on the GPU with contiguous rows")
+    m, k = x.shape
+    n = weight.shape[0]
+    if weight.shape[1] != k:
+        raise KernelError(f"{what}: input has {k} features, weight expects {weight.shape[1]}")
+    if k % 8 or x.stride(0) % 8 or weight.stride(0) % 8 or x.data_ptr() % 16 or weight.data_ptr() % 16:
+        raise KernelError(f"{what}: K = {k} and the row strides must be multiples of 8 and the operands aligned to 16 bytes")
+    if bias is not None:
+        _need(bias, "linear bias", torch.float32, (n,))
+    return m, n, k
+
+
+def big_supported(x: torch.Tensor, weight: torch.Tensor) -> bool:
+    """The many-rows kernel takes these operands (bfloat16, K a multiple of 8, 16-byte alignment)."""
+    return (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and x.dim() == 2 and x.stride(1) == 1
+            and x.shape[1] % 8 == 0 and x.stride(0) % 8 == 0 and weight.stride(0) % 8 == 0
+            and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0)
+
+
+def linear_big(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None, *, swiglu: bool = False,
+               eps: float = 0.0, stats: torch.Tensor | None = None, tile: int = 0,
+               out: torch.Tensor | None = None) -> torch.Tensor:
+    """s * (x @ weight.T) (+ bias) -> bfloat16 for any number of rows, on 256-row tiles of the matrix cores.
+    With ``stats`` ([blocks, width >= M] partial sums of squares, from :func:`linear_big_residual` or
+    :func:`linear_residual`) the rows are scaled by s = 1 / sqrt(stats.sum(0) / K + eps): the product of
+    RMS-normed rows when x holds ``norm_weight * h``.  With ``swiglu`` weight is [2 I, K] with gate and up rows
+    interleaved in blocks of 16 and the result is silu(s g) * (s u) -> [M, I].  ``tile``: 0 lets the launcher
+    choose the tile width, 128 or 256 asks for it."""
+    m, n, k = _big_operands(x, weight, bias, "linear_big")
+    if swiglu and (n % 32 or bias is not None):
+        raise KernelError(f"linear_big: the gated form needs an even number of 16-row blocks and no bias, got N = {n}")
+    blocks = width = 0
+    if stats is not None:
+        _need(stats, "row statistics", torch.float32)
+        if stats.dim() != 2 or stats.shape[1] < m:
+            raise KernelError(f"linear_big: row statistics must be [blocks, >= {m}], got {tuple(stats.shape)}")
+        blocks, width = stats.shape
+    cols = n // 2 if swiglu else n
+    if out is None:
+        out = torch.empty((m, cols), dtype=torch.bfloat16, device=x.device)
+    _need(out, "linear_big out", torch.bfloat16, (m, cols))
+    _check(library().somi_linear_big(_ptr(x), ctypes.c_int64(x.stride(0)), _ptr(weight), ctypes.c_int64(weight.stride(0)),
+                                     _ptr(bias), _ptr(out), m, n, k, _ptr(stats), blocks, width, ctypes.c_float(eps),
+                                     1 if swiglu else 0, int(tile), _stream()))
+    return out
+
+
+def linear_big_residual(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, h: torch.Tensor,
+                        next_norm_weight: torch.Tensor | None = None, tile: int = 0
+                        ) -> tuple[torch.Tensor, torch.Tensor | None]:
+    """h += x @ weight.T (+ bias) in float32, in place, for any number of rows.  Returns the row statistics
+    ``[blocks, 16 ceil(M / 16)]`` (sums of squares of the new h, each over the 64 columns of one wavefront) and,
+    with ``next_norm_weight``, the rows ``bfloat16(next_norm_weight * h)``: what :func:`linear_big` scales."""
+    m, n, k = _big_operands(x, weight, bias, "linear_big_residual")
+    _need(h, "residual stream", torch.float32, (m, n))
+    lib = library()
+    blocks = lib.somi_linear_big_stats_blocks(m, n, int(tile))
+    stats = torch.empty((blocks, _stats_width(m)), dtype=torch.float32, device=x.device)
+    weighted = None
+    if next_norm_weight is not None:
+        _need(next_norm_weight, "norm weight", torch.float32, (n,))
+        weighted = torch.empty((m, n), dtype=torch.bfloat16, device=x.device)
+    _check(lib.somi_linear_big_residual(_ptr(x), ctypes.c_int64(x.stride(0)), _ptr(weight), ctypes.c_int64(weight.stride(0)),
+                                        _ptr(bias), _ptr(h), _ptr(next_norm_weight), _ptr(weighted), _ptr(stats),
+                                        stats.shape[1], m, n, k, int(tile), _stream()))
+    return stats, weighted
+
+
 def linear_residual(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, h: torch.Tensor,
                     next_norm_weight: torch.Tensor | None = None, mid: bool = False
                     ) -> tuple[torch.Tensor, torch.Tensor | None]:

@@ -107,7 +107,7 @@ class GroupedQueryAttention(Mixer):
         inv_freq, rotary_dim = rotation
         rows = x.shape[0]
         if (rotary_dim != self.head_dim or self.head_dim % 32 or cache.k.dtype != torch.bfloat16
-                or not self.qkv.fusable(rows)):
+                or rows > ops.FUSED_MAX_ROWS or not self.qkv.fusable(rows)):
             return None
         if isinstance(x, NormedRows):
             weighted, eps, stats = x.weighted, x.norm.eps, x.stats

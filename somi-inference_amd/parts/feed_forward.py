@@ -55,6 +55,6 @@ class SwiGLU(FeedForward):
             x = x.materialize()
         if not self.interleaved:
             return self.down.deferred(ops.silu_mul(self.gate_up(x)))
-        if x.shape[0] <= linear_kernels.SKINNY_ROWS and x.data_ptr() % 16 == 0:
+        if x.data_ptr() % 16 == 0:
             return self.down.deferred(linear_kernels.linear_swiglu(x, self.gate_up.weight))
         return self.down.deferred(ops.silu_mul(self.gate_up(x), block=self.INTERLEAVE))

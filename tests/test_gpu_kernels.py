@@ -593,3 +593,96 @@ def test_qkv_product_with_the_rotation_and_the_cache_store(m, nq, nkv, d, hidden
 
 def plain_rms(h, w, eps):
     return w * h * torch.rsqrt(h.pow(2).mean(dim=-1, keepdim=True) + eps)
+
+
+# ------------------------------------------------------------------------------ the many-rows product
+BIG_SHAPES = [(65, 130, 64), (128, 256, 192), (300, 520, 200), (512, 96, 72), (2048, 264, 1032), (257, 384, 8)]
+
+
+def _interleave16(gate, up):
+    b, h = 16, gate.shape[1]
+    return torch.stack([gate.view(-1, b, h), up.view(-1, b, h)], dim=1).reshape(-1, h).contiguous()
+
+
+@pytest.mark.parametrize("tile", [0, 128, 256])
+@pytest.mark.parametrize("m,n,k", BIG_SHAPES)
+def test_many_rows_product_plain_with_bias_and_row_scale(m, n, k, tile):
+    """x . w^T (+ bias) against F.linear in float32, with tails in M, N and K (K = 200 and 72 end inside a stage,
+    K = 8 is one piece), for both tile widths; then the same with the rows scaled as an RMS norm would."""
+    x, w, bias = rnd(m, k, dtype="bfloat16", seed=1), rnd(n, k, dtype="bfloat16", seed=2, scale=0.3), rnd(n, seed=3)
+    want = F.linear(x.float(), w.float(), bias)
+    got = ops.linear_big(x, w, bias, tile=tile)
+    assert got.dtype == torch.bfloat16
+    torch.testing.assert_close(got.float(), want, atol=0.02 * float(want.abs().max()), rtol=2e-2)
+    plain = ops.linear_big(x, w, tile=tile)
+    torch.testing.assert_close(plain.float(), F.linear(x.float(), w.float()), atol=0.02 * float(want.abs().max()), rtol=2e-2)
+    # row statistics in 3 partial sums, wider than M as the producers make them
+    eps = 1e-5
+    width = 16 * ((m + 15) // 16)
+    stats = torch.zeros(3, width, device=DEV)
+    stats[:, :m] = torch.rand(3, m, device=DEV) * k
+    scale = torch.rsqrt(stats[:, :m].sum(0) / k + eps)
+    scaled = ops.linear_big(x, w, bias, eps=eps, stats=stats, tile=tile)
+    want_scaled = scale[:, None] * F.linear(x.float(), w.float()) + bias
+    torch.testing.assert_close(scaled.float(), want_scaled, atol=0.02 * float(want_scaled.abs().max()), rtol=2e-2)
+
+
+def test_many_rows_product_reads_strided_rows_and_refuses_what_it_cannot_take():
+    wide = rnd(300, 256 + 64, dtype="bfloat16", seed=4)
+    x = wide[:, :256]                                # a view: rows 320 elements apart
+    w = rnd(200, 256, dtype="bfloat16", seed=5, scale=0.2)
+    torch.testing.assert_close(ops.linear_big(x, w).float(), F.linear(x.float(), w.float()), atol=0.1, rtol=2e-2)
+    with pytest.raises(KernelError, match="multiples of 8"):
+        ops.linear_big(rnd(70, 36, dtype="bfloat16"), rnd(8, 36, dtype="bfloat16"))
+    with pytest.raises(KernelError, match="features"):
+        ops.linear_big(rnd(70, 64, dtype="bfloat16"), rnd(8, 32, dtype="bfloat16"))
+    with pytest.raises(KernelError, match="bfloat16"):
+        ops.linear_big(rnd(70, 64), rnd(8, 64))
+    with pytest.raises(KernelError, match="tile width"):
+        ops.linear_big(rnd(70, 64, dtype="bfloat16"), rnd(8, 64, dtype="bfloat16"), tile=64)
+
+
+@pytest.mark.parametrize("tile", [128, 256])
+@pytest.mark.parametrize("m,inter,k", [(65, 16, 64), (130, 272, 200), (512, 1040, 192), (2048, 48, 72)])
+def test_many_rows_product_with_the_gate_in_its_end(m, inter, k, tile):
+    x = rnd(m, k, dtype="bfloat16", seed=6)
+    gate, up = rnd(inter, k, dtype="bfloat16", seed=7, scale=0.2), rnd(inter, k, dtype="bfloat16", seed=8, scale=0.2)
+    want = F.silu(x.float() @ gate.float().t()) * (x.float() @ up.float().t())
+    got = ops.linear_big(x, _interleave16(gate, up), swiglu=True, tile=tile)
+    assert got.shape == (m, inter)
+    torch.testing.assert_close(got.float(), want, atol=0.02 * float(want.abs().max()), rtol=2e-2)
+    eps, width = 1e-6, 16 * ((m + 15) // 16)
+    stats = torch.zeros(2, width, device=DEV)
+    stats[:, :m] = torch.rand(2, m, device=DEV) * k * 4
+    s = torch.rsqrt(stats[:, :m].sum(0) / k + eps)[:, None]
+    want = F.silu(s * (x.float() @ gate.float().t())) * (s * (x.float() @ up.float().t()))
+    got = ops.linear_big(x, _interleave16(gate, up), swiglu=True, eps=eps, stats=stats, tile=tile)
+    torch.testing.assert_close(got.float(), want, atol=0.02 * float(want.abs().max()) + 1e-3, rtol=2e-2)
+
+
+@pytest.mark.parametrize("tile", [0, 128, 256])
+@pytest.mark.parametrize("m,n,k", [(65, 132, 64), (300, 520, 200), (1024, 72, 1032), (257, 256, 136)])
+def test_many_rows_product_into_the_residual_stream(m, n, k, tile):
+    """h += x . w^T + bias in float32, with the next norm's weighted rows and the rows' sums of squares; feeding
+    those into the scaled product gives the product of the normed rows."""
+    x, w, bias = rnd(m, k, dtype="bfloat16", seed=9), rnd(n, k, dtype="bfloat16", seed=10, scale=0.2), rnd(n, seed=11)
+    h0 = rnd(m, n, seed=12)
+    norm_w = rnd(n, seed=13).abs() + 0.5
+    want_h = h0 + F.linear(x.float(), w.float(), bias)
+    h = h0.clone()
+    stats, weighted = ops.linear_big_residual(x, w, bias, h, norm_w, tile=tile)
+    torch.testing.assert_close(h, want_h, atol=2e-4 * float(want_h.abs().max()) + 1e-4, rtol=1e-4)
+    torch.testing.assert_close(weighted.float(), norm_w * want_h, atol=0.01 * float((norm_w * want_h).abs().max()), rtol=1e-2)
+    torch.testing.assert_close(stats[:, :m].sum(0), want_h.pow(2).sum(1), rtol=1e-4, atol=1e-3)
+    plain_h = h0.clone()
+    none_stats, none_weighted = ops.linear_big_residual(x, w, None, plain_h, tile=tile)
+    assert none_weighted is None
+    torch.testing.assert_close(plain_h, h0 + F.linear(x.float(), w.float()), atol=2e-4 * float(want_h.abs().max()) + 1e-4, rtol=1e-4)
+    # the next product, of the normed rows: norm(h) . w2^T
+    eps = 1e-5
+    w2 = rnd(96, n, dtype="bfloat16", seed=14, scale=0.2)
+    if n % 8 == 0:
+        got = ops.linear_big(weighted, w2, eps=eps, stats=stats)
+        normed = norm_w * want_h * torch.rsqrt(want_h.pow(2).mean(1, keepdim=True) + eps)
+        want = normed @ w2.float().t()
+        torch.testing.assert_close(got.float(), want, atol=0.02 * float(want.abs().max()), rtol=2e-2)
