@@ -58,8 +58,6 @@ def parse_args() -> argparse.Namespace:
     p.add_argument("--serving", type=int, default=0, metavar="REQUESTS",
                    help="also run this many requests (prompts of 128 to 2,048 tokens, 256 new tokens each) through "
                         "the scheduler with portions of 512, and report it under 'serving'")
-    p.add_argument("--no-tune", action="store_true",
-                   help="leave the library's matrix products of the prompt portions at its own heuristic")
     return p.parse_args()
 
 
@@ -94,8 +92,6 @@ def main() -> int:
     runner = make_runner(model, block_size=args.block_size, num_blocks=num_blocks, max_requests=max(batches) + 1)
     sampler, greedy = Sampler(), SamplingParams(temperature=0.0)
     gen = torch.Generator().manual_seed(args.seed)
-    # untimed warm-up, as LLM.warm_up() does it: the library times its solutions for a full prompt portion
-    tuned = 0 if args.no_tune or args.dtype != "bfloat16" else runner.tune_library_products(args.prefill_tokens)
 
     weight_bytes = sum(t.numel() * t.element_size() for t in _decode_weights(model))
     kv_bytes_per_token = 2 * config.num_key_value_heads * config.head_dim * elem * layers
@@ -186,8 +182,6 @@ def main() -> int:
         engine = Engine(runner, scheduler, sampler, eos_token_id=-1)
         arrivals = deque((0, Request(f"s{i}", torch.randint(0, config.vocab_size, (n,), generator=gen).tolist(),
                                      new_tokens, greedy, seed=i)) for i, n in enumerate(lengths))
-        if tuned:
-            runner.tune_library_products(512)
         # as LLM.warm_up() does it: the decode graphs that the requests will replay are captured before they arrive
         captured = runner.capture_decode_graphs(concurrent, 2048 + new_tokens)
         sync()
@@ -216,7 +210,7 @@ def main() -> int:
                    "intermediate_size": config.intermediate_size, "num_attention_heads": config.num_attention_heads,
                    "num_key_value_heads": config.num_key_value_heads, "head_dim": config.head_dim,
                    "vocab_size": config.vocab_size, "tie_word_embeddings": tied, "block_size": args.block_size,
-                   "context_at_end": args.context, "library_gemm_tuned": tuned > 0},
+                   "context_at_end": args.context},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4)},
         "points": {f"decode_b{b}": round(r["tok_s"], 2) for b, r in results.items() if b in (1, 64)},

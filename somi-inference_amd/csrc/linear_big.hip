@@ -65,14 +65,13 @@ struct BigArgs {
     int tiles_m, tiles_n;
     // plain / swiglu
     bf16* out;                        // [M, N] or [M, N / 2]
-    const float* stats_in;            // [stats_blocks][stats_width] partial sums of squares of the rows, or null
-    int stats_blocks, stats_width;
-    float eps;
+    const float* row_scale;           // [M] the rows' scales s, or null
     // residual
     float* h;                         // [M, N] float32, in and out
     const float* norm_w;              // [N] or null
     bf16* weighted;                   // [M, N] = bfloat16(norm_w * h) or null
     float* stats_out;                 // [tiles_n * waves along n][stats_width] or null
+    int stats_width;
 };
 
 template <int N> __device__ __forceinline__ void big_wait_vmcnt() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
@@ -81,6 +80,12 @@ template <int N> __device__ __forceinline__ void big_wait_vmcnt() { asm volatile
 // precedes its first use (so that no use can be moved before the wait).
 #define BIG_DS_READ(dst, addr, off) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(off))
 
+// S: 3 = a ring of three whole stages (narrow tile); 5 = five slots of 32 KB that hold one operand's stage each
+// (wide tile), filled in the order A0 B0 A1 B1 A2 ...: piece q goes to slot q % 5.  While stage kt is computed,
+// both pieces of stage kt + 1 and A of kt + 2 are in the ring or on their way; the barrier that ends the reads of
+// stage kt frees two slots, which take B of kt + 2 and A of kt + 3.
+// The wide form is persistent: a workgroup walks its die's tiles 32 apart, and the first pieces of the next
+// tile are asked for before the finished tile is stored, so the stores and the first loads overlap.
 template <int BN, int S, int NW, int EPI, bool KTAIL>
 __global__ void __launch_bounds__(NW * 64, 1)
 linear_big_kernel(const BigArgs p) {
@@ -92,80 +97,82 @@ linear_big_kernel(const BigArgs p) {
     static_assert(BM / 2 == WTM * 32 && BN / WAVES_N == WTN * 32, "a wavefront owns 128 x 64 of the tile");
     constexpr int LA = BM / 8 / NW, LB = BN / 8 / NW, L = LA + LB;  // direct loads a lane issues per stage (8 rows each)
     constexpr int KK = BK / 16, NM = WTM * WTN, NF = WTM + WTN;
-    constexpr bool TWO = S == 2;
-    static_assert(TWO || L % KK == 0, "loads divisible over the sub-steps");
-    constexpr int LPS = TWO ? 0 : L / KK;
-    constexpr int AHEAD = TWO ? 2 : S - 1;                        // stages issued before the loop
+    constexpr bool HALF = S == 5;
+    static_assert(HALF || (S == 3 && L % KK == 0), "three whole stages, loads divisible over the sub-steps");
+    static_assert(!HALF || (LA == LB && BN == 256), "halves of equal size");
+    constexpr int LPS = HALF ? 0 : L / KK;
+    constexpr int HB = 256 * ROW_BYTES;                           // bytes of a slot of the wide ring
+    constexpr int STG = HALF ? 3 * HB : 0;                        // where the epilogue stages: slots 3 and 4, or the ring
+    constexpr int STG_WAVE = 8192;
+    constexpr int SYNC_AFTER = 2;                                 // products of the last sub-step issued before the barrier
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave / WAVES_N, wn = wave % WAVES_N;
     const int M = p.M, N = p.N, K = p.K;
-
-    const int total = p.tiles_m * p.tiles_n, per = (total + 7) / 8;
-    const int logical = (blockIdx.x & 7) * per + (blockIdx.x >> 3);
-    if (logical >= total) return;
-    const int tn = logical / p.tiles_m, tm = logical % p.tiles_m;
-    const int m0 = tm * BM, n0 = tn * BN;
-    const char* xa = (const char*)(p.x + (int64_t)m0 * p.ldx);
-    const char* wb = (const char*)(p.w + (int64_t)n0 * p.ldw);
-    const int mlim = M - m0, nlim = N - n0;
     const int KT = (K + BK - 1) / BK;
+    const int lrow = lane >> 3, lpos = lane & 7;
+    const int frow = lane & 31, fk = lane >> 5;
+    const int ml = lane & 31, nh = lane >> 5;
+
+    // tiles of this workgroup: the die (blockIdx % 8) owns a contiguous range of tiles with the row tiles of a
+    // column tile next to each other; its workgroups take them 32 (wide, persistent) apart, or one each
+    const int total = p.tiles_m * p.tiles_n, per = (total + 7) / 8;
+    const int die_first = (blockIdx.x & 7) * per, die_end = die_first + per < total ? die_first + per : total;
+    const int stride = HALF ? (int)(gridDim.x >> 3) : per;
+    int logical = die_first + (blockIdx.x >> 3);
+    if (logical >= die_end) return;
 
     // ------------------------------------------------------------------ loads: global -> LDS
     // An instruction covers 8 rows of 128 bytes; lane l writes LDS position l % 8 of row l / 8 and reads the
     // global piece that belongs there.  Rows past the matrix repeat its last row (never stored).
-    const int lrow = lane >> 3, lpos = lane & 7;
+    const char *xa, *wb;                       // first rows of the tile being loaded
     uint32_t offa[LA], offb[LB];
     int piece_a[LA], piece_b[LB];
 #pragma unroll
-    for (int i = 0; i < LA; ++i) {
-        const int row = (wave * LA + i) * 8 + lrow;
-        piece_a[i] = lpos ^ ((row >> 1) & 7);
-        offa[i] = (uint32_t)(row < mlim ? row : mlim - 1) * (uint32_t)p.ldx * 2u + (piece_a[i] << 4);
-    }
+    for (int i = 0; i < LA; ++i) piece_a[i] = lpos ^ ((((wave * LA + i) * 8 + lrow) >> 1) & 7);
 #pragma unroll
-    for (int i = 0; i < LB; ++i) {
-        const int row = (wave * LB + i) * 8 + lrow;
-        piece_b[i] = lpos ^ ((row >> 1) & 7);
-        offb[i] = (uint32_t)(row < nlim ? row : nlim - 1) * (uint32_t)p.ldw * 2u + (piece_b[i] << 4);
-    }
-    auto issue_load = [&](int kt, int buf, int i) {
-        const char* src;
-        char* dst;
-        int piece;
-        if (i < LA) {
-            src = xa + (int64_t)kt * ROW_BYTES + offa[i];
-            dst = lds + buf * STAGE + (wave * LA + i) * 1024;
-            piece = piece_a[i];
-        } else {
-            src = wb + (int64_t)kt * ROW_BYTES + offb[i - LA];
-            dst = lds + buf * STAGE + A_BYTES + (wave * LB + i - LA) * 1024;
-            piece = piece_b[i - LA];
+    for (int i = 0; i < LB; ++i) piece_b[i] = lpos ^ ((((wave * LB + i) * 8 + lrow) >> 1) & 7);
+    auto aim = [&](int tile) {                 // point the loads at a tile
+        const int tn = tile / p.tiles_m, tm = tile % p.tiles_m;
+        const int mlim = M - tm * BM, nlim = N - tn * BN;
+        xa = (const char*)(p.x + (int64_t)tm * BM * p.ldx);
+        wb = (const char*)(p.w + (int64_t)tn * BN * p.ldw);
+#pragma unroll
+        for (int i = 0; i < LA; ++i) {
+            const int row = (wave * LA + i) * 8 + lrow;
+            offa[i] = (uint32_t)(row < mlim ? row : mlim - 1) * (uint32_t)p.ldx * 2u + (piece_a[i] << 4);
         }
+#pragma unroll
+        for (int i = 0; i < LB; ++i) {
+            const int row = (wave * LB + i) * 8 + lrow;
+            offb[i] = (uint32_t)(row < nlim ? row : nlim - 1) * (uint32_t)p.ldw * 2u + (piece_b[i] << 4);
+        }
+    };
+    // load i of operand A (is_b false) or B of stage kt into LDS at byte offset `at`; a stage past the end repeats
+    // the last one (it lands in a slot that is never read again)
+    auto issue = [&](bool is_b, int kt, int at, int i) {
+        kt = kt < KT ? kt : KT - 1;
+        const char* src = (is_b ? wb + offb[i] : xa + offa[i]) + (int64_t)kt * ROW_BYTES;
         if (KTAIL) {
-            if (kt * BK + piece * 8 >= K) src = (const char*)big_zero_piece;
+            if (kt * BK + (is_b ? piece_b[i] : piece_a[i]) * 8 >= K) src = (const char*)big_zero_piece;
         }
+        char* dst = lds + at + (wave * (is_b ? LB : LA) + i) * 1024;
         __builtin_amdgcn_global_load_lds((const BIG_GLOBAL void*)src, (BIG_LDS void*)dst, 16, 0, 0);
     };
-
-    f32x16 acc[WTM][WTN];
-#pragma unroll
-    for (int i = 0; i < WTM; ++i)
-#pragma unroll
-        for (int j = 0; j < WTN; ++j)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+    auto issue_piece = [&](int q, int slot, int i) { issue(q & 1, q >> 1, slot * HB, i); };                 // wide ring
+    auto issue_stage = [&](int kt, int buf, int i) {                                                       // narrow ring
+        if (i < LA) issue(false, kt, buf * STAGE, i); else issue(true, kt, buf * STAGE + A_BYTES, i - LA);
+    };
 
     // ------------------------------------------------------------------ fragments: LDS -> registers
-    const int frow = lane & 31, fk = lane >> 5;
     const uint32_t lds_base = (uint32_t)(uintptr_t)(BIG_LDS char*)lds;
-    uint32_t foffa[KK], foffb[KK];
+    uint32_t foffa[KK], foffb[KK];              // relative to the start of the operand's stage
 #pragma unroll
     for (int kk = 0; kk < KK; ++kk) {
         const uint32_t f = frow * ROW_BYTES + (((kk * 2 + fk) ^ ((frow >> 1) & 7)) << 4);
         foffa[kk] = lds_base + f + wm * (BM / 2) * ROW_BYTES;
-        foffb[kk] = lds_base + f + A_BYTES + wn * (BN / WAVES_N) * ROW_BYTES;
+        foffb[kk] = lds_base + f + wn * (BN / WAVES_N) * ROW_BYTES;
     }
     // read q of a set, in the order the products need them: a[0], every b, then the other a
     auto read_one = [&](bf16x8 (&a)[WTM], bf16x8 (&b)[WTN], uint32_t aa, uint32_t ab, int q) {
@@ -179,214 +186,298 @@ linear_big_kernel(const BigArgs p) {
     auto wait_frags = [&](bf16x8 (&a)[WTM], bf16x8 (&b)[WTN]) {
         asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(b[0]), "+v"(b[1]));
     };
-    auto product = [&](bf16x8 (&a)[WTM], bf16x8 (&b)[WTN], int q) {
-        const int i = q / WTN, j = q % WTN;
-        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b[j], a[i], acc[i][j], 0, 0, 0);    // D[n][m]
-    };
 
-    // ------------------------------------------------------------------ the ring
-    // Three stages or more: the slot freed one iteration ago is refilled evenly over the sub-steps.  Two: the
-    // stage just read is refilled in a burst after the barrier.
+    // the first tile's first pieces
+    aim(logical);
+    if (HALF) {
 #pragma unroll
-    for (int st = 0; st < AHEAD; ++st)
+        for (int q = 0; q < 5; ++q)
 #pragma unroll
-        for (int i = 0; i < L; ++i) issue_load(st < KT ? st : KT - 1, st, i);
-    big_wait_vmcnt<(AHEAD - 1) * L>();
-    __syncthreads();
-
-    bf16x8 a0[WTM], b0[WTN], a1[WTM], b1[WTN];
-#pragma unroll
-    for (int q = 0; q < NF; ++q) read_one(a0, b0, foffa[0], foffb[0], q);
-    int buf = 0, rbuf = TWO ? 0 : S - 1;    // the stage computed on; the slot being refilled
-    constexpr int SYNC_AFTER = 2;           // products of the last sub-step issued before the barrier
-    for (int kt = 0; kt < KT; ++kt) {
-        const int nbuf = buf + 1 == S ? 0 : buf + 1;
-        const int rstage = kt + AHEAD < KT ? kt + AHEAD : KT - 1;      // past the end: a harmless repeat
-        if (TWO) rbuf = buf;
-        BIG_FENCE();
-#pragma unroll
-        for (int kk = 0; kk < KK; ++kk) {
-            const bool last = kk == KK - 1;
-            const uint32_t aa = (last ? foffa[0] + nbuf * STAGE : foffa[kk + 1 < KK ? kk + 1 : 0] + buf * STAGE);
-            const uint32_t ab = (last ? foffb[0] + nbuf * STAGE : foffb[kk + 1 < KK ? kk + 1 : 0] + buf * STAGE);
-            BIG_FENCE();
-            if (kk & 1) wait_frags(a1, b1); else wait_frags(a0, b0);
-            BIG_FENCE();
-            int reads = 0, loads = 0;
-            constexpr int PER_SLOT = TWO ? (L + NF - 1) / NF : 1;
-#pragma unroll
-            for (int q = 0; q < NM; ++q) {
-                if (last && q == SYNC_AFTER) {
-                    // the next stage has landed and everybody has read this one
-                    big_wait_vmcnt<TWO ? 0 : (S - 3) * L + LPS * (KK - 1)>();
-                    __builtin_amdgcn_s_barrier();
-                    BIG_FENCE();
-                }
-                if (kk & 1) product(a1, b1, q); else product(a0, b0, q);
-                BIG_FENCE();
-                if ((!last || q >= SYNC_AFTER) && reads < NF) {
-                    if (kk & 1) read_one(a0, b0, aa, ab, reads); else read_one(a1, b1, aa, ab, reads);
-                    ++reads;
-                    if (TWO) {
-                        if (last)
-#pragma unroll
-                            for (int e = 0; e < PER_SLOT; ++e)
-                                if (loads < L) { issue_load(rstage, rbuf, loads); ++loads; }
-                    } else if (loads < LPS) { issue_load(rstage, rbuf, kk * LPS + loads); ++loads; }
-                    BIG_FENCE();
-                }
-            }
-        }
-        if (!TWO) rbuf = buf;
-        buf = nbuf;
-    }
-    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
-    __syncthreads();                       // the ring is free: its memory serves the epilogue
-
-    // ------------------------------------------------------------------ epilogue
-    // A product holds D[n][m]: lane l has row m = l % 32 and, in registers 4 g .. 4 g + 3, the columns
-    // 8 g + 4 (l / 32) + 0..3 of its 32.  A wavefront turns 32 rows at a time through its own 16 KB of LDS
-    // into whole rows and stores 16 bytes a lane.
-    char* stg = lds + wave * 16384;
-    const int ml = lane & 31, nh = lane >> 5;
-    const int wave_n0 = n0 + wn * (BN / WAVES_N);            // first column of the wavefront
-
-    // the row scale of the norm whose rows x holds (plain and swiglu)
-    float scale[WTM];
-#pragma unroll
-    for (int i = 0; i < WTM; ++i) scale[i] = 1.f;
-    if (EPI != BIG_RESIDUAL && p.stats_in != nullptr) {
-#pragma unroll
-        for (int i = 0; i < WTM; ++i) {
-            const int gm = m0 + wm * (BM / 2) + i * 32 + ml;
-            float sum = 0.f;
-            if (gm < M)
-                for (int b = 0; b < p.stats_blocks; ++b) sum += p.stats_in[(int64_t)b * p.stats_width + gm];
-            scale[i] = rsqrtf(sum / (float)K + p.eps);
-        }
-    }
-
-    if (EPI == BIG_PLAIN || EPI == BIG_SWIGLU) {
-        constexpr int CW = EPI == BIG_SWIGLU ? WTN * 16 : WTN * 32;      // output columns of the wavefront per row
-        constexpr int SROW = CW * 2 + 8;                                   // staged row: 8 bytes of padding spread the banks
-        constexpr int LPR = CW * 2 / 16;                                   // lanes per row when reading back
-        const int out_n = EPI == BIG_SWIGLU ? N / 2 : N;
-        const int out_c0 = EPI == BIG_SWIGLU ? wave_n0 / 2 : wave_n0;
-        const bool aligned = (out_n & 7) == 0 && ((uintptr_t)p.out & 15) == 0;
-#pragma unroll
-        for (int i = 0; i < WTM; ++i) {
-            const float s = scale[i];
-#pragma unroll
-            for (int j = 0; j < WTN; ++j) {
-                const f32x16& t = acc[i][j];
-                if (EPI == BIG_SWIGLU) {
-                    // registers r and r + 8 are gate and up of one channel (columns 16 apart)
-#pragma unroll
-                    for (int g = 0; g < 2; ++g) {
-                        bf16x4 v;
-#pragma unroll
-                        for (int c = 0; c < 4; ++c) {
-                            const float gate = s * t[4 * g + c], up = s * t[4 * g + c + 8];
-                            v[c] = (bf16)(gate / (1.f + expf(-gate)) * up);
-                        }
-                        *(bf16x4*)(stg + ml * SROW + (j * 16 + 8 * g + 4 * nh) * 2) = v;
-                    }
-                } else {
-#pragma unroll
-                    for (int g = 0; g < 4; ++g) {
-                        bf16x4 v;
-#pragma unroll
-                        for (int c = 0; c < 4; ++c) {
-                            float val = s * t[4 * g + c];
-                            if (p.bias != nullptr) {
-                                const int gn = wave_n0 + j * 32 + 8 * g + 4 * nh + c;
-                                val += p.bias[gn < N ? gn : N - 1];
-                            }
-                            v[c] = (bf16)val;
-                        }
-                        *(bf16x4*)(stg + ml * SROW + (j * 32 + 8 * g + 4 * nh) * 2) = v;
-                    }
-                }
-            }
-            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-#pragma unroll
-            for (int pass = 0; pass < 32 * LPR / 64; ++pass) {
-                const int row = pass * (64 / LPR) + lane / LPR, piece = lane % LPR;
-                const u32x4 v = *(const u32x4*)(stg + row * SROW + piece * 16);
-                const int gm = m0 + wm * (BM / 2) + i * 32 + row;
-                const int gc = out_c0 + piece * 8;
-                if (gm < M) {
-                    bf16* dst = p.out + (int64_t)gm * out_n + gc;
-                    if (aligned && gc + 8 <= out_n) *(u32x4*)dst = v;
-                    else {
-                        const bf16* e = (const bf16*)&v;
-                        for (int c = 0; c < 8; ++c)
-                            if (gc + c < out_n) dst[c] = e[c];
-                    }
-                }
-            }
-            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        }
+            for (int i = 0; i < LA; ++i) issue_piece(q, q, i);
     } else {
-        // h += product (+ bias), 32 rows x 64 columns of float32 at a time; a row is read back by 16 lanes
-        constexpr int CW = WTN * 32;
-        constexpr int SROW = CW * 4 + 16;
-        const bool aligned = (N & 3) == 0 && ((uintptr_t)p.h & 15) == 0 &&
-                             (p.weighted == nullptr || ((uintptr_t)p.weighted & 7) == 0);
-        const int stats_row0 = (tn * WAVES_N + wn);
 #pragma unroll
-        for (int i = 0; i < WTM; ++i) {
+        for (int st = 0; st < S - 1; ++st)
+#pragma unroll
+            for (int i = 0; i < L; ++i) issue_stage(st, st, i);
+    }
+
+    while (true) {
+        const int tn = logical / p.tiles_m, tm = logical % p.tiles_m;
+        const int m0 = tm * BM, n0 = tn * BN;
+        const int next = logical + stride;
+        const bool has_next = HALF && next < die_end;
+
+        f32x16 acc[WTM][WTN];
+#pragma unroll
+        for (int i = 0; i < WTM; ++i)
 #pragma unroll
             for (int j = 0; j < WTN; ++j)
 #pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                    const f32x16& t = acc[i][j];
-                    f32x4 v = {t[4 * g], t[4 * g + 1], t[4 * g + 2], t[4 * g + 3]};
-                    *(f32x4*)(stg + ml * SROW + (j * 32 + 8 * g + 4 * nh) * 4) = v;
-                }
-            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+        auto product = [&](bf16x8 (&a)[WTM], bf16x8 (&b)[WTN], int q) {
+            const int i = q / WTN, j = q % WTN;
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b[j], a[i], acc[i][j], 0, 0, 0);    // D[n][m]
+        };
+        bf16x8 a0[WTM], b0[WTN], a1[WTM], b1[WTN];
+
+        // ---------------------------------------------------------------- the loop over K
+        if constexpr (HALF) {
+            big_wait_vmcnt<3 * LA>();          // pieces 0 and 1 have landed
+            __syncthreads();
 #pragma unroll
-            for (int pass = 0; pass < 8; ++pass) {
-                const int row = pass * 4 + (lane >> 4), piece = lane & 15;
-                f32x4 v = *(const f32x4*)(stg + row * SROW + piece * 16);
-                const int gm = m0 + wm * (BM / 2) + i * 32 + row;
-                const int gn = wave_n0 + piece * 4;
-                float sq = 0.f;
-                if (gm < M && gn < N) {
-                    float* hp = p.h + (int64_t)gm * N + gn;
-                    if (aligned && gn + 4 <= N) {
-                        f32x4 hv = *(const f32x4*)hp;
+            for (int q = 0; q < NF; ++q) read_one(a0, b0, foffa[0], foffb[0] + HB, q);
+            int sa = 0, sb = 1;                // slots of the stage computed on
+            for (int kt = 0; kt < KT; ++kt) {
+                const int na = sa + 2 >= 5 ? sa - 3 : sa + 2, nb = sb + 2 >= 5 ? sb - 3 : sb + 2;     // slots of the next stage
+                BIG_FENCE();
 #pragma unroll
-                        for (int c = 0; c < 4; ++c) {
-                            hv[c] += v[c] + (p.bias != nullptr ? p.bias[gn + c] : 0.f);
-                            sq += hv[c] * hv[c];
+                for (int kk = 0; kk < KK; ++kk) {
+                    const bool last = kk == KK - 1;
+                    const uint32_t aa = last ? foffa[0] + na * HB : foffa[kk + 1 < KK ? kk + 1 : 0] + sa * HB;
+                    const uint32_t ab = last ? foffb[0] + nb * HB : foffb[kk + 1 < KK ? kk + 1 : 0] + sb * HB;
+                    BIG_FENCE();
+                    if (kk & 1) wait_frags(a1, b1); else wait_frags(a0, b0);
+                    BIG_FENCE();
+                    int reads = 0, loads = 0;
+#pragma unroll
+                    for (int q = 0; q < NM; ++q) {
+                        if (last && q == SYNC_AFTER) {
+                            // stage kt + 1 has landed (only A of kt + 2 may still be on its way); everybody has read stage kt
+                            big_wait_vmcnt<LA>();
+                            __builtin_amdgcn_s_barrier();
+                            BIG_FENCE();
                         }
-                        *(f32x4*)hp = hv;
-                        if (p.weighted != nullptr) {
-                            bf16x4 wv;
+                        if (kk & 1) product(a1, b1, q); else product(a0, b0, q);
+                        BIG_FENCE();
+                        if ((!last || q >= SYNC_AFTER) && reads < NF) {
+                            if (kk & 1) read_one(a0, b0, aa, ab, reads); else read_one(a1, b1, aa, ab, reads);
+                            ++reads;
+                            if (last) {
+                                // B of stage kt + 2 into the slot A of kt had, then A of kt + 3 into the slot B of kt had
 #pragma unroll
-                            for (int c = 0; c < 4; ++c) wv[c] = (bf16)(p.norm_w[gn + c] * hv[c]);
-                            *(bf16x4*)(p.weighted + (int64_t)gm * N + gn) = wv;
-                        }
-                    } else {
-                        for (int c = 0; c < 4; ++c)
-                            if (gn + c < N) {
-                                const float hv = hp[c] + v[c] + (p.bias != nullptr ? p.bias[gn + c] : 0.f);
-                                hp[c] = hv;
-                                sq += hv * hv;
-                                if (p.weighted != nullptr) p.weighted[(int64_t)gm * N + gn + c] = (bf16)(p.norm_w[gn + c] * hv);
+                                for (int e = 0; e < 2; ++e)
+                                    if (loads < 2 * LA) {
+                                        if (loads < LA) issue_piece(2 * kt + 5, sa, loads);
+                                        else issue_piece(2 * kt + 6, sb, loads - LA);
+                                        ++loads;
+                                    }
                             }
+                            BIG_FENCE();
+                        }
                     }
                 }
-                if (p.stats_out != nullptr) {
-                    // the 16 lanes of a row add their squares in a fixed order
+                sa = na;
+                sb = nb;
+            }
+        } else {
+            // three whole stages: the slot freed one iteration ago is refilled evenly over the sub-steps
+            big_wait_vmcnt<(S - 2) * L>();
+            __syncthreads();
 #pragma unroll
-                    for (int off = 8; off > 0; off >>= 1) sq += __shfl_xor(sq, off, 64);
-                    if (piece == 0 && gm < M) p.stats_out[(int64_t)stats_row0 * p.stats_width + gm] = sq;
+            for (int q = 0; q < NF; ++q) read_one(a0, b0, foffa[0], foffb[0] + A_BYTES, q);
+            int buf = 0, rbuf = S - 1;          // the stage computed on; the slot being refilled
+            for (int kt = 0; kt < KT; ++kt) {
+                const int nbuf = buf + 1 == S ? 0 : buf + 1;
+                BIG_FENCE();
+#pragma unroll
+                for (int kk = 0; kk < KK; ++kk) {
+                    const bool last = kk == KK - 1;
+                    const uint32_t aa = last ? foffa[0] + nbuf * STAGE : foffa[kk + 1 < KK ? kk + 1 : 0] + buf * STAGE;
+                    const uint32_t ab = (last ? foffb[0] + nbuf * STAGE : foffb[kk + 1 < KK ? kk + 1 : 0] + buf * STAGE) + A_BYTES;
+                    BIG_FENCE();
+                    if (kk & 1) wait_frags(a1, b1); else wait_frags(a0, b0);
+                    BIG_FENCE();
+                    int reads = 0, loads = 0;
+#pragma unroll
+                    for (int q = 0; q < NM; ++q) {
+                        if (last && q == SYNC_AFTER) {
+                            // the next stage has landed and everybody has read this one
+                            big_wait_vmcnt<(S - 3) * L + LPS * (KK - 1)>();
+                            __builtin_amdgcn_s_barrier();
+                            BIG_FENCE();
+                        }
+                        if (kk & 1) product(a1, b1, q); else product(a0, b0, q);
+                        BIG_FENCE();
+                        if ((!last || q >= SYNC_AFTER) && reads < NF) {
+                            if (kk & 1) read_one(a0, b0, aa, ab, reads); else read_one(a1, b1, aa, ab, reads);
+                            ++reads;
+                            if (loads < LPS) { issue_stage(kt + S - 1, rbuf, kk * LPS + loads); ++loads; }
+                            BIG_FENCE();
+                        }
+                    }
+                }
+                rbuf = buf;
+                buf = nbuf;
+            }
+        }
+        // every load of this tile has landed, every wavefront is done with the ring
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+        __syncthreads();
+        // what the epilogue reads beside the sums, asked for before the next tile's loads: loads return in order,
+        // so these must not queue behind them
+        const int wave_n0 = n0 + wn * (BN / WAVES_N);            // first column of the wavefront
+        float scale[WTM];
+        float bv[WTN][EPI == BIG_PLAIN ? 16 : 1];
+        if (EPI != BIG_RESIDUAL) {
+#pragma unroll
+            for (int i = 0; i < WTM; ++i) {
+                const int sm = m0 + wm * (BM / 2) + i * 32 + ml;
+                scale[i] = p.row_scale != nullptr ? p.row_scale[sm < M ? sm : M - 1] : 1.f;
+            }
+            if (EPI == BIG_PLAIN) {
+#pragma unroll
+                for (int j = 0; j < WTN; ++j)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const int gn = wave_n0 + j * 32 + 8 * (r >> 2) + 4 * nh + (r & 3);
+                        bv[j][r] = p.bias != nullptr ? p.bias[gn < N ? gn : N - 1] : 0.f;
+                    }
+            }
+        }
+        if (has_next) {
+            // the next tile's pieces A0 B0 A1 go out now, into the slots the stores below do not use
+            aim(next);
+#pragma unroll
+            for (int q = 0; q < 3; ++q)
+#pragma unroll
+                for (int i = 0; i < LA; ++i) issue_piece(q, q, i);
+        }
+
+        // ---------------------------------------------------------------- epilogue
+        // A product holds D[n][m]: lane l has row m = l % 32 and, in registers 4 g .. 4 g + 3, the columns
+        // 8 g + 4 (l / 32) + 0..3 of its 32.  A wavefront turns 32 rows at a time through its own 8 KB of LDS
+        // into whole rows and stores 16 bytes a lane.
+        char* stg = lds + STG + wave * STG_WAVE;
+
+        if (EPI == BIG_PLAIN || EPI == BIG_SWIGLU) {
+            constexpr int CW = EPI == BIG_SWIGLU ? WTN * 16 : WTN * 32;      // output columns of the wavefront per row
+            constexpr int SROW = CW * 2 + 8;                                   // staged row: 8 bytes of padding spread the banks
+            constexpr int LPR = CW * 2 / 16;                                   // lanes per row when reading back
+            const int out_n = EPI == BIG_SWIGLU ? N / 2 : N;
+            const int out_c0 = EPI == BIG_SWIGLU ? wave_n0 / 2 : wave_n0;
+            const bool aligned = (out_n & 7) == 0 && ((uintptr_t)p.out & 15) == 0;
+#pragma unroll
+            for (int i = 0; i < WTM; ++i) {
+                const float s = scale[i];            // the row scale of the norm whose rows x holds
+#pragma unroll
+                for (int j = 0; j < WTN; ++j) {
+                    const f32x16& t = acc[i][j];
+                    if (EPI == BIG_SWIGLU) {
+                        // registers r and r + 8 are gate and up of one channel (columns 16 apart)
+#pragma unroll
+                        for (int g = 0; g < 2; ++g) {
+                            bf16x4 v;
+#pragma unroll
+                            for (int c = 0; c < 4; ++c) {
+                                const float gate = s * t[4 * g + c], up = s * t[4 * g + c + 8];
+                                v[c] = (bf16)(gate / (1.f + expf(-gate)) * up);
+                            }
+                            *(bf16x4*)(stg + ml * SROW + (j * 16 + 8 * g + 4 * nh) * 2) = v;
+                        }
+                    } else {
+#pragma unroll
+                        for (int g = 0; g < 4; ++g) {
+                            bf16x4 v;
+#pragma unroll
+                            for (int c = 0; c < 4; ++c) v[c] = (bf16)(s * t[4 * g + c] + bv[j][4 * g + c]);
+                            *(bf16x4*)(stg + ml * SROW + (j * 32 + 8 * g + 4 * nh) * 2) = v;
+                        }
+                    }
+                }
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+                for (int pass = 0; pass < 32 * LPR / 64; ++pass) {
+                    const int row = pass * (64 / LPR) + lane / LPR, piece = lane % LPR;
+                    const u32x4 v = *(const u32x4*)(stg + row * SROW + piece * 16);
+                    const int gm = m0 + wm * (BM / 2) + i * 32 + row;
+                    const int gc = out_c0 + piece * 8;
+                    if (gm < M) {
+                        bf16* dst = p.out + (int64_t)gm * out_n + gc;
+                        if (aligned && gc + 8 <= out_n) *(u32x4*)dst = v;
+                        else {
+                            const bf16* e = (const bf16*)&v;
+                            for (int c = 0; c < 8; ++c)
+                                if (gc + c < out_n) dst[c] = e[c];
+                        }
+                    }
+                }
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            }
+        } else {
+            // h += product (+ bias): 32 rows x 32 columns of float32 at a time; a row is read back by 8 lanes
+            constexpr int SROW = 32 * 4 + 16;
+            const bool aligned = (N & 3) == 0 && ((uintptr_t)p.h & 15) == 0 &&
+                                 (p.weighted == nullptr || ((uintptr_t)p.weighted & 7) == 0);
+            const int stats_row = tn * WAVES_N + wn;
+#pragma unroll
+            for (int i = 0; i < WTM; ++i) {
+                float sq[4] = {0.f, 0.f, 0.f, 0.f};            // of the rows this lane reads back, over both products
+#pragma unroll
+                for (int j = 0; j < WTN; ++j) {
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                        const f32x16& t = acc[i][j];
+                        f32x4 v = {t[4 * g], t[4 * g + 1], t[4 * g + 2], t[4 * g + 3]};
+                        *(f32x4*)(stg + ml * SROW + (8 * g + 4 * nh) * 4) = v;
+                    }
+                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+                    for (int pass = 0; pass < 4; ++pass) {
+                        const int row = pass * 8 + (lane >> 3), piece = lane & 7;
+                        f32x4 v = *(const f32x4*)(stg + row * SROW + piece * 16);
+                        const int gm = m0 + wm * (BM / 2) + i * 32 + row;
+                        const int gn = wave_n0 + j * 32 + piece * 4;
+                        if (gm < M && gn < N) {
+                            float* hp = p.h + (int64_t)gm * N + gn;
+                            if (aligned && gn + 4 <= N) {
+                                f32x4 hv = *(const f32x4*)hp;
+#pragma unroll
+                                for (int c = 0; c < 4; ++c) {
+                                    hv[c] += v[c] + (p.bias != nullptr ? p.bias[gn + c] : 0.f);
+                                    sq[pass] += hv[c] * hv[c];
+                                }
+                                *(f32x4*)hp = hv;
+                                if (p.weighted != nullptr) {
+                                    bf16x4 wv;
+#pragma unroll
+                                    for (int c = 0; c < 4; ++c) wv[c] = (bf16)(p.norm_w[gn + c] * hv[c]);
+                                    *(bf16x4*)(p.weighted + (int64_t)gm * N + gn) = wv;
+                                }
+                            } else {
+                                for (int c = 0; c < 4; ++c)
+                                    if (gn + c < N) {
+                                        const float hv = hp[c] + v[c] + (p.bias != nullptr ? p.bias[gn + c] : 0.f);
+                                        hp[c] = hv;
+                                        sq[pass] += hv * hv;
+                                        if (p.weighted != nullptr) p.weighted[(int64_t)gm * N + gn + c] = (bf16)(p.norm_w[gn + c] * hv);
+                                    }
+                            }
+                        }
+                    }
+                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                }
+                if (p.stats_out != nullptr) {
+                    // the 8 lanes of a row add their squares in a fixed order
+#pragma unroll
+                    for (int pass = 0; pass < 4; ++pass) {
+                        float v = sq[pass];
+#pragma unroll
+                        for (int off = 4; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+                        const int gm = m0 + wm * (BM / 2) + i * 32 + pass * 8 + (lane >> 3);
+                        if ((lane & 7) == 0 && gm < M) p.stats_out[(int64_t)stats_row * p.stats_width + gm] = v;
+                    }
                 }
             }
-            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         }
+
+        if (!has_next) break;
+        // the staging is read: slots 3 and 4 take the next tile's B1 and A2
+        __syncthreads();
+#pragma unroll
+        for (int q = 3; q < 5; ++q)
+#pragma unroll
+            for (int i = 0; i < LA; ++i) issue_piece(q, q, i);
+        logical = next;
     }
 }
 
@@ -416,7 +507,7 @@ static bool big_use_wide(int m, int n) {
 
 template <int BN, int S, int NW, int EPI, bool KTAIL>
 static int big_launch_one(const BigArgs& args, hipStream_t stream) {
-    const int lds_bytes = S * (BIG_BM + BN) * BIG_ROW_BYTES;
+    const int lds_bytes = S == 5 ? 5 * 256 * BIG_ROW_BYTES : S * (BIG_BM + BN) * BIG_ROW_BYTES;
     static bool raised[64];
     int device = 0;
     hipError_t err = hipGetDevice(&device);
@@ -427,8 +518,15 @@ static int big_launch_one(const BigArgs& args, hipStream_t stream) {
         if (err != hipSuccess) return somi_fail("linear_big: %d bytes of LDS refused: %s", lds_bytes, hipGetErrorString(err));
         raised[device] = true;
     }
+    // one workgroup per tile; the wide form is persistent: at most one workgroup per compute unit, a multiple of 8
+    // (the dies), each walking its die's tiles
     const int per = ceil_div(args.tiles_m * args.tiles_n, 8);
-    hipLaunchKernelGGL((linear_big_kernel<BN, S, NW, EPI, KTAIL>), dim3(per * 8), dim3(NW * 64), lds_bytes, stream, args);
+    int per_die = per;
+    if (S == 5) {
+        const int cus_per_die = big_compute_units() / 8 > 0 ? big_compute_units() / 8 : 1;
+        per_die = per < cus_per_die ? per : cus_per_die;
+    }
+    hipLaunchKernelGGL((linear_big_kernel<BN, S, NW, EPI, KTAIL>), dim3(per_die * 8), dim3(NW * 64), lds_bytes, stream, args);
     SOMI_LAUNCH_CHECK("linear_big");
     return 0;
 }
@@ -439,7 +537,7 @@ static int big_launch(BigArgs& args, int tile, hipStream_t stream) {
     args.tiles_m = ceil_div(args.M, BIG_BM);
     args.tiles_n = ceil_div(args.N, wide ? 256 : 128);
     const bool ktail = args.K % BIG_BK != 0;
-    if (wide) return ktail ? big_launch_one<256, 2, 8, EPI, true>(args, stream) : big_launch_one<256, 2, 8, EPI, false>(args, stream);
+    if (wide) return ktail ? big_launch_one<256, 5, 8, EPI, true>(args, stream) : big_launch_one<256, 5, 8, EPI, false>(args, stream);
     return ktail ? big_launch_one<128, 3, 4, EPI, true>(args, stream) : big_launch_one<128, 3, 4, EPI, false>(args, stream);
 }
 
@@ -455,6 +553,32 @@ static int big_check(const char* what, const void* x, int64_t ldx, const void* w
     return 0;
 }
 
+// s[m] = 1 / sqrt(sum_b stats[b][m] / k + eps): the scale an RMS norm gives row m, from the partial sums of squares
+// that the residual forms leave (here and in linear_fused.hip), added in the order of the blocks.
+__global__ void __launch_bounds__(256)
+row_scale_kernel(const float* __restrict__ stats, int blocks, int width, int m, float inv_k, float eps, float* __restrict__ out) {
+    const int row = blockIdx.x * 256 + threadIdx.x;
+    if (row >= m) return;
+    const float* sp = stats + row;
+    float part[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) part[e] = 0.f;
+    for (int b = 0; b < blocks; b += 8)
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+            if (b + e < blocks) part[e] += sp[(int64_t)(b + e) * width];
+    const float sum = ((part[0] + part[1]) + (part[2] + part[3])) + ((part[4] + part[5]) + (part[6] + part[7]));
+    out[row] = rsqrtf(sum * inv_k + eps);
+}
+
+extern "C" int somi_row_scale(const float* stats, int blocks, int width, int m, int k, float eps, float* out, hipStream_t stream) {
+    SOMI_REQUIRE(stats != nullptr && out != nullptr && blocks > 0 && m > 0 && width >= m && k > 0,
+                 "row_scale: bad arguments (blocks=%d width=%d m=%d k=%d)", blocks, width, m, k);
+    hipLaunchKernelGGL(row_scale_kernel, dim3(ceil_div(m, 256)), dim3(256), 0, stream, stats, blocks, width, m, 1.f / (float)k, eps, out);
+    SOMI_LAUNCH_CHECK("row_scale");
+    return 0;
+}
+
 // Workgroup columns that write row statistics in the residual form: the first size of stats_out.
 // tile: 0 lets the launcher choose, 128 or 256 asks for that tile width.
 extern "C" int somi_linear_big_stats_blocks(int m, int n, int tile) {
@@ -463,21 +587,17 @@ extern "C" int somi_linear_big_stats_blocks(int m, int n, int tile) {
 }
 
 // out = s * (x . w^T) + bias -> bfloat16 [M, N]; with swiglu w is [N, K] with gate and up rows interleaved in blocks
-// of 16 and out is [M, N / 2] = silu(s g) * (s u).  stats (or null): [stats_blocks][stats_width] partial sums of
-// squares; s[m] = 1 / sqrt(sum_b stats[b][m] / K + eps).
+// of 16 and out is [M, N / 2] = silu(s g) * (s u).  row_scale (or null): s [M], see somi_row_scale.
 extern "C" int somi_linear_big(const void* x, int64_t ldx, const void* w, int64_t ldw, const float* bias, void* out,
-                               int m, int n, int k, const float* stats, int stats_blocks, int stats_width, float eps,
-                               int swiglu, int tile, hipStream_t stream) {
+                               int m, int n, int k, const float* row_scale, int swiglu, int tile, hipStream_t stream) {
     if (big_check("linear_big", x, ldx, w, ldw, m, n, k) != 0) return 1;
     SOMI_REQUIRE(out != nullptr, "linear_big: no output");
     SOMI_REQUIRE(!swiglu || (n % 32 == 0 && bias == nullptr), "linear_big: the gated form needs N a multiple of 32 and no bias");
-    SOMI_REQUIRE(stats == nullptr || (stats_blocks > 0 && stats_width >= m), "linear_big: row statistics of %d x %d do not cover %d rows",
-                 stats_blocks, stats_width, m);
     SOMI_REQUIRE(tile == 0 || tile == 128 || tile == 256, "linear_big: tile width %d (0, 128 or 256)", tile);
     BigArgs args = {};
     args.x = (const bf16*)x; args.ldx = ldx; args.w = (const bf16*)w; args.ldw = ldw; args.bias = bias;
     args.M = m; args.N = n; args.K = k; args.out = (bf16*)out;
-    args.stats_in = stats; args.stats_blocks = stats_blocks; args.stats_width = stats_width; args.eps = eps;
+    args.row_scale = row_scale;
     return swiglu ? big_launch<BIG_SWIGLU>(args, tile, stream) : big_launch<BIG_PLAIN>(args, tile, stream);
 }
 

@@ -17,7 +17,6 @@ import torch
 
 from ..cache.manager import CacheManager
 from ..cache.pool import OutOfPages
-from ..kernels import library_tuning
 from ..models.decoder import DecoderModel
 from .batch import StaticStep, StepBatch, StepEntry, build_step
 
@@ -132,28 +131,6 @@ class ModelRunner:
             self.cache.commit(request_id, count)
         self.steps_run += 1
         return logits
-
-    # ----------------------------------------------------------------- warm-up
-    def tune_library_products(self, rows: int) -> int:
-        """Times the library's solutions for the products of a portion of ``rows`` tokens.
-
-        Runs one throw-away portion of that length (fewer if the free pages do not hold it) for a
-        request of its own, with the library's autotuning on, and gives the pages back.  Later steps
-        with exactly this many tokens use the recorded solutions; other sizes are not affected.
-        Returns the number of tokens the portion had (0: nothing was free).
-        """
-        probe = ("library tuning probe", id(self))
-        self.cache.register(probe)
-        try:
-            while rows > 0 and not self.cache.can_reserve([(probe, rows)]):
-                rows //= 2
-            if rows > 0:
-                with library_tuning.tuning():
-                    self.step([StepEntry(probe, [0] * rows, [])])
-                torch.cuda.synchronize()
-        finally:
-            self.cache.free(probe)
-        return rows
 
     # ------------------------------------------------------------- HIP graphs
     def _capture(self, entries: list[StepEntry], rows: int, widths: list[int],

@@ -50,7 +50,7 @@ def parse_args(argv: list[str] | None = None) -> argparse.Namespace:
                         help="Repetition penalty applied by the sampler.")
     parser.add_argument("--output-file", type=str, default=None, help="Append results to a JSONL file.")
     parser.add_argument("--warm-up", action="store_true",
-                        help="Let the library time its matrix products for full prompt portions first.")
+                        help="Capture the decode steps as graphs before the prompt is served.")
     return parser.parse_args(argv)
 
 

@@ -92,17 +92,12 @@ class LLM:
     def warm_up(self, max_context: int | None = None) -> int:
         """Optional work before requests are served; not in the reference.
 
-        In bfloat16 the library times its solutions for the matrix products of a full prompt portion (the
-        float32 engine has no library products), and the decode steps of up to ``max_concurrent`` requests
-        with contexts of up to ``max_context`` tokens (default: 4,096, or what the pool holds if that is less)
-        are captured as graphs, so that serving never stops to capture one.  Returns the portion length that
-        was tuned.
+        The decode steps of up to ``max_concurrent`` requests with contexts of up to ``max_context`` tokens
+        (default: 4,096, or what the pool holds if that is less) are captured as graphs, so that serving never
+        stops to capture one.  Returns the number of graphs captured.
         """
         pool_tokens = self.options.num_blocks * self.options.block_size
-        self.runner.capture_decode_graphs(self.options.max_concurrent, min(max_context or 4096, pool_tokens))
-        if self.dtype != "bfloat16":
-            return 0
-        return self.runner.tune_library_products(min(self.options.chunk, self.options.max_num_batched_tokens))
+        return self.runner.capture_decode_graphs(self.options.max_concurrent, min(max_context or 4096, pool_tokens))
 
     # ---------------------------------------------------------------- generate
     def _encode(self, prompt) -> tuple[list[int], bool]:

@@ -8,8 +8,7 @@ from . import ops
 
 SKINNY_MAX_ROWS = 64   # what the skinny MFMA kernel takes
 MID_PASSES_ROWS = 192  # up to here a product with long K and few columns runs the split-K kernel in passes of 64 rows
-SKINNY_ROWS = 64       # up to here it beats the library product at 7B layer sizes (measured inside decode steps
-                       # of 64 requests: gate_up with the gate fused in 80 us against 90 + 5, down 55 against 60)
+SKINNY_ROWS = 64       # up to here the few-rows kernels run; beyond, the many-rows kernel (ops.linear_big)
 
 
 def _mid_is_faster(m: int, n: int, k: int) -> bool:
@@ -22,10 +21,11 @@ def _mid_is_faster(m: int, n: int, k: int) -> bool:
     return (k >= 8192 and n <= 8192) or n >= 16384
 
 
-# Above SKINNY_ROWS rows the products of the feed-forward run the many-rows kernel (ops.linear_big), also with
-# the norm before them and the residual add after them taken in.  The other products of that size (q/k/v, o,
-# logits of many rows) are plain library GEMMs in the reference; which of the two runs them here:
-BIG_FOR_ALL = True
+def prefers_mid_passes(m: int, n: int, k: int) -> bool:
+    """More than SKINNY_ROWS rows, but few enough that a product with a long K and few columns (down) runs faster
+    as passes of the split-K kernel over 64 rows each than on the 256-row tiles of the many-rows kernel, which are
+    too few to fill the device there (7B down projection: 62 to 67 us at 65 to 128 rows, 99 at 192, against 157)."""
+    return SKINNY_ROWS < m <= MID_PASSES_ROWS and k >= 8192 and n <= 8192
 
 
 def linear_swiglu(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
@@ -60,14 +60,14 @@ def linear_scaled(x: torch.Tensor, eps: float, stats: torch.Tensor, weight: torc
 
 
 def linear(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None,
-           out_dtype: torch.dtype | None = None, bias_lowp: torch.Tensor | None = None) -> torch.Tensor:
+           out_dtype: torch.dtype | None = None) -> torch.Tensor:
     """x @ weight.T (+ bias).
 
     float32 always takes the plain FMA kernel (the true 32-bit path).  bfloat16 with few rows takes the
-    hand-written skinny MFMA kernel; with many rows the product is a plain library GEMM, as it is in the
-    reference (nn.Linear / F.linear), with float32 outputs (logits) produced 64 rows at a time by the
-    skinny kernel so that they are never rounded to bfloat16.  The library product is also what runs inside
-    captured decode steps of more than SKINNY_ROWS requests; tests replay such graphs against eager steps.
+    hand-written few-rows MFMA kernels, with more rows the many-rows MFMA kernel (256-row tiles); float32
+    outputs of many rows (logits) are produced 64 rows at a time by the few-rows kernel so that they are never
+    rounded to bfloat16.  Operands the MFMA kernels do not take (K no multiple of 8, unaligned) run the plain
+    kernel.
     """
     out_dtype = out_dtype or x.dtype
     if x.dtype == torch.float32:
@@ -79,18 +79,14 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = No
         if _mid_is_faster(m, weight.shape[0], k):
             return ops.linear_mid(x, weight, bias, out_dtype)
         return ops.linear_skinny(x, weight, bias, out_dtype)
-    if BIG_FOR_ALL and out_dtype == x.dtype and ops.big_supported(x, weight):
-        return ops.linear_big(x, weight, bias)
-    if m <= MID_PASSES_ROWS and k >= 8192 and weight.shape[0] <= 8192 and out_dtype == x.dtype:
-        # long K and few columns (down): the library's product leaves most of the device idle here (95 us at 65 to
-        # 128 rows of the 7B down projection, 111 at 192); the split-K kernel, 64 rows at a time, takes 62 to 67 and 99
+    if prefers_mid_passes(m, weight.shape[0], k) and out_dtype == x.dtype:
         out = torch.empty((m, weight.shape[0]), dtype=out_dtype, device=x.device)
         for at in range(0, m, SKINNY_MAX_ROWS):
             ops.linear_mid(x[at:at + SKINNY_MAX_ROWS], weight, bias, out_dtype, out=out[at:at + SKINNY_MAX_ROWS])
         return out
+    if out_dtype == x.dtype and ops.big_supported(x, weight):
+        return ops.linear_big(x, weight, bias)
     if out_dtype == torch.float32:
         return torch.cat([ops.linear_skinny(x[at:at + SKINNY_MAX_ROWS], weight, bias, out_dtype)
                           for at in range(0, m, SKINNY_MAX_ROWS)])
-    if bias is not None and bias_lowp is None:
-        bias_lowp = bias.to(x.dtype)
-    return torch.nn.functional.linear(x, weight, bias_lowp)
+    return ops.linear_plain(x, weight, bias, out_dtype)

@@ -353,19 +353,20 @@ def linear_big(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None 
     m, n, k = _big_operands(x, weight, bias, "linear_big")
     if swiglu and (n % 32 or bias is not None):
         raise KernelError(f"linear_big: the gated form needs an even number of 16-row blocks and no bias, got N = {n}")
-    blocks = width = 0
+    row_scale = None
     if stats is not None:
         _need(stats, "row statistics", torch.float32)
         if stats.dim() != 2 or stats.shape[1] < m:
             raise KernelError(f"linear_big: row statistics must be [blocks, >= {m}], got {tuple(stats.shape)}")
-        blocks, width = stats.shape
+        row_scale = torch.empty((m,), dtype=torch.float32, device=x.device)
+        _check(library().somi_row_scale(_ptr(stats), stats.shape[0], stats.shape[1], m, k, ctypes.c_float(eps),
+                                        _ptr(row_scale), _stream()))
     cols = n // 2 if swiglu else n
     if out is None:
         out = torch.empty((m, cols), dtype=torch.bfloat16, device=x.device)
     _need(out, "linear_big out", torch.bfloat16, (m, cols))
     _check(library().somi_linear_big(_ptr(x), ctypes.c_int64(x.stride(0)), _ptr(weight), ctypes.c_int64(weight.stride(0)),
-                                     _ptr(bias), _ptr(out), m, n, k, _ptr(stats), blocks, width, ctypes.c_float(eps),
-                                     1 if swiglu else 0, int(tile), _stream()))
+                                     _ptr(bias), _ptr(out), m, n, k, _ptr(row_scale), 1 if swiglu else 0, int(tile), _stream()))
     return out
 
 

@@ -53,9 +53,6 @@ class Projection:
         self.weight = weight
         self.bias = bias
         self.out_features, self.in_features = weight.shape
-        # the library GEMM used for many rows wants the bias in the compute dtype (exact for a
-        # bias that came from a bfloat16 checkpoint)
-        self.bias_lowp = bias.to(weight.dtype) if bias is not None and weight.dtype != torch.float32 else None
 
     @classmethod
     def stacked(cls, weights: list[torch.Tensor], biases: list[torch.Tensor] | None = None) -> "Projection":
@@ -70,12 +67,16 @@ class Projection:
             if out_dtype in (None, torch.bfloat16) and self.fusable(x.h.shape[0]):
                 return linear_kernels.linear_scaled(x.weighted, x.norm.eps, x.stats, self.weight, self.bias)
             x = x.materialize()
-        return linear_kernels.linear(x, self.weight, self.bias, out_dtype, self.bias_lowp)
+        return linear_kernels.linear(x, self.weight, self.bias, out_dtype)
 
     def fusable(self, rows: int) -> bool:
         """The kernels that fuse this product with the norm before it or the residual add after it take it."""
-        return (self.weight.dtype == torch.bfloat16 and rows > 0 and self.in_features % 8 == 0
-                and self.weight.data_ptr() % 16 == 0)
+        if not (self.weight.dtype == torch.bfloat16 and rows > 0 and self.in_features % 8 == 0
+                and self.weight.data_ptr() % 16 == 0):
+            return False
+        # some dozens of rows beyond what the few-rows kernels take, over a long K and few columns: the split-K
+        # kernel in passes of 64 rows (kernels.linear.linear) is faster there than one 256-row tile per column tile
+        return not linear_kernels.prefers_mid_passes(rows, self.out_features, self.in_features)
 
     def deferred(self, x: torch.Tensor) -> "torch.Tensor | DeferredProduct":
         """The product, or a promise of it where the residual stream can compute and add it in one kernel."""

@@ -271,18 +271,17 @@ def test_command_line_generates_and_appends_jsonl(model_folders, tmp_path):
     assert json.loads(out_file.read_text().strip()) == record
 
 
-def test_warm_up_tunes_library_products_without_changing_results(model_folders, tmp_path, monkeypatch):
-    """The optional warm-up lets the library pick its matrix-product solutions for full prompt portions: the
-    tokens stay what the plain implementation gives, the pages are all given back, and no file appears in
-    the working directory."""
+def test_warm_up_captures_decode_graphs_without_changing_results(model_folders, tmp_path, monkeypatch):
+    """The optional warm-up captures the decode graphs ahead of any request: the tokens stay what the plain
+    implementation gives, the pages are all given back, generation captures no graph of its own, and no file
+    appears in the working directory."""
     monkeypatch.chdir(tmp_path)
     folder = model_folders["B"]
     llm = LLM(folder, dtype="bfloat16", num_blocks=64, block_size=8, max_num_batched_tokens=96, max_concurrent=4,
               eos_token_id=-1)
     free_before = llm.kv_manager.free_pages()
-    assert llm.warm_up() == 96
-    # and the decode graphs of up to 4 requests (1, 2 and 4 rows) with tables of 16, 32 and 64 pages (the pool's 512
-    # tokens) are captured before any request came
+    # up to 4 requests (1, 2 and 4 rows) with tables of 16, 32 and 64 pages (the pool's 512 tokens)
+    assert llm.warm_up() == 9
     assert sorted(llm.runner._graphs) == [(rows, (width,)) for rows in (1, 2, 4) for width in (16, 32, 64)]
     assert llm.kv_manager.free_pages() == free_before
     llm.kv_manager.check_invariants()
@@ -292,7 +291,7 @@ def test_warm_up_tunes_library_products_without_changing_results(model_folders, 
     assert_greedy_matches(got, want, prompts, cfg, weights, exact=False)
     assert len(llm.runner._graphs) == 9 and llm.runner.graph_replays > 0, "generation captured a graph of its own"
     assert list(tmp_path.iterdir()) == []
-    assert LLM(folder, dtype="float32", num_blocks=64, block_size=8).warm_up() == 0
+    assert LLM(folder, dtype="float32", num_blocks=64, block_size=8, max_concurrent=2).warm_up() == 6
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
