@@ -73,7 +73,7 @@ template <int DT, int QB>
 __global__ void __launch_bounds__(256)
 attention_prefill_kernel(const bf16* __restrict__ q, int64_t q_stride, const bf16* __restrict__ kc,
                          const bf16* __restrict__ vc, const int* __restrict__ block_table, int max_blocks,
-                         const int* __restrict__ entry_start, const int* __restrict__ entry_first_pos, int nq,
+                         const int* __restrict__ entry_start, const int* __restrict__ entry_first_pos, const int* __restrict__ entry_len, int nq,
                          int nkv, int page_size, int window, float scale_log2, bf16* __restrict__ out) {
     constexpr int D = DT * 16;
     constexpr int QK_STEPS = (DT + 1) / 2;
@@ -82,7 +82,7 @@ attention_prefill_kernel(const bf16* __restrict__ q, int64_t q_stride, const bf1
     const int kvh = h / (nq / nkv);
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4;
     const int start = entry_start[e];
-    const int len = entry_start[e + 1] - start;
+    const int len = entry_len != nullptr ? entry_len[e] : entry_start[e + 1] - start;
     const int q0 = (blockIdx.x * (blockDim.x >> 6) + wave) * QW;
     if (q0 >= len) return;                              // no workgroup barrier is used below
     const int pos0 = entry_first_pos[e];
@@ -246,7 +246,7 @@ template <int DT, int QB, int KS>
 __global__ void __launch_bounds__(256 * KS, 2 * KS)     // the second figure: wavefronts per SIMD to leave room for
 attention_prefill_lds_kernel(const bf16* __restrict__ q, int64_t q_stride, const bf16* __restrict__ kc,
                              const bf16* __restrict__ vc, const int* __restrict__ block_table, int max_blocks,
-                             const int* __restrict__ entry_start, const int* __restrict__ entry_first_pos, int nq,
+                             const int* __restrict__ entry_start, const int* __restrict__ entry_first_pos, const int* __restrict__ entry_len, int nq,
                              int nkv, int page_size, int window, float scale_log2, bf16* __restrict__ out) {
     constexpr int D = DT * 16;
     constexpr int QK_STEPS = (DT + 1) / 2;
@@ -273,7 +273,7 @@ attention_prefill_lds_kernel(const bf16* __restrict__ q, int64_t q_stride, const
     const int kh = tid >> 8;                                // which of a step's KS tiles it computes and fetches
     const int tid256 = tid & 255;
     const int start = entry_start[e];
-    const int len = entry_start[e + 1] - start;
+    const int len = entry_len != nullptr ? entry_len[e] : entry_start[e + 1] - start;
     const int group = gridDim.z - 1 - blockIdx.z;
     const int g0 = group * QG;
     if (g0 >= len) return;                                  // the whole workgroup leaves together
@@ -549,7 +549,7 @@ static int prefill_page_entries(int max_blocks, int page_size, int window) {
 
 template <int DT>
 static int launch_prefill_lds(const void* q, int64_t q_stride, const void* kc, const void* vc, const int* block_table,
-                              int max_blocks, const int* entry_start, const int* entry_first_pos, int n_entries,
+                              int max_blocks, const int* entry_start, const int* entry_first_pos, const int* entry_len, int n_entries,
                               int max_entry_len, int max_context, int shape, int nq, int nkv, int page_size,
                               int window, float scale, void* out, hipStream_t stream) {
     // 128 queries per workgroup read every key and value tile half as often as 64 do, but the longest
@@ -570,7 +570,7 @@ static int launch_prefill_lds(const void* q, int64_t q_stride, const void* kc, c
                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)page_list);
         hipLaunchKernelGGL((attention_prefill_lds_kernel<DT, 2, 1>), grid, dim3(256), page_list, stream, (const bf16*)q,
                            q_stride, (const bf16*)kc, (const bf16*)vc, block_table, max_blocks, entry_start,
-                           entry_first_pos, nq, nkv, page_size, window, scale * 1.44269504088896341f, (bf16*)out);
+                           entry_first_pos, entry_len, nq, nkv, page_size, window, scale * 1.44269504088896341f, (bf16*)out);
     } else if (shape == PREFILL_SHAPE_AUTO
                    ? (int64_t)grid.x * grid.y * grid.z < PREFILL_KEY_SPLIT_BELOW && reach >= PREFILL_KEY_SPLIT_REACH
                    : shape == PREFILL_SHAPE_SPLIT) {
@@ -580,14 +580,14 @@ static int launch_prefill_lds(const void* q, int64_t q_stride, const void* kc, c
                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)page_list);
         hipLaunchKernelGGL((attention_prefill_lds_kernel<DT, 1, 2>), grid, dim3(512), page_list, stream, (const bf16*)q,
                            q_stride, (const bf16*)kc, (const bf16*)vc, block_table, max_blocks, entry_start,
-                           entry_first_pos, nq, nkv, page_size, window, scale * 1.44269504088896341f, (bf16*)out);
+                           entry_first_pos, entry_len, nq, nkv, page_size, window, scale * 1.44269504088896341f, (bf16*)out);
     } else {
         if (page_list > 16 * 1024)
             (void)hipFuncSetAttribute((const void*)attention_prefill_lds_kernel<DT, 1, 1>,
                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)page_list);
         hipLaunchKernelGGL((attention_prefill_lds_kernel<DT, 1, 1>), grid, dim3(256), page_list, stream, (const bf16*)q,
                            q_stride, (const bf16*)kc, (const bf16*)vc, block_table, max_blocks, entry_start,
-                           entry_first_pos, nq, nkv, page_size, window, scale * 1.44269504088896341f, (bf16*)out);
+                           entry_first_pos, entry_len, nq, nkv, page_size, window, scale * 1.44269504088896341f, (bf16*)out);
     }
     SOMI_LAUNCH_CHECK("attention_prefill_lds");
     return 0;
@@ -595,14 +595,14 @@ static int launch_prefill_lds(const void* q, int64_t q_stride, const void* kc, c
 
 template <int DT, int QB>
 static int launch_prefill(const void* q, int64_t q_stride, const void* kc, const void* vc, const int* block_table,
-                          int max_blocks, const int* entry_start, const int* entry_first_pos, int n_entries,
+                          int max_blocks, const int* entry_start, const int* entry_first_pos, const int* entry_len, int n_entries,
                           int max_entry_len, int nq, int nkv, int page_size, int window, float scale, void* out,
                           hipStream_t stream) {
     constexpr int WAVES = 4;
     const int per_group = WAVES * QB * 16;
     const dim3 grid(ceil_div(max_entry_len, per_group), n_entries, nq);
     hipLaunchKernelGGL((attention_prefill_kernel<DT, QB>), grid, dim3(WAVES * 64), 0, stream, (const bf16*)q, q_stride,
-                       (const bf16*)kc, (const bf16*)vc, block_table, max_blocks, entry_start, entry_first_pos, nq, nkv,
+                       (const bf16*)kc, (const bf16*)vc, block_table, max_blocks, entry_start, entry_first_pos, entry_len, nq, nkv,
                        page_size, window, scale * 1.44269504088896341f, (bf16*)out);
     SOMI_LAUNCH_CHECK("attention_prefill");
     return 0;
@@ -610,13 +610,14 @@ static int launch_prefill(const void* q, int64_t q_stride, const void* kc, const
 
 // Attention of every token of every entry (portion) over its request's pages.  entry_start: [n_entries + 1]
 // offsets of the portions in the flat token batch; entry_first_pos: [n_entries] position of each portion's
-// first token; max_entry_len: the longest portion (sizes the grid).  bfloat16 only; head_dim a multiple of 16
+// first token; entry_len (or null): [n_entries] the portions' lengths where they differ from the offsets' (0 leaves a
+// portion out: its tokens are somebody else's); max_entry_len: the longest portion (sizes the grid).  bfloat16 only; head_dim a multiple of 16
 // up to 256; page_size a multiple of 4.  k_cache [pages, nkv, page_size, D], v_cache [pages, nkv, D, page_size];
 // out: [n_tokens, nq * D].  max_context: the longest context a portion ends at (a hint for the launch shape; 0: unknown).
 // shape: 0 lets the launcher choose; 1..3 ask for a launch shape of the LDS kernel (PREFILL_SHAPE_*).
 extern "C" int somi_attention_prefill(const void* q, int64_t q_stride, const void* k_cache, const void* v_cache,
                                       const int* block_table, int max_blocks, const int* entry_start,
-                                      const int* entry_first_pos, int n_entries, int max_entry_len, int max_context,
+                                      const int* entry_first_pos, const int* entry_len, int n_entries, int max_entry_len, int max_context,
                                       int shape, int nq, int nkv, int D, int page_size, int window, float scale,
                                       void* out, hipStream_t stream) {
     SOMI_REQUIRE(n_entries >= 0 && max_entry_len >= 0 && nq > 0 && nkv > 0 && max_blocks > 0,
@@ -635,16 +636,16 @@ extern "C" int somi_attention_prefill(const void* q, int64_t q_stride, const voi
 #define SOMI_PREFILL(DT, QB)                                                                                       \
     case DT:                                                                                                       \
         return launch_prefill<DT, QB>(q, q_stride, k_cache, v_cache, block_table, max_blocks, entry_start,         \
-                                      entry_first_pos, n_entries, max_entry_len, nq, nkv, page_size, window, scale, \
+                                      entry_first_pos, entry_len, n_entries, max_entry_len, nq, nkv, page_size, window, scale, \
                                       out, stream)
 #define SOMI_PREFILL_LDS(DT)                                                                                       \
     case DT:                                                                                                       \
         if (!lds_ok)                                                                                               \
             return launch_prefill<DT, 4>(q, q_stride, k_cache, v_cache, block_table, max_blocks, entry_start,      \
-                                         entry_first_pos, n_entries, max_entry_len, nq, nkv, page_size, window,    \
+                                         entry_first_pos, entry_len, n_entries, max_entry_len, nq, nkv, page_size, window,    \
                                          scale, out, stream);                                                      \
         return launch_prefill_lds<DT>(q, q_stride, k_cache, v_cache, block_table, max_blocks, entry_start,         \
-                                      entry_first_pos, n_entries, max_entry_len, max_context, shape, nq, nkv,      \
+                                      entry_first_pos, entry_len, n_entries, max_entry_len, max_context, shape, nq, nkv,      \
                                       page_size, window, scale, out, stream)
     // head sizes 32..128 stage keys and values through LDS; the others (LDS would not hold two tiles, or a
     // tile is smaller than the workgroup's loads) keep them in registers per wavefront, and so do page sizes

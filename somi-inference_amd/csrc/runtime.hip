@@ -28,4 +28,12 @@ extern "C" int somi_device_arch(char* out, int capacity) {
     return 0;
 }
 
+// Compute units of the current device (256 on an MI355X); what launch shapes aim their workgroup counts at.
+extern "C" int somi_compute_units() {
+    int device = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&device) != hipSuccess || hipGetDeviceProperties(&prop, device) != hipSuccess) return -1;
+    return prop.multiProcessorCount;
+}
+
 extern "C" int somi_abi_version() { return 1; }

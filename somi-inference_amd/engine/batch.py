@@ -59,11 +59,16 @@ class StepBatch:
     context_lens: torch.Tensor      # [E] int32: tokens of each request after this step
     state_slots: torch.Tensor       # [E] int32
     logit_rows: torch.Tensor        # [R] int32 flat token indices whose logits are wanted
+    long_entry_len: torch.Tensor    # [E] int32: an entry's length if it is longer than SHORT_ENTRY tokens, else 0
+    short_tokens: torch.Tensor      # [Ns] int32: flat indices of the tokens of the entries of at most SHORT_ENTRY tokens
     paged: list[PagedView]
     entries: list[EntryInfo]        # host mirror
     max_entry_len: int
     max_context: int
     block_size: int
+
+
+SHORT_ENTRY = 8      # entries of at most this many tokens are attended token by token (the decode kernel)
 
 
 class _Padding:
@@ -130,6 +135,8 @@ def _layout(entries: list[StepEntry], cache: CacheManager, table_widths: list[in
         np.asarray([i.first_position + i.length for i in infos], dtype=np.int32),
         np.asarray([i.state_slot for i in infos], dtype=np.int32),
         np.asarray(logit_rows, dtype=np.int32),
+        np.asarray([i.length if i.length > SHORT_ENTRY else 0 for i in infos], dtype=np.int32),
+        np.asarray([t for i in infos if i.length <= SHORT_ENTRY for t in range(i.start, i.start + i.length)], dtype=np.int32),
     ]
     for table, slots in zip(tables, slot_maps):
         sections += [slots, table.reshape(-1)]
@@ -144,12 +151,12 @@ def _views(on_device: torch.Tensor, sizes: list[int], infos: list[EntryInfo], wi
         return on_device[int(offsets[i]):int(offsets[i + 1])]
 
     e = len(infos)
-    paged = [PagedView(part(8 + 2 * g), part(9 + 2 * g).view(e, widths[g])) for g in range(num_groups)]
+    paged = [PagedView(part(10 + 2 * g), part(11 + 2 * g).view(e, widths[g])) for g in range(num_groups)]
     return StepBatch(
         num_tokens=sizes[0], num_entries=e, num_logit_rows=sizes[7],
         token_ids=part(0), positions=part(1), token_entry=part(2), entry_start=part(3),
         entry_first_position=part(4), context_lens=part(5), state_slots=part(6), logit_rows=part(7),
-        paged=paged, entries=infos,
+        long_entry_len=part(8), short_tokens=part(9), paged=paged, entries=infos,
         max_entry_len=max((i.length for i in infos), default=0),
         max_context=max_context if max_context is not None else max((i.first_position + i.length for i in infos), default=0),
         block_size=block_size,

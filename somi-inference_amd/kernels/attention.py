@@ -6,20 +6,20 @@ import torch
 
 from . import ops
 
-TARGET_WORKGROUPS = 256         # one per compute unit (whole decode steps at 4,096 keys, 7B sizes: 8 / 16 / 32 / 64 requests
-                                # 3.42 / 3.99 / 5.27 / 7.20 ms against 3.43 / 4.05 / 5.39 / 7.29 with 512; 192 and 128 are slower)
+# The decode kernel aims at one workgroup per compute unit (whole decode steps at 4,096 keys, 7B sizes, 256 units:
+# 8 / 16 / 32 / 64 requests 3.42 / 3.99 / 5.27 / 7.20 ms against 3.43 / 4.05 / 5.39 / 7.29 with two per unit; fewer are slower).
 MIN_SPLIT = 64                  # keys per split at least (a multiple of the 16-key tile)
 MAX_SPLITS = 1024               # what the merge kernel holds
-DECODE_PORTION = 8              # batches whose longest portion is at most this take the decode kernel
+DECODE_PORTION = 8              # portions of at most this many tokens take the decode kernel (engine.batch.SHORT_ENTRY)
 
 
 def decode_splits(num_tokens: int, groups: int, max_context: int) -> tuple[int, int]:
     """(split_len, num_splits): how the keys of a request are cut over workgroups so that
-    ``num_tokens * groups * num_splits`` is about TARGET_WORKGROUPS.  Boundaries are multiples of
+    ``num_tokens * groups * num_splits`` is about the number of compute units.  Boundaries are multiples of
     MIN_SPLIT in absolute positions."""
     max_context = max(1, max_context)
     most = (max_context + MIN_SPLIT - 1) // MIN_SPLIT
-    splits = max(1, min(TARGET_WORKGROUPS // max(1, num_tokens * groups), most, MAX_SPLITS))
+    splits = max(1, min(ops.compute_units() // max(1, num_tokens * groups), most, MAX_SPLITS))
     split_len = ((max_context + splits - 1) // splits + MIN_SPLIT - 1) // MIN_SPLIT * MIN_SPLIT
     return split_len, (max_context + split_len - 1) // split_len
 
@@ -45,11 +45,17 @@ def paged_attention(qkv: torch.Tensor, num_heads: int, k_cache: torch.Tensor, v_
     groups = nkv * ((num_heads // nkv + 15) // 16)
     out = torch.empty((qkv.shape[0], num_heads * head_dim), dtype=qkv.dtype, device=qkv.device)
     if step.max_entry_len > DECODE_PORTION:
-        # portions of prompts: query tiles against key tiles (single tokens in the same batch ride along
-        # as portions of one)
+        # portions of prompts: query tiles against key tiles.  Single tokens (and portions of a few) in the same
+        # batch keep the kernel that splits a request's keys over workgroups: as a query tile with one live row
+        # one workgroup would walk the whole context.
+        short = step.short_tokens.numel()
         ops.attention_prefill(qkv, qkv.shape[1], k_cache, v_cache, block_table, step.entry_start,
                               step.entry_first_position, step.max_entry_len, num_heads, window, scale, out,
-                              max_context=step.max_context)
+                              max_context=step.max_context, entry_len=step.long_entry_len if short else None)
+        if short:
+            split_len, num_splits = decode_splits(short, groups, step.max_context)
+            ops.attention_decode(qkv, qkv.shape[1], k_cache, v_cache, block_table, step.token_entry, step.positions,
+                                 num_heads, window, scale, split_len, num_splits, out, token_list=step.short_tokens)
         return out
     split_len, num_splits = decode_splits(step.num_tokens, groups, step.max_context)
     ops.attention_decode(qkv, qkv.shape[1], k_cache, v_cache, block_table, step.token_entry, step.positions,

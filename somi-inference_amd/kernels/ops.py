@@ -34,6 +34,20 @@ def dtype_code(dtype: torch.dtype) -> int:
     raise KernelError(f"unsupported dtype {dtype}; kernels take float32 and bfloat16")
 
 
+_compute_units: dict[int, int] = {}
+
+
+def compute_units() -> int:
+    """Compute units of the current device, asked once per device."""
+    device = torch.cuda.current_device()
+    if device not in _compute_units:
+        count = library().somi_compute_units()
+        if count <= 0:
+            raise KernelError("the device does not report its compute units")
+        _compute_units[device] = count
+    return _compute_units[device]
+
+
 def _stream() -> ctypes.c_void_p:
     # the raw handle of torch's current stream on the current device, without building a Stream object
     # (torch.cuda.current_stream() costs several microseconds, and every launch asks)
@@ -243,12 +257,14 @@ def attention_decode(q: torch.Tensor, q_stride: int, k_cache: torch.Tensor, v_ca
 def attention_prefill(q: torch.Tensor, q_stride: int, k_cache: torch.Tensor, v_cache: torch.Tensor,
                       block_table: torch.Tensor, entry_start: torch.Tensor, entry_first_position: torch.Tensor,
                       max_entry_len: int, nq: int, window: int, scale: float, out: torch.Tensor,
-                      max_context: int = 0, shape: int = 0) -> None:
+                      max_context: int = 0, shape: int = 0, entry_len: torch.Tensor | None = None) -> None:
     """MFMA causal attention of every token of every portion over its request's pages, into ``out``
     ([N, nq * D] bfloat16).  entry_start: [E + 1] int32 offsets of the portions in the flat batch;
     entry_first_position: [E] int32.  ``max_context``: the longest context a portion ends at, a hint for the
     launch shape (0: unknown).  ``shape``: 0 lets the launcher choose; 1 (64 queries a workgroup), 2 (the same
-    with a query block's keys split over two wavefronts) or 3 (128 queries) asks for that shape of the LDS kernel."""
+    with a query block's keys split over two wavefronts) or 3 (128 queries) asks for that shape of the LDS kernel.
+    ``entry_len``: [E] int32 lengths that stand for the offsets' own; 0 leaves a portion out (its rows of ``out`` are
+    not written)."""
     _need(q, "q", torch.bfloat16)
     n = q.shape[0]
     _need(k_cache, "k cache", torch.bfloat16)
@@ -262,12 +278,14 @@ def attention_prefill(q: torch.Tensor, q_stride: int, k_cache: torch.Tensor, v_c
     entries = block_table.shape[0]
     _need(entry_start, "entry offsets", torch.int32, (entries + 1,))
     _need(entry_first_position, "entry first positions", torch.int32, (entries,))
+    if entry_len is not None:
+        _need(entry_len, "entry lengths", torch.int32, (entries,))
     _need(out, "attention out", torch.bfloat16, (n, nq * head_dim))
     if not 0 <= max_entry_len <= n:
         raise KernelError(f"attention_prefill: longest portion {max_entry_len} does not fit {n} tokens")
     _check(library().somi_attention_prefill(
         _ptr(q), ctypes.c_int64(q_stride), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), block_table.shape[1],
-        _ptr(entry_start), _ptr(entry_first_position), entries, max_entry_len, max(0, int(max_context)), int(shape), nq, nkv,
+        _ptr(entry_start), _ptr(entry_first_position), _ptr(entry_len), entries, max_entry_len, max(0, int(max_context)), int(shape), nq, nkv,
         head_dim, page_size, window, ctypes.c_float(scale), _ptr(out), _stream()))
 
 

@@ -186,6 +186,8 @@ def test_step_arrays_for_a_mixed_batch():
     assert table[0].tolist() == m.page_list(0, "p") and table[1].tolist() == m.page_list(0, "d")
     assert step.paged[0].slot_mapping.tolist() == m.slots(0, "p", 0, 6) + m.slots(0, "d", 5, 1)
     assert step.max_entry_len == 6 and step.max_context == 6
+    # no portion is longer than 8 tokens: every token is listed for the kernel that attends token by token
+    assert step.long_entry_len.tolist() == [0, 0] and step.short_tokens.tolist() == [0, 1, 2, 3, 4, 5, 6]
     assert all(t.dtype == torch.int32 for t in (step.token_ids, step.positions, table, step.logit_rows))
 
 

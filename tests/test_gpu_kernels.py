@@ -438,6 +438,16 @@ def test_attention_prefill_mfma_against_dense_softmax(nq, nkv, d, page, window, 
     torch.testing.assert_close(out.float().view(n, nq, d).cpu(), torch.cat(want), atol=2e-2, rtol=2e-2)
     plain_out = ops.paged_attention_plain(q, nq * d, kc, vc, block_table, i32(entry), i32(positions), nq, window, scale)
     torch.testing.assert_close(out.float(), plain_out.float(), atol=2e-2, rtol=2e-2)
+    # a mixed step: the long portions by this kernel, the short ones (two tokens, single tokens) token by token by
+    # the decode kernel with the keys of a request split over workgroups; one output tensor
+    mixed = torch.full((n, nq * d), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ops.attention_prefill(q, nq * d, kc, vc, block_table, i32(starts), i32(cached), max(new), nq, window, scale, mixed,
+                          shape=shape, entry_len=i32([k if k > 8 else 0 for k in new]))
+    short = [t for e, k in enumerate(new) if k <= 8 for t in range(starts[e], starts[e] + k)]
+    assert bool(torch.isnan(mixed[short].float()).all()) and not bool(torch.isnan(mixed[:starts[2]].float()).any())
+    ops.attention_decode(q, nq * d, kc, vc, block_table, i32(entry), i32(positions), nq, window, scale, 64, 3, mixed,
+                         token_list=i32(short))
+    torch.testing.assert_close(mixed.float(), plain_out.float(), atol=2e-2, rtol=2e-2)
 
 
 @pytest.mark.parametrize("m, inter, k", [(1, 48, 72), (8, 18944 // 8, 512), (17, 160, 200), (40, 4096 + 32, 64), (64, 32, 3584)])
