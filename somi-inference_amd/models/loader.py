@@ -45,11 +45,12 @@ def load_model(model_dir: str | os.PathLike, dtype: object = "bfloat16",
 
 
 def random_model(config: ModelConfig, seed: int, dtype: object = "bfloat16",
-                 device: str | torch.device = "cuda:0") -> DecoderModel:
-    """A model of seeded random weights drawn on the device (no folder is written)."""
+                 device: str | torch.device = "cuda:0", draw_on: str = "auto") -> DecoderModel:
+    """A model of seeded random weights (no folder is written).  Small models are drawn on the host and equal what
+    ``write_random_model`` writes for the seed; large ones are drawn on the device (see ``RandomSource``)."""
     arch = resolve_architecture(config.architecture)
     model = DecoderModel(arch.build_plan(config), make_runtime(dtype, device))
-    model.load(RandomSource(model.weight_specs(), seed))
+    model.load(RandomSource(model.weight_specs(), seed, draw_on=draw_on))
     return model
 
 

@@ -95,13 +95,35 @@ def random_tensor(spec: WeightSpec, seed: int, device: torch.device | str,
     return out.to(float_dtype)
 
 
-class RandomSource(WeightSource):
-    """Seeded random tensors made on demand on the target device (no file, no host copy)."""
+HOST_DRAW_ELEMENTS = 1 << 28      # models of up to this many weights are drawn on the host by default
 
-    def __init__(self, specs: list[WeightSpec], seed: int, stored: torch.dtype = torch.bfloat16) -> None:
+
+class RandomSource(WeightSource):
+    """Seeded random tensors made on demand (no file).
+
+    ``draw_on``: "host" draws with the host's generator, so the tensors equal those that
+    :func:`~somi_inference_amd.weights.write_random_model` writes for the same seed (a plain implementation can
+    read the same model from a folder); "device" draws on the target device without a host copy, which is what
+    models of tens of gigabytes need, and gives another (equally valid) model for the same seed.  "auto" takes
+    the host up to HOST_DRAW_ELEMENTS weights in all.
+    """
+
+    def __init__(self, specs: list[WeightSpec], seed: int, stored: torch.dtype = torch.bfloat16,
+                 draw_on: str = "auto") -> None:
         self._specs = {s.name: s for s in specs}
         self.seed = int(seed)
         self.stored = stored
+        if draw_on not in ("auto", "host", "device"):
+            raise ValueError(f"draw_on must be auto, host or device, got {draw_on!r}")
+        if draw_on == "auto":
+            total = 0
+            for s in specs:
+                count = 1
+                for dim in s.shape:
+                    count *= int(dim)
+                total += count
+            draw_on = "host" if total <= HOST_DRAW_ELEMENTS else "device"
+        self.draw_on = draw_on
 
     def names(self) -> list[str]:
         return list(self._specs)
@@ -113,6 +135,8 @@ class RandomSource(WeightSource):
         return torch.int32 if self._specs[name].role == TABLE else self.stored
 
     def read(self, name: str, device: torch.device | str) -> torch.Tensor:
+        if self.draw_on == "host":
+            return random_tensor(self._specs[name], self.seed, "cpu", self.stored).to(device)
         return random_tensor(self._specs[name], self.seed, device, self.stored)
 
 

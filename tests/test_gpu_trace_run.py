@@ -17,10 +17,11 @@ pytestmark = pytest.mark.gpu
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
-def run_trace(folder, dtype, out_dir, max_tokens, steps):
+def run_trace(folder, dtype, out_dir, max_tokens, steps, extra=()):
     lines = "".join(json.dumps(s) + "\n" for s in steps)
+    sizing = ["--max-tokens", str(max_tokens)] if max_tokens is not None else []
     done = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", dtype,
-                           "--out", str(out_dir), "--max-tokens", str(max_tokens)],
+                           "--out", str(out_dir), *sizing, *extra],
                           input=lines, capture_output=True, text=True, timeout=600, cwd="/")
     assert done.returncode == 0, done.stderr[-3000:]
     assert done.stdout.split() == [w for s in steps for w in ("done", str(s["step"]))]
@@ -69,8 +70,16 @@ def test_replay_whole_decoded_in_portions_and_mixed(name, dtype, model_folders, 
         at += size
         k += 1
         number += 1
+    # the configuration's own page size: 16 for A (the program's default), 8 for B
+    page = TINY[name]["block_size"]
+    extra = [] if page == 16 else ["--block-size", str(page)]
     out1 = tmp_path / "single"
-    run_trace(folder, dtype, out1, round64(len(c)), steps)
+    run_trace(folder, dtype, out1, round64(len(c)), steps, extra)
+    header = json.loads((out1 / "0.json").read_text())
+    assert header["shape"] == [len(a), vocab] and header["block_size"] == page and header["dtype"] == "float32"
+    assert header["rows"][3] == {"id": "whole", "place": 3, "position": 3}
+    last = json.loads((out1 / f"{number - 1}.json").read_text())
+    assert last["rows"][-1]["position"] == len(c) - 1
     for step, logits in expect.items():
         assert_close(read_logits(out1, step, vocab), logits, dtype, f"{name} {dtype} step {step}")
     assert not os.path.exists(out1 / "999.f32")
@@ -96,7 +105,30 @@ def test_replay_whole_decoded_in_portions_and_mixed(name, dtype, model_folders, 
         if sum(r.shape[0] for r in rows):
             expect[number] = torch.cat(rows)
     out2 = tmp_path / "mixed"
-    run_trace(folder, dtype, out2, peak, steps)
+    run_trace(folder, dtype, out2, peak, steps, extra)
     for step, logits in expect.items():
         assert_close(read_logits(out2, step, vocab), logits, dtype, f"{name} {dtype} mixed step {step}")
     assert sorted(int(f[:-4]) for f in os.listdir(out2) if f.endswith(".f32")) == sorted(expect)
+
+
+def test_replay_of_seeded_random_weights_with_the_pool_given_in_pages(tmp_path):
+    """--model random:<config.json>:<seed> draws the weights that the random-weights mode writes for that seed, and
+    --num-blocks sizes the pool in pages: the logits equal the plain implementation's on the written folder."""
+    from somi_inference_amd.weights import write_random_model
+    config, seed = TINY["A"]["config"], 77
+    folder = write_random_model(str(tmp_path / "written"), config, seed=seed)
+    cfg, weights = plain.read_model(folder)
+    tokens = token_ids(config.vocab_size, 40, 5)
+    want = plain.model_logits(cfg, weights, tokens)
+    steps = [{"step": 0, "entries": [{"id": "r", "tokens": tokens[:29], "want": [28]}], "end": []},
+             {"step": 1, "entries": [{"id": "r", "tokens": tokens[29:], "want": list(range(11))}], "end": ["r"]}]
+    out = tmp_path / "out"
+    run_trace(f"random:{folder}/config.json:{seed}", "float32", out, None, steps, ["--num-blocks", "3", "--block-size", "16"])
+    assert_close(read_logits(out, 0, config.vocab_size), want[28:29], "float32", "random weights, step 0")
+    assert_close(read_logits(out, 1, config.vocab_size), want[29:], "float32", "random weights, step 1")
+    # two pages would not hold 40 tokens
+    lines = "".join(json.dumps(s) + "\n" for s in steps)
+    failed = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", f"random:{folder}:{seed}",
+                             "--dtype", "float32", "--out", str(tmp_path / "small"), "--num-blocks", "2"],
+                            input=lines, capture_output=True, text=True, timeout=600, cwd="/")
+    assert failed.returncode != 0 and "pages" in failed.stderr
