@@ -2,8 +2,8 @@
 
 ``python bench.py --gpus 1 --steps K --warmup W`` builds a random-weights model of the 7B layer
 sizes in bfloat16, fills the cache of ``--batch`` requests by running their prompts through the
-engine's own step function, then times exactly K decode steps (one token per request per step:
-model step plus greedy sampling) between two synchronisations.  It prints ONE JSON line; ``value``
+engine's own generation loop (scheduler, step function, sampler), then times exactly K of that loop's
+decode steps (one token per request per step) between two synchronisations.  It prints ONE JSON line; ``value``
 is decoded tokens per second.  The same line carries a 2,048-token prefill measurement, the decode
 step's HBM roofline figures and decode throughput at batch 1 and 64.
 
@@ -55,10 +55,76 @@ def parse_args() -> argparse.Namespace:
     p.add_argument("--seed", type=int, default=0)
     p.add_argument("--no-points", action="store_true", help="skip the batch 1 / batch 64 decode points")
     p.add_argument("--no-prefill", action="store_true", help="skip the prefill measurement")
+    p.add_argument("--no-peaks", action="store_true", help="skip the measurement of the machine's own peaks")
+    p.add_argument("--output-file", type=str, default=None, help="Append the result line to a JSONL file.")
     p.add_argument("--serving", type=int, default=0, metavar="REQUESTS",
                    help="also run this many requests (prompts of 128 to 2,048 tokens, 256 new tokens each) through "
                         "the scheduler with portions of 512, and report it under 'serving'")
     return p.parse_args()
+
+
+def summarize_ms(samples_ms: list[float]) -> dict:
+    """Mean, median, tail, spread and range of latency samples, as the reference summarises them
+    (benchmarks/common.py:159-170)."""
+    import numpy as np
+    x = np.asarray(samples_ms, dtype=np.float64)
+    return {"mean": round(float(x.mean()), 4), "median": round(float(np.percentile(x, 50)), 4),
+            "p95": round(float(np.percentile(x, 95)), 4), "p99": round(float(np.percentile(x, 99)), 4),
+            "std": round(float(x.std()), 4), "min": round(float(x.min()), 4), "max": round(float(x.max()), 4)}
+
+
+def environment(device) -> dict:
+    """Where the numbers come from (the reference's collect_environment_metadata, benchmarks/common.py:231-251)."""
+    import platform
+    import subprocess
+
+    import torch
+
+    def git(*args: str) -> str | None:
+        try:
+            done = subprocess.run(["git", *args], cwd=ROOT, capture_output=True, text=True, timeout=10)
+            return done.stdout.strip() if done.returncode == 0 else None
+        except (OSError, subprocess.SubprocessError):
+            return None
+
+    props = torch.cuda.get_device_properties(device)
+    dirty = git("status", "--porcelain")
+    return {"git_sha": git("rev-parse", "HEAD"), "git_dirty": bool(dirty) if dirty is not None else None,
+            "python_version": platform.python_version(), "platform": platform.platform(),
+            "torch_version": torch.__version__, "hip_version": torch.version.hip,
+            "device_name": props.name, "device_arch": getattr(props, "gcnArchName", None),
+            "compute_units": props.multi_processor_count, "device_memory_gb": round(props.total_memory / 2**30, 1),
+            "executable": sys.executable}
+
+
+def measure_peaks(device) -> dict:
+    """What this machine reaches on the two resources the step is bound by: streaming memory into the compute units
+    (2 GiB, beyond every cache) and bfloat16 matrix instructions on every SIMD."""
+    import torch
+
+    from somi_inference_amd.kernels import ops
+    buffer = torch.empty(2 << 30, dtype=torch.uint8, device=device)
+    buffer.zero_()
+
+    def timed(fn, reps):
+        fn()
+        torch.cuda.synchronize()
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(reps):
+            fn()
+        end.record()
+        torch.cuda.synchronize()
+        return start.elapsed_time(end) / reps / 1000.0
+    read_s = timed(lambda: ops.probe_stream_read(buffer), 5)
+    flops = ops.probe_mfma(20000, device)
+    mfma_s = timed(lambda: ops.probe_mfma(20000, device), 3)
+    del buffer
+    return {"stream_read_gbs": round(buffer_bytes_gb(2 << 30) / read_s, 1), "mfma_bf16_tflops": round(flops / mfma_s / 1e12, 1)}
+
+
+def buffer_bytes_gb(n: int) -> float:
+    return n / 1e9
 
 
 def main() -> int:
@@ -72,7 +138,7 @@ def main() -> int:
     import torch
 
     from somi_inference_amd.config import Qwen2Config
-    from somi_inference_amd.engine import StepEntry
+    from somi_inference_amd.engine import Engine, Request, Scheduler, StepEntry
     from somi_inference_amd.models import make_runner, random_model
     from somi_inference_amd.sampling import Sampler, SamplingParams
 
@@ -83,10 +149,16 @@ def main() -> int:
                          head_dim=head_dim, rope_theta=1e6, rms_norm_eps=eps, tie_word_embeddings=tied,
                          max_position_embeddings=32768)
     torch.manual_seed(args.seed)
-    model = random_model(config, seed=args.seed, dtype=args.dtype)
+    device = torch.device("cuda:0")
+    model = random_model(config, seed=args.seed, dtype=args.dtype, draw_on="device")
     elem = 2 if args.dtype == "bfloat16" else 4
     batches = [args.batch] if args.no_points else sorted({1, args.batch, 64})
-    pages_per_request = (args.context + args.block_size - 1) // args.block_size + 1
+    # Decoding is measured through the generation loop itself (scheduler, step function, sampler, running ahead of
+    # the device).  The scheduler runs the prompts in portions of 2,048 tokens and lets the requests that are done
+    # with theirs decode meanwhile, so a request has decoded up to `ramp` tokens before the timed steps begin.
+    portion = 2048
+    ramp = max(batches) * ((args.context + portion - 1) // portion) + 8
+    pages_per_request = (args.context + ramp + args.block_size - 1) // args.block_size + 1
     num_blocks = max(max(batches) * pages_per_request,
                      (args.prefill_tokens + args.block_size - 1) // args.block_size + 1)
     runner = make_runner(model, block_size=args.block_size, num_blocks=num_blocks, max_requests=max(batches) + 1)
@@ -99,61 +171,56 @@ def main() -> int:
     def sync() -> None:
         torch.cuda.synchronize()
 
-    def decode_run(batch: int, steps: int, warmup: int) -> tuple[float, float]:
-        """Fill ``batch`` requests up to context - (warmup + steps), then time ``steps`` decode steps.
-        Returns (seconds, mean context length during the timed steps)."""
+    def decode_run(batch: int, steps: int, warmup: int) -> dict:
+        """``batch`` requests whose prompts end ``warmup + steps`` tokens before the context length, run by the
+        engine; times ``steps`` of its decode steps.  Every step is one scheduling decision, one model step for all
+        requests and one sampling call, launched ahead of the device as generation does it."""
+        scheduler = Scheduler(runner.cache, max_concurrent=batch, max_num_batched_tokens=max(portion, batch), chunk=portion)
+        engine = Engine(runner, scheduler, sampler, eos_token_id=-1)
         prompt_len = args.context - (warmup + steps + 1)
-        ids = [f"b{batch}_{i}" for i in range(batch)]
-        for rid in ids:
-            runner.begin(rid)
-            tokens = torch.randint(0, config.vocab_size, (prompt_len,), generator=gen).tolist()
-            for at in range(0, prompt_len, 2048):
-                runner.step([StepEntry(rid, tokens[at:at + 2048], [])])
-        last = torch.randint(0, config.vocab_size, (batch,), generator=gen).tolist()
-
-        placeholders = [StepEntry(rid, [0], [0]) for rid in ids]
-
-        def launch(previous):
-            """One decode step and its greedy pick, launched without waiting: the step takes the previous
-            pick straight from the device; the host reads every pick one step late."""
-            if isinstance(previous, list):
-                logits = runner.step([StepEntry(rid, [tok], [0]) for rid, tok in zip(ids, previous)])
-            else:
-                logits = runner.step(placeholders, device_tokens=previous.device)
-            return sampler.sample_async(logits, greedy)
-
-        newest = launch(last)
+        requests = [Request(f"b{batch}_{i}", torch.randint(0, config.vocab_size, (prompt_len,), generator=gen).tolist(),
+                            ramp + warmup + steps + 8, greedy, seed=i) for i in range(batch)]
+        runner.capture_decode_graphs(batch, args.context + ramp)
+        for request in requests:
+            engine.add_request(request)
+        while scheduler.waiting or any(r.num_computed < len(r.prompt_tokens) for r in requests):
+            engine.step()
         for _ in range(warmup):
-            older, newest = newest, launch(newest)
-            older.tolist()
+            engine.step()
         sync()
+        cached_before = sum(runner.cache.num_tokens(r.request_id) for r in requests)
+        marks = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
+        marks[0].record()
         start = time.perf_counter()
-        for _ in range(steps):
-            older, newest = newest, launch(newest)
-            older.tolist()
+        for i in range(steps):
+            engine.step()
+            marks[i + 1].record()
         sync()
         seconds = time.perf_counter() - start
-        for rid in ids:
-            runner.end(rid)
-        return seconds, args.context - steps / 2.0
+        cached_after = sum(runner.cache.num_tokens(r.request_id) for r in requests)
+        assert cached_after - cached_before == batch * steps, "a timed step was not a decode step of every request"
+        step_ms = [marks[i].elapsed_time(marks[i + 1]) for i in range(steps)]
+        engine.abort(requests)
+        return dict(tok_s=batch * steps / seconds, ms=1000.0 * seconds / steps, steps=steps, warmup=warmup,
+                    mean_ctx=(cached_before + cached_after) / 2.0 / batch, step_ms=step_ms,
+                    run_ahead=engine.steps_run_ahead)
 
     results = {}
     for batch in batches:
         steps = args.steps if batch == args.batch else max(8, args.steps // 2)
         warmup = args.warmup if batch == args.batch else max(2, args.warmup // 2)
-        seconds, mean_ctx = decode_run(batch, steps, warmup)
-        results[batch] = dict(tok_s=batch * steps / seconds, ms=1000.0 * seconds / steps, steps=steps,
-                              warmup=warmup, mean_ctx=mean_ctx)
+        results[batch] = decode_run(batch, steps, warmup)
 
     main_run = results[args.batch]
     step_bytes = weight_bytes + args.batch * main_run["mean_ctx"] * kv_bytes_per_token
     achieved = step_bytes / (main_run["ms"] / 1000.0) / 1e9
+    peaks = None if args.no_peaks else measure_peaks(device)
 
     prefill = None
     if not args.no_prefill:
         tokens = torch.randint(0, config.vocab_size, (args.prefill_tokens,), generator=gen).tolist()
         times = []
-        for rep in range(4):
+        for rep in range(6):
             runner.begin("prefill")
             sync()
             start = time.perf_counter()
@@ -161,18 +228,20 @@ def main() -> int:
             sync()
             times.append(time.perf_counter() - start)
             runner.end("prefill")
-        seconds = min(times[1:])
+        times = sorted(times[1:])                     # the first run pays one-time set-up
+        seconds = times[len(times) // 2]              # the median of five
         flops = _prefill_flops(config, args.prefill_tokens)
         prefill = {"value": round(args.prefill_tokens / seconds, 1), "tokens": args.prefill_tokens,
-                   "ms": round(seconds * 1000.0, 3), "frac": round(flops / seconds / PEAK_FLOPS[args.dtype], 4)}
+                   "ms": round(seconds * 1000.0, 3), "frac": round(flops / seconds / PEAK_FLOPS[args.dtype], 4),
+                   "ms_min": round(times[0] * 1000.0, 3), "ms_max": round(times[-1] * 1000.0, 3)}
+        if peaks is not None and args.dtype == "bfloat16":
+            prefill["frac_of_measured_mfma"] = round(flops / seconds / (peaks["mfma_bf16_tflops"] * 1e12), 4)
 
     serving = None
     if args.serving > 0:
         # continuous batching through the engine's own scheduler: everything arrives at once, prompts are cut
         # into portions of 512 under a budget of 2,048 tokens a step, finished requests free their pages
         from collections import deque
-
-        from somi_inference_amd.engine import Engine, Request, Scheduler
         lengths = torch.randint(128, 2049, (args.serving,), generator=gen).tolist()
         new_tokens = 256
         # the pool made for the decode runs serves here too; at most as many requests at once as fit whole
@@ -196,6 +265,11 @@ def main() -> int:
                    "steps_run_ahead": engine.steps_run_ahead, "max_concurrent": concurrent,
                    "preemptions": sum(r.num_preemptions for r in done), "graphs_captured_ahead": captured}
 
+    roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": round(achieved / HBM_PEAK_GBS, 4)}
+    if peaks is not None:
+        roofline["measured_peak"] = peaks["stream_read_gbs"]
+        roofline["frac_of_measured"] = round(achieved / peaks["stream_read_gbs"], 4)
     line = {
         "metric": f"decode tok/s at batch {args.batch}, Qwen2.5-{args.sizes.upper()} layer sizes "
                   f"(plus prefill tok/s at {args.prefill_tokens:,} tokens, batch 1/64 points)",
@@ -203,23 +277,32 @@ def main() -> int:
         "steps": main_run["steps"], "warmup": main_run["warmup"], "ms_per_step": round(main_run["ms"], 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
-        "data": "synthetic: seeded random N(0,0.02) weights, seeded uniform token ids; caches filled by running the prompts",
+        "data": "synthetic: seeded random N(0,0.02) weights, seeded uniform token ids; prompts run and tokens decoded "
+                "by the engine's own generation loop",
         "config": {"model": f"Qwen2.5-{args.sizes.upper()} layer sizes (random weights)", "global_batch": args.batch,
                    "seq_len": args.context, "parallelism": "single GPU", "layers": layers,
                    "layers_of_config": full_layers, "hidden_size": config.hidden_size,
                    "intermediate_size": config.intermediate_size, "num_attention_heads": config.num_attention_heads,
                    "num_key_value_heads": config.num_key_value_heads, "head_dim": config.head_dim,
                    "vocab_size": config.vocab_size, "tie_word_embeddings": tied, "block_size": args.block_size,
-                   "context_at_end": args.context},
-        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4)},
+                   "mean_context": round(main_run["mean_ctx"], 1)},
+        "roofline": roofline,
+        "latency_ms": summarize_ms(main_run["step_ms"]),
         "points": {f"decode_b{b}": round(r["tok_s"], 2) for b, r in results.items() if b in (1, 64)},
     }
     if prefill is not None:
         line["prefill"] = prefill
     if serving is not None:
         line["serving"] = serving
-    print(json.dumps(line))
+    if peaks is not None:
+        line["measured_peaks"] = peaks
+    line["environment"] = environment(device)
+    text = json.dumps(line)
+    print(text)
+    if args.output_file:
+        os.makedirs(os.path.dirname(os.path.abspath(args.output_file)), exist_ok=True)
+        with open(args.output_file, "a", encoding="utf-8") as handle:      # appended, as the reference's runs are
+            handle.write(text + "\n")
     return 0
 
 

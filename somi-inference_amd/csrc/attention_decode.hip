@@ -463,6 +463,13 @@ attention_combine_kernel(const float* __restrict__ part_acc, const float* __rest
     }
 }
 
+// The longest range of keys (a multiple of 64) that one workgroup of the kernel that stages tiles through LDS takes
+// for this page size: its list of pages is in LDS.  Longer splits run the slower kernel that keeps tiles in registers.
+extern "C" int somi_attention_decode_lds_split(int page_size) {
+    if (page_size <= 0) return 0;
+    return (DECODE_LDS_PAGES - 2 - 8) * page_size / 64 * 64;
+}
+
 template <int DT>
 static int launch_decode(const void* q, int64_t q_stride, const void* kc, const void* vc, const int* block_table,
                          int max_blocks, const int* token_list, const int* token_entry, const int* positions,

@@ -576,3 +576,22 @@ def sample_filter(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.
     _need(top_p, "top_p", torch.float32, (rows,))
     _check(library().somi_sample_filter(_ptr(logits), rows, vocab, _ptr(temperature), _ptr(top_k), _ptr(top_p),
                                         _stream()))
+
+
+def probe_stream_read(buffer: torch.Tensor) -> None:
+    """Streams ``buffer`` (any dtype, contiguous, a multiple of 16 bytes) once through the compute units: the
+    time of this call is what reading that many bytes costs on this machine."""
+    _need(buffer, "probe buffer")
+    size = buffer.numel() * buffer.element_size()
+    lib = library()
+    sink = torch.zeros((lib.somi_probe_stream_blocks(),), dtype=torch.int32, device=buffer.device)
+    _check(lib.somi_probe_stream_read(_ptr(buffer), ctypes.c_int64(size), _ptr(sink), _stream()))
+
+
+def probe_mfma(iters: int, device: torch.device | str = "cuda:0") -> float:
+    """Runs ``iters`` rounds of four bfloat16 32 x 32 x 16 matrix instructions on every wavefront slot the launch
+    fills (two per SIMD); returns the flops the launch does."""
+    sink = torch.zeros((1,), dtype=torch.float32, device=device)
+    flops = ctypes.c_double(0.0)
+    _check(library().somi_probe_mfma(int(iters), _ptr(sink), ctypes.byref(flops), _stream()))
+    return float(flops.value)
