@@ -20,6 +20,16 @@
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
 typedef __attribute__((ext_vector_type(4))) short short4_t;
+
+// Four values (keys vpos .. vpos + 3 of one channel) with those outside [lo, hi] set to zero.  A masked key has the
+// weight 0, but 0 x NaN is NaN: what lies beyond a request's tokens in a page that is used again, or before its
+// window, must not reach the products, whatever it holds.
+__device__ __forceinline__ short4_t keep_visible(short4_t v, int vpos, int lo, int hi) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+        if (vpos + e < lo || vpos + e > hi) v[e] = 0;
+    return v;
+}
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 
 __device__ __forceinline__ bf16x8 ld8(const bf16* p) { return *reinterpret_cast<const bf16x8*>(p); }
@@ -100,6 +110,10 @@ attention_decode_kernel(const bf16* __restrict__ q, int64_t q_stride, const bf16
             if (DT & 1) kf[QK_STEPS - 1] = half_step(krow + (DT - 1) * 16 + g * 4);
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) vf[dt] = ld4(vbase + (int64_t)(dt * 16 + r) * page_size);
+            if (vpos == vlo || vpos == vhi) {          // the groups that hold the first and the last visible key
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) vf[dt] = keep_visible(vf[dt], vpos, begin, end);
+            }
             f32x4 s = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int c = 0; c < QK_STEPS; ++c) s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[c], qf[c], s, 0, 0, 0);
@@ -292,6 +306,10 @@ attention_decode_lds_kernel(const bf16* __restrict__ q, int64_t q_stride, const 
             for (int i = 0; i < V_PER_THREAD; ++i) {
                 const int d = (tid >> 3) + 32 * i;
                 if (D % 32 == 0 || d < D) vreg[i] = ld4(vbase + (int64_t)d * page_size);
+            }
+            if (vpos == vlo || vpos == vhi) {          // the groups that hold the first and the last visible key
+#pragma unroll
+                for (int i = 0; i < V_PER_THREAD; ++i) vreg[i] = keep_visible(vreg[i], vpos, begin, end);
             }
         };
         auto stash = [&](const bf16x8 (&kreg)[K_PER_THREAD], const short4_t (&vreg)[V_PER_THREAD], int buf) {

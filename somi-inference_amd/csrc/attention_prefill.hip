@@ -22,6 +22,16 @@
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
 typedef __attribute__((ext_vector_type(4))) short short4_t;
+
+// Four values (keys vpos .. vpos + 3 of one channel) with those outside [lo, hi] set to zero.  A masked key has the
+// weight 0, but 0 x NaN is NaN: what lies beyond a request's tokens in a page that is used again, or before its
+// window, must not reach the products, whatever it holds.
+__device__ __forceinline__ short4_t keep_visible(short4_t v, int vpos, int lo, int hi) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+        if (vpos + e < lo || vpos + e > hi) v[e] = 0;
+    return v;
+}
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 
 __device__ __forceinline__ bf16x8 pld8(const bf16* p) { return *reinterpret_cast<const bf16x8*>(p); }
@@ -141,9 +151,13 @@ attention_prefill_kernel(const bf16* __restrict__ q, int64_t q_stride, const bf1
             const bf16* vbase_a = vc + (pa * nkv + kvh) * (int64_t)D * page_size + va % page_size;
             const bf16* vbase_b = vc + (pb * nkv + kvh) * (int64_t)D * page_size + vb % page_size;
 #pragma unroll
-            for (int dt = 0; dt < DT; ++dt)
-                vf[dt] = pjoin(pld4(vbase_a + (int64_t)(dt * 16 + r) * page_size),
-                               pld4(vbase_b + (int64_t)(dt * 16 + r) * page_size));
+            for (int dt = 0; dt < DT; ++dt) {
+                short4_t a4 = pld4(vbase_a + (int64_t)(dt * 16 + r) * page_size);
+                short4_t b4 = pld4(vbase_b + (int64_t)(dt * 16 + r) * page_size);
+                if (va == vlo || va == vhi) a4 = keep_visible(a4, va, lo, p_last);     // the first and the last visible key's groups
+                if (vb == vlo || vb == vhi) b4 = keep_visible(b4, vb, lo, p_last);
+                vf[dt] = pjoin(a4, b4);
+            }
         }
 #pragma unroll
         for (int qb = 0; qb < QB; ++qb) {
@@ -354,6 +368,10 @@ attention_prefill_lds_kernel(const bf16* __restrict__ q, int64_t q_stride, const
             for (int i = 0; i < V_PER_THREAD; ++i) {
                 const int d = (tid256 >> 3) + 32 * i;
                 if (D % 32 == 0 || d < D) vreg[i] = pld4(vbase + (int64_t)d * page_size);
+            }
+            if (vpos == vlo || vpos == vhi) {          // the groups that hold the first and the last visible key
+#pragma unroll
+                for (int i = 0; i < V_PER_THREAD; ++i) vreg[i] = keep_visible(vreg[i], vpos, lo, wg_last);
             }
         }
     };

@@ -696,3 +696,67 @@ def test_many_rows_product_into_the_residual_stream(m, n, k, tile):
         normed = norm_w * want_h * torch.rsqrt(want_h.pow(2).mean(1, keepdim=True) + eps)
         want = normed @ w2.float().t()
         torch.testing.assert_close(got.float(), want, atol=0.02 * float(want.abs().max()), rtol=2e-2)
+
+
+@pytest.mark.parametrize("nq, nkv, d, page, window", [(8, 2, 64, 16, 0), (6, 3, 128, 16, 21), (4, 1, 32, 8, 0), (14, 2, 256, 16, 0),
+                                                     (5, 5, 80, 4, 9)])
+def test_attention_ignores_whatever_lies_beyond_a_requests_keys(nq, nkv, d, page, window):
+    """Pages are handed out again without being cleared, and pages a window has passed read as page 0.  Everything
+    in the cache that is not a visible key of the request is NaN here (the tail of its last page, every other
+    page, the pages below the window): a masked key has the weight 0, but 0 x NaN is NaN, so the kernels must not
+    let such a value reach a product.  Decode (with the keys split) and prefill (every launch shape), MFMA and
+    plain kernels."""
+    cached, new = [37, 150, 0, 77], [1, 1, 70, 12]
+    total = [c + n for c, n in zip(cached, new)]
+    n_pages = sum((t + page - 1) // page for t in total) + 2
+    perm = torch.randperm(n_pages - 1, generator=torch.Generator().manual_seed(6)).add(1).tolist()     # page 0 stays poisoned
+    tables, at = [], 0
+    for t in total:
+        count = (t + page - 1) // page
+        tables.append(perm[at:at + count])
+        at += count
+    kc = torch.full((n_pages, nkv, page, d), float("nan"), dtype=torch.bfloat16, device=DEV)
+    vc = torch.full((n_pages, nkv, d, page), float("nan"), dtype=torch.bfloat16, device=DEV)
+    keys = [rnd(t, nkv, d, dtype="bfloat16", seed=30 + i) for i, t in enumerate(total)]
+    values = [rnd(t, nkv, d, dtype="bfloat16", seed=40 + i) for i, t in enumerate(total)]
+    for r, t in enumerate(total):
+        first_kept = 0
+        if window:
+            # a page wholly below the window of the request's first new token has been given back: page 0
+            first_kept = max(0, cached[r] - window + 1) // page
+            tables[r] = [0] * first_kept + tables[r][first_kept:]
+        for pos in range(first_kept * page, t):
+            kc[tables[r][pos // page], :, pos % page] = keys[r][pos]
+            vc[tables[r][pos // page], :, :, pos % page] = values[r][pos]
+    width = max(len(t) for t in tables)
+    block_table = i32([t + [0] * (width - len(t)) for t in tables])
+    n = sum(new)
+    q = rnd(n, nq * d, dtype="bfloat16", seed=7, scale=2.0)
+    positions, entry, starts = [], [], [0]
+    for e, (c, k) in enumerate(zip(cached, new)):
+        positions += [c + i for i in range(k)]
+        entry += [e] * k
+        starts.append(starts[-1] + k)
+    scale = d ** -0.5
+    qh = q.float().view(n, nq, d).cpu()
+    want, at = [], 0
+    for e, k in enumerate(new):
+        want.append(dense_attention_reference(qh[at:at + k], keys[e].float().cpu(), values[e].float().cpu(),
+                                              positions[at:at + k], cached[e], window, scale))
+        at += k
+    want = torch.cat(want).view(n, nq * d)
+    plain_out = ops.paged_attention_plain(q, nq * d, kc, vc, block_table, i32(entry), i32(positions), nq, window, scale)
+    assert bool(torch.isfinite(plain_out.float()).all()), "the plain kernel let a value from outside the visible keys through"
+    torch.testing.assert_close(plain_out.float().cpu(), want, atol=2e-2, rtol=2e-2)
+    for shape in (0, 1, 2, 3):
+        out = torch.full((n, nq * d), float("nan"), dtype=torch.bfloat16, device=DEV)
+        ops.attention_prefill(q, nq * d, kc, vc, block_table, i32(starts), i32(cached), max(new), nq, window, scale, out,
+                              shape=shape)
+        assert bool(torch.isfinite(out.float()).all()), f"prefill shape {shape}: not finite"
+        torch.testing.assert_close(out.float().cpu(), want, atol=2e-2, rtol=2e-2)
+    for split_len, splits in ((64, 4), (256, 1), (16, 15)):
+        out = torch.full((n, nq * d), float("nan"), dtype=torch.bfloat16, device=DEV)
+        ops.attention_decode(q, nq * d, kc, vc, block_table, i32(entry), i32(positions), nq, window, scale, split_len,
+                             splits, out)
+        assert bool(torch.isfinite(out.float()).all()), f"decode splits of {split_len}: not finite"
+        torch.testing.assert_close(out.float().cpu(), want, atol=2e-2, rtol=2e-2)
