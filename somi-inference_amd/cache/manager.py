@@ -7,13 +7,16 @@ one allocator, one tensor per layer, per-sequence page lists and token counts;
 (:202-221, :294-296); ``free_sequence`` returns every page (:195-200); a
 duplicate ``register_sequence`` raises "already registered" (:150-156).
 
-Beyond the reference: layers are put into *groups* by what they need.  Layers
-that keep every key share one page pool and one block table per request; layers
-that see a window of keys form a group of their own whose pages are released as
-soon as the window has passed them, while the request is still live.  Mixers
-with fixed-size state get one slot per request in a state tensor (this
-architecture has none; the slot is assigned all the same so nothing changes
-when one is added).
+Beyond the reference: a layer says what it keeps per token (a ``PagedSpec``: the
+tensors of a page, a window, a page size of its own if its kernels want one) and
+layers are put into *groups* by window and page size.  The layers of a group
+share one page pool and one block table per request; each has tensors of its own,
+allocated as its spec lists them.  A group with a window releases a page as soon
+as the window has passed it, while the request is still live.  Every group's pool
+holds the same number of tokens, ``num_blocks * block_size``, cut into pages of
+the group's size.  Mixers with fixed-size state get one slot per request in a
+state tensor (this architecture has none; the slot is assigned all the same so
+nothing changes when one is added).
 """
 
 from __future__ import annotations
@@ -24,7 +27,7 @@ from typing import Hashable
 import numpy as np
 import torch
 
-from ..parts.base import FixedStateSpec, LayerCache, PagedKVSpec
+from ..parts.base import FixedStateSpec, LayerCache, PagedSpec
 from .pool import CacheError, OutOfPages, PagePool
 
 RELEASED = -1     # host-side mark of a logical page a window has passed
@@ -34,6 +37,7 @@ RELEASED = -1     # host-side mark of a logical page a window has passed
 class PagedGroup:
     window: int | None
     pool: PagePool
+    page_size: int = 0
     runs: list[int] = field(default_factory=list)      # layer runs whose tensors use this group's page ids
 
 
@@ -57,31 +61,36 @@ class RequestCache:
 
 
 class CacheManager:
-    def __init__(self, needs: list[PagedKVSpec | FixedStateSpec | int | None], *, block_size: int,
+    def __init__(self, needs: list[PagedSpec | FixedStateSpec | int | None], *, block_size: int,
                  num_blocks: int, max_requests: int, dtype: torch.dtype, device: torch.device | str,
                  allocate_tensors: bool = True) -> None:
+        """``block_size``: tokens per page where a spec names no page size of its own.  ``num_blocks``: pages of
+        that size per group; a group with another page size gets as many pages as hold the same tokens."""
         if block_size < 1 or num_blocks < 1 or max_requests < 1:
             raise ValueError("block_size, num_blocks and max_requests must be >= 1")
         self.block_size, self.num_blocks, self.max_requests = int(block_size), int(num_blocks), int(max_requests)
         self.dtype, self.device = dtype, torch.device(device)
         self.groups: list[PagedGroup] = []
         self.layer_caches: list[LayerCache | None] = [None] * len(needs)
-        by_window: dict[int | None, int] = {}
+        by_need: dict[tuple[int | None, int], int] = {}
         for run, need in enumerate(needs):
-            if isinstance(need, PagedKVSpec):
-                if need.window not in by_window:
-                    by_window[need.window] = len(self.groups)
-                    self.groups.append(PagedGroup(need.window, PagePool(self.num_blocks)))
-                group = by_window[need.window]
+            if isinstance(need, PagedSpec):
+                page_size = int(need.page_size or self.block_size)
+                key = (need.window, page_size)
+                if key not in by_need:
+                    pages = self.pool_tokens // page_size
+                    if pages < 1:
+                        raise ValueError(f"a pool of {self.pool_tokens} tokens holds no page of {page_size}")
+                    by_need[key] = len(self.groups)
+                    self.groups.append(PagedGroup(need.window, PagePool(pages), page_size))
+                group = by_need[key]
                 self.groups[group].runs.append(run)
-                k = v = None
+                tensors = {}
                 if allocate_tensors:
-                    # V is transposed inside a page: consecutive positions of one channel are adjacent
-                    k = torch.zeros((self.num_blocks, need.num_kv_heads, self.block_size, need.head_dim),
-                                    dtype=dtype, device=self.device)
-                    v = torch.zeros((self.num_blocks, need.num_kv_heads, need.head_dim, self.block_size),
-                                    dtype=dtype, device=self.device)
-                self.layer_caches[run] = LayerCache(need, group, k=k, v=v)
+                    pages = self.groups[group].pool.num_pages
+                    tensors = {t.name: torch.zeros((pages, *t.page_shape(page_size)), dtype=t.dtype or dtype,
+                                                   device=self.device) for t in need.tensors}
+                self.layer_caches[run] = LayerCache(need, group, tensors=tensors, page_size=page_size)
             elif isinstance(need, FixedStateSpec):
                 state = None
                 if allocate_tensors:
@@ -93,18 +102,25 @@ class CacheManager:
                 source = self.layer_caches[need]
                 if source is None:
                     raise CacheError(f"run {run} reads the cache of run {need}, which has none")
-                self.layer_caches[run] = LayerCache(source.spec, source.group, k=source.k, v=source.v,
-                                                    state=source.state, writes=False)
+                self.layer_caches[run] = LayerCache(source.spec, source.group, tensors=source.tensors,
+                                                    state=source.state, writes=False, page_size=source.page_size)
         self._requests: dict[Hashable, RequestCache] = {}
         self._free_slots = list(range(self.max_requests - 1, -1, -1))
         self.padding_state_slot = self.max_requests       # never handed to a request
 
+    @property
+    def pool_tokens(self) -> int:
+        """Tokens that each group's pool holds."""
+        return self.num_blocks * self.block_size
+
     @staticmethod
     def page_bytes(needs: list, block_size: int, dtype: torch.dtype) -> int:
-        """Bytes of device memory that one more page per group costs: keys and values of every run that writes."""
-        item = torch.empty((), dtype=dtype).element_size()
-        return sum(2 * need.num_kv_heads * need.head_dim * int(block_size) * item
-                   for need in needs if isinstance(need, PagedKVSpec))
+        """Bytes of device memory that ``block_size`` more tokens per group cost: every tensor of every run that
+        writes (a group with pages of another size holds the same tokens in other pages)."""
+        def item(kind: torch.dtype | None) -> int:
+            return torch.empty((), dtype=kind or dtype).element_size()
+        return sum(t.elements_per_token() * int(block_size) * item(t.dtype)
+                   for need in needs if isinstance(need, PagedSpec) for t in need.tensors)
 
     # --------------------------------------------------------------- requests
     def has(self, request_id: Hashable) -> bool:
@@ -147,14 +163,25 @@ class CacheManager:
         return self._get(request_id).state_slot
 
     # ------------------------------------------------------------------ pages
-    def _pages_for(self, length: int) -> int:
-        return (length + self.block_size - 1) // self.block_size
+    def _pages_for(self, group: PagedGroup, length: int) -> int:
+        return (length + group.page_size - 1) // group.page_size
+
+    def holds(self, tokens: int) -> bool:
+        """Whether a request of this many tokens fits the pools when it runs alone."""
+        return all(self._pages_for(group, tokens) <= group.pool.num_pages for group in self.groups)
 
     def pages_needed(self, request_id: Hashable, new_tokens: int) -> list[int]:
         """Per group, how many pages a portion of ``new_tokens`` more tokens has to take."""
         record = self._get(request_id)
-        total = self._pages_for(record.num_tokens + new_tokens)
-        return [max(0, total - len(pages)) for pages in record.pages]
+        return [max(0, self._pages_for(group, record.num_tokens + new_tokens) - len(pages))
+                for group, pages in zip(self.groups, record.pages)]
+
+    def tokens_within(self, request_id: Hashable, free: list[int]) -> int:
+        """How many more tokens the request can hold if group g may take ``free[g]`` more pages."""
+        record = self._get(request_id)
+        room = min(((len(pages) + spare) * group.page_size
+                    for group, pages, spare in zip(self.groups, record.pages, free)), default=None)
+        return max(0, room - record.num_tokens) if room is not None else 1 << 62
 
     def free_pages(self) -> list[int]:
         return [group.pool.num_free for group in self.groups]
@@ -187,8 +214,8 @@ class CacheManager:
         """Give back the pages that were reserved beyond the committed tokens (a step that failed after
         ``reserve`` and before ``commit``); what the committed tokens hold stays."""
         record = self._get(request_id)
-        keep = self._pages_for(record.num_tokens)
         for group, pages in zip(self.groups, record.pages):
+            keep = self._pages_for(group, record.num_tokens)
             while len(pages) > keep:
                 page = pages.pop()
                 if page != RELEASED:
@@ -199,14 +226,14 @@ class CacheManager:
         record = self._get(request_id)
         record.num_tokens += new_tokens
         for g, (group, pages) in enumerate(zip(self.groups, record.pages)):
-            if self._pages_for(record.num_tokens) > len(pages):
+            if self._pages_for(group, record.num_tokens) > len(pages):
                 raise CacheError(f"request {request_id!r}: tokens committed beyond the reserved pages")
             if group.window is None:
                 continue
             # The next token sits at position num_tokens and sees keys from
             # num_tokens - window + 1 on; pages wholly below that are done.
             first_visible = record.num_tokens - group.window + 1
-            for logical in range(min(len(pages), max(0, first_visible) // self.block_size)):
+            for logical in range(min(len(pages), max(0, first_visible) // group.page_size)):
                 if pages[logical] != RELEASED:
                     group.pool.release(pages[logical])
                     pages[logical] = RELEASED
@@ -222,14 +249,15 @@ class CacheManager:
         return record.rows[group][:len(record.pages[group])]
 
     def slots(self, group: int, request_id: Hashable, start: int, count: int) -> list[int]:
-        """Physical slot (page * block_size + offset) of positions start .. start + count - 1."""
+        """Physical slot (page * page size + offset) of positions start .. start + count - 1."""
         pages = self._get(request_id).pages[group]
+        size = self.groups[group].page_size
         out = []
         for pos in range(start, start + count):
-            page = pages[pos // self.block_size]
+            page = pages[pos // size]
             if page == RELEASED:
                 raise CacheError(f"position {pos} of request {request_id!r} lies in a released page")
-            out.append(page * self.block_size + pos % self.block_size)
+            out.append(page * size + pos % size)
         return out
 
     # -------------------------------------------------------------- invariants

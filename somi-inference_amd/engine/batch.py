@@ -42,8 +42,9 @@ class EntryInfo:
 class PagedView:
     """A cache group's view of the step."""
 
-    slot_mapping: torch.Tensor      # [N] int32: page * block_size + offset where token t's k/v go
+    slot_mapping: torch.Tensor      # [N] int32: page * page_size + offset where what token t keeps goes
     block_table: torch.Tensor       # [E, max_blocks] int32 physical pages of each entry's request
+    page_size: int = 0              # tokens per page of this group
 
 
 @dataclass
@@ -144,14 +145,14 @@ def _layout(entries: list[StepEntry], cache: CacheManager, table_widths: list[in
 
 
 def _views(on_device: torch.Tensor, sizes: list[int], infos: list[EntryInfo], widths: list[int],
-           num_groups: int, block_size: int, max_context: int | None = None) -> StepBatch:
+           page_sizes: list[int], block_size: int, max_context: int | None = None) -> StepBatch:
     offsets = np.cumsum([0] + sizes)
 
     def part(i: int) -> torch.Tensor:
         return on_device[int(offsets[i]):int(offsets[i + 1])]
 
     e = len(infos)
-    paged = [PagedView(part(10 + 2 * g), part(11 + 2 * g).view(e, widths[g])) for g in range(num_groups)]
+    paged = [PagedView(part(10 + 2 * g), part(11 + 2 * g).view(e, widths[g]), size) for g, size in enumerate(page_sizes)]
     return StepBatch(
         num_tokens=sizes[0], num_entries=e, num_logit_rows=sizes[7],
         token_ids=part(0), positions=part(1), token_entry=part(2), entry_start=part(3),
@@ -171,7 +172,8 @@ def build_step(entries: list[StepEntry], cache: CacheManager, device: torch.devi
     """
     sections, infos, widths = _layout(entries, cache, None)
     packed = torch.from_numpy(np.concatenate(sections))
-    return _views(packed.to(device), [s.size for s in sections], infos, widths, len(cache.groups), cache.block_size)
+    return _views(packed.to(device), [s.size for s in sections], infos, widths,
+                  [group.page_size for group in cache.groups], cache.block_size)
 
 
 class StaticStep:
@@ -192,8 +194,9 @@ class StaticStep:
         self.turn = 0
         self.device_buffer = torch.empty(sum(self.sizes), dtype=torch.int32, device=device)
         # kernels that size their launch by the context use the widest the tables allow
-        self.batch = _views(self.device_buffer, self.sizes, infos, widths, len(cache.groups), cache.block_size,
-                            max_context=max(self.table_widths, default=1) * cache.block_size)
+        sizes = [group.page_size for group in cache.groups]
+        self.batch = _views(self.device_buffer, self.sizes, infos, widths, sizes, cache.block_size,
+                            max_context=min((w * s for w, s in zip(self.table_widths, sizes)), default=cache.block_size))
         self._fill(sections, infos)
 
     STAGING = 4

@@ -32,6 +32,18 @@ class _DecodeGraph:
         self.static, self.graph, self.logits = static, graph, logits
 
 
+TABLE_WIDTH_FLOOR = 16
+
+
+def table_width(pages: int) -> int:
+    """The width of a captured step's block table that holds ``pages`` pages: the next power of two, at least
+    TABLE_WIDTH_FLOOR, so that a graph serves until a request has doubled its pages."""
+    width = TABLE_WIDTH_FLOOR
+    while width < pages:
+        width *= 2
+    return width
+
+
 def graph_rows(entries: int) -> int:
     """How many rows the captured step for this many single-token entries has: the next power of two up to
     16, then the next multiple of 16 (the row tile of the matrix products, which cost the same for 17 as for 32
@@ -157,16 +169,20 @@ class ModelRunner:
         tables.  Returns how many graphs were captured."""
         if not self.decode_graphs or max_entries < 1:
             return 0
-        pages = (max(1, max_context) + self.cache.block_size - 1) // self.cache.block_size
-        widths = [16]
-        while widths[-1] < pages:
-            widths.append(widths[-1] * 2)
+        sizes = [group.page_size for group in self.cache.groups]
+        # the contexts at which some group's table doubles, and the widths of all groups at each of them
+        contexts = {max(1, max_context)}
+        for size in sizes:
+            width = TABLE_WIDTH_FLOOR
+            while width * size < max_context:
+                contexts.add(width * size)
+                width *= 2
+        shapes = sorted({tuple(table_width((c + s - 1) // s) for s in sizes) for c in contexts})
         captured = 0
         for rows in sorted({graph_rows(n) for n in range(1, max_entries + 1)}):
-            for width in widths:
-                per_group = [width] * len(self.cache.groups)
-                if (rows, tuple(per_group)) not in self._graphs:
-                    self._capture([], rows, per_group)
+            for per_group in shapes:
+                if (rows, per_group) not in self._graphs:
+                    self._capture([], rows, list(per_group))
                     captured += 1
         return captured
 
@@ -180,11 +196,7 @@ class ModelRunner:
         """
         widths = []
         for g in range(len(self.cache.groups)):
-            longest = max(len(self.cache.page_list(g, e.request_id)) for e in entries)
-            width = 16
-            while width < longest:
-                width *= 2
-            widths.append(width)
+            widths.append(table_width(max(len(self.cache.page_list(g, e.request_id)) for e in entries)))
         real, rows = len(entries), graph_rows(len(entries))
         key = (rows, tuple(widths))
         held = self._graphs.get(key)

@@ -86,8 +86,8 @@ class Scheduler:
     # -------------------------------------------------------------- requests
     def check_request(self, request: Request) -> None:
         """Raises :class:`SchedulerError` if the request can never run; changes nothing."""
-        pages = (request.max_cached_tokens + self.cache.block_size - 1) // self.cache.block_size
-        if pages > self.cache.num_blocks:
+        if not self.cache.holds(request.max_cached_tokens):
+            pages = (request.max_cached_tokens + self.cache.block_size - 1) // self.cache.block_size
             raise SchedulerError(
                 f"request {request.request_id!r} needs {pages} pages for {request.max_cached_tokens} tokens "
                 f"(prompt {len(request.prompt_tokens)} + max_new_tokens {request.max_new_tokens} - 1), "
@@ -169,10 +169,7 @@ class Scheduler:
             if all(n <= f for n, f in zip(need, free)):
                 return count
             # shrink to the end of the last page that still fits
-            cached = self.cache.num_tokens(request.request_id)
-            pages_ok = min(len(self.cache.page_list(g, request.request_id)) + free[g]
-                           for g in range(len(free)))
-            count = self._whole(request, min(count - 1, pages_ok * self.cache.block_size - cached))
+            count = self._whole(request, min(count - 1, self.cache.tokens_within(request.request_id, free)))
         return 0
 
     def schedule(self) -> SchedulerOutput:

@@ -10,7 +10,7 @@ from __future__ import annotations
 import torch
 
 from ..kernels import ops
-from ..parts.base import FixedStateSpec, LayerCache, PagedKVSpec, Runtime
+from ..parts.base import FixedStateSpec, LayerCache, PagedSpec, Runtime
 from ..parts.registry import build_part
 from ..parts.residual import ResidualStream
 from ..weights.loader import WeightFetcher, check_weights
@@ -82,10 +82,10 @@ class DecoderModel:
         return math.lcm(*[int(getattr(layer.mixer, "portion_granule", 1)) for layer in self.layers] or [1])
 
     # -------------------------------------------------------------------- cache
-    def cache_needs(self) -> list[PagedKVSpec | FixedStateSpec | int | None]:
+    def cache_needs(self) -> list[PagedSpec | FixedStateSpec | int | None]:
         """For each run of a layer: the cache its mixer needs, the index of the earlier
         run whose cache it reads, or None."""
-        needs: list[PagedKVSpec | FixedStateSpec | int | None] = []
+        needs: list[PagedSpec | FixedStateSpec | int | None] = []
         for run, index in enumerate(self.order):
             if run in self.plan.cache_from:
                 needs.append(self.plan.cache_from[run])

@@ -1,8 +1,8 @@
 """Parts a layer is put together from, and the registries that name them."""
 
 from .attention import GroupedQueryAttention
-from .base import (Block, FeedForward, FixedStateSpec, LayerCache, Mixer, Norm, PagedKVSpec, Part,
-                   PartSpec, PositionEncoding, Runtime)
+from .base import (PAGE, Block, FeedForward, FixedStateSpec, LayerCache, Mixer, Norm, PagedKVSpec, PagedSpec,
+                   PageTensor, Part, PartSpec, PositionEncoding, Runtime)
 from .block import PreNormBlock
 from .embedding import LMHead, TokenEmbedding
 from .feed_forward import SwiGLU
@@ -22,7 +22,7 @@ register_part("head", "lm_head", LMHead)
 
 __all__ = [
     "Block", "FeedForward", "FixedStateSpec", "GroupedQueryAttention", "LMHead", "LayerCache", "Mixer",
-    "NoPosition", "Norm", "PagedKVSpec", "Part", "PartSpec", "PositionEncoding", "PreNormBlock", "RMSNorm",
+    "NoPosition", "Norm", "PAGE", "PageTensor", "PagedKVSpec", "PagedSpec", "Part", "PartSpec", "PositionEncoding", "PreNormBlock", "RMSNorm",
     "ResidualStream", "RotaryPosition", "Runtime", "SwiGLU", "TokenEmbedding", "build_part", "part_kinds",
     "register_part", "unregister_part",
 ]

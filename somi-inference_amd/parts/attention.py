@@ -29,8 +29,16 @@ class GroupedQueryAttention(Mixer):
 
     def __init__(self, prefix: str, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  position: PartSpec, qkv_bias: bool = True, out_bias: bool = False,
-                 window: int | None = None, scale: float | None = None, shares_cache: bool = False) -> None:
+                 window: int | None = None, scale: float | None = None, shares_cache: bool = False,
+                 names: dict[str, str] | None = None) -> None:
+        """``names``: what the checkpoint calls this part's tensors, role -> name under the prefix.  Roles: ``q``,
+        ``k``, ``v``, ``o`` (defaults ``q_proj`` ... ``o_proj``), ``position`` (``rotary_emb``), and ``qkv`` for a
+        checkpoint that stores the three projections as one matrix, q rows first, then k, then v."""
         super().__init__(prefix)
+        unknown = set(names or {}) - set(self.ROLES) - {"qkv"}
+        if unknown:
+            raise ValueError(f"{prefix}: unknown tensor roles {sorted(unknown)}; known: {sorted(self.ROLES)} and 'qkv'")
+        self.names = {**self.ROLES, **(names or {})}
         if num_heads % num_kv_heads != 0:
             # the reference's message (qwen2.py:116-123)
             raise ValueError(f"num_q_heads ({num_heads}) must be divisible by num_kv_heads ({num_kv_heads})")
@@ -40,14 +48,19 @@ class GroupedQueryAttention(Mixer):
         self.window = int(window) if window else None
         self.scale = float(scale) if scale is not None else self.head_dim ** -0.5
         self.shares_cache = bool(shares_cache)     # reads the cache another layer writes: no k/v of its own
-        self.position = build_part("position", position, prefix=self.name("rotary_emb"))
+        self.position = build_part("position", position, prefix=self.name(self.names["position"]))
+
+    ROLES = {"q": "q_proj", "k": "k_proj", "v": "v_proj", "o": "o_proj", "position": "rotary_emb"}
 
     # ------------------------------------------------------------------ weights
     def _projections(self) -> list[tuple[str, int]]:
-        names = [("q_proj", self.num_heads * self.head_dim)]
-        if not self.shares_cache:
-            names += [("k_proj", self.num_kv_heads * self.head_dim), ("v_proj", self.num_kv_heads * self.head_dim)]
-        return names
+        """The checkpoint's input projections in the order their rows are stacked, with their widths."""
+        q_width, kv_width = self.num_heads * self.head_dim, self.num_kv_heads * self.head_dim
+        if self.shares_cache:
+            return [(self.names["q"], q_width)]
+        if "qkv" in self.names:
+            return [(self.names["qkv"], q_width + 2 * kv_width)]
+        return [(self.names["q"], q_width), (self.names["k"], kv_width), (self.names["v"], kv_width)]
 
     def weight_specs(self) -> list[WeightSpec]:
         specs = []
@@ -55,9 +68,10 @@ class GroupedQueryAttention(Mixer):
             specs.append(WeightSpec(self.name(f"{proj}.weight"), (width, self.hidden_size), MATRIX))
             if self.qkv_bias:
                 specs.append(WeightSpec(self.name(f"{proj}.bias"), (width,), VECTOR))
-        specs.append(WeightSpec(self.name("o_proj.weight"), (self.hidden_size, self.num_heads * self.head_dim), MATRIX))
+        out = self.names["o"]
+        specs.append(WeightSpec(self.name(f"{out}.weight"), (self.hidden_size, self.num_heads * self.head_dim), MATRIX))
         if self.out_bias:
-            specs.append(WeightSpec(self.name("o_proj.bias"), (self.hidden_size,), VECTOR))
+            specs.append(WeightSpec(self.name(f"{out}.bias"), (self.hidden_size,), VECTOR))
         return specs + self.position.weight_specs()
 
     def load(self, fetch: Fetch, runtime: Runtime) -> None:
@@ -66,8 +80,9 @@ class GroupedQueryAttention(Mixer):
         self.qkv = Projection.stacked(
             [fetch(self.name(f"{p}.weight")) for p in names],
             [fetch(self.name(f"{p}.bias")) for p in names] if self.qkv_bias else None)
-        self.out = Projection(fetch(self.name("o_proj.weight")),
-                              fetch(self.name("o_proj.bias")) if self.out_bias else None)
+        out = self.names["o"]
+        self.out = Projection(fetch(self.name(f"{out}.weight")),
+                              fetch(self.name(f"{out}.bias")) if self.out_bias else None)
         self.position.load(fetch, runtime)
 
     # -------------------------------------------------------------------- cache

@@ -55,14 +55,62 @@ class Runtime:
 
 
 # ---------------------------------------------------------------- cache needs
-@dataclass(frozen=True)
-class PagedKVSpec:
-    """Keys and values of every past token, in pages.  ``window``: how many keys
-    (the current one included) stay visible; None = all."""
+PAGE = "page"       # stands in a page tensor's shape where the tokens of a page go
 
-    num_kv_heads: int
-    head_dim: int
+
+@dataclass(frozen=True)
+class PageTensor:
+    """One tensor of a paged cache: what a page of it holds.  ``shape`` is the shape of one page with PAGE in
+    the place of the page's tokens, e.g. ``(kv_heads, PAGE, head_dim)``; ``dtype`` None means the engine's."""
+
+    name: str
+    shape: tuple
+    dtype: torch.dtype | None = None
+
+    def __post_init__(self) -> None:
+        if list(self.shape).count(PAGE) != 1:
+            raise ValueError(f"page tensor {self.name!r}: its shape {self.shape} must hold PAGE exactly once")
+
+    def page_shape(self, page_size: int) -> tuple[int, ...]:
+        return tuple(int(page_size) if dim == PAGE else int(dim) for dim in self.shape)
+
+    def elements_per_token(self) -> int:
+        count = 1
+        for dim in self.shape:
+            if dim != PAGE:
+                count *= int(dim)
+        return count
+
+
+@dataclass(frozen=True)
+class PagedSpec:
+    """Something kept for every past token, in pages: the tensors a page holds, how many of the latest tokens
+    stay visible (``window``, the current one included; None = all), and the page size the mixer's kernels want
+    (None = the engine's).  Layers whose window and page size agree share one pool of pages and one block table
+    per request; each layer run has its own tensors."""
+
+    tensors: tuple[PageTensor, ...]
     window: int | None = None
+    page_size: int | None = None
+
+    def __post_init__(self) -> None:
+        names = [t.name for t in self.tensors]
+        if not names or len(set(names)) != len(names):
+            raise ValueError(f"a paged cache needs at least one tensor and distinct names, got {names}")
+        if self.page_size is not None and self.page_size < 1:
+            raise ValueError(f"page size {self.page_size} must be >= 1")
+
+
+class PagedKVSpec(PagedSpec):
+    """Keys and values of every past token: K ``[pages, kv_heads, page, head_dim]`` and V transposed inside a
+    page, ``[pages, kv_heads, head_dim, page]`` (consecutive positions of one channel are adjacent: the operand
+    layout of the weights-times-values product)."""
+
+    def __init__(self, num_kv_heads: int, head_dim: int, window: int | None = None, page_size: int | None = None) -> None:
+        super().__init__((PageTensor("k", (int(num_kv_heads), PAGE, int(head_dim))),
+                          PageTensor("v", (int(num_kv_heads), int(head_dim), PAGE))), window, page_size)
+        object.__setattr__(self, "num_kv_heads", int(num_kv_heads))
+        object.__setattr__(self, "head_dim", int(head_dim))
 
 
 @dataclass(frozen=True)
@@ -77,17 +125,25 @@ class FixedStateSpec:
 class LayerCache:
     """What one run of a layer sees of the cache: the tensors of its call site.
 
-    ``group`` indexes ``step.paged`` (paged) — the block table and slot mapping
-    of the layer's group.  ``writes`` is False for a layer that reads the cache
-    another layer wrote.
+    ``group`` indexes ``step.paged`` (paged) — the block table and slot mapping of the layer's group, whose pages
+    hold ``page_size`` tokens.  ``tensors[name]`` is ``[pages, *page shape]`` for each tensor of the spec.
+    ``writes`` is False for a layer that reads the cache another layer wrote.
     """
 
-    spec: PagedKVSpec | FixedStateSpec
+    spec: PagedSpec | FixedStateSpec
     group: int
-    k: torch.Tensor | None = None        # [pages, kv_heads, page_size, head_dim]
-    v: torch.Tensor | None = None        # [pages, kv_heads, head_dim, page_size]
+    tensors: dict[str, torch.Tensor] = field(default_factory=dict)
     state: torch.Tensor | None = None    # [slots, *shape]
     writes: bool = True
+    page_size: int = 0
+
+    @property
+    def k(self) -> torch.Tensor | None:      # [pages, kv_heads, page_size, head_dim]
+        return self.tensors.get("k")
+
+    @property
+    def v(self) -> torch.Tensor | None:      # [pages, kv_heads, head_dim, page_size]
+        return self.tensors.get("v")
 
 
 Fetch = Callable[[str], torch.Tensor]
@@ -144,7 +200,7 @@ class PositionEncoding(Part):
 
 
 class Mixer(Part):
-    def cache_spec(self) -> PagedKVSpec | FixedStateSpec | None:
+    def cache_spec(self) -> PagedSpec | FixedStateSpec | None:
         return None
 
     takes_normed_rows = False      # True: x may arrive as parts.linear.NormedRows (rows still to be normed)

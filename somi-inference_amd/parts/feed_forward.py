@@ -18,21 +18,36 @@ class SwiGLU(FeedForward):
     graph_safe = True
     takes_normed_rows = True
 
-    def __init__(self, prefix: str, hidden_size: int, intermediate_size: int) -> None:
+    ROLES = {"gate": "gate_proj", "up": "up_proj", "down": "down_proj"}
+
+    def __init__(self, prefix: str, hidden_size: int, intermediate_size: int,
+                 names: dict[str, str] | None = None) -> None:
+        """``names``: what the checkpoint calls this part's matrices, role -> name under the prefix.  Roles:
+        ``gate``, ``up``, ``down`` (defaults ``gate_proj``, ``up_proj``, ``down_proj``), and ``gate_up`` for a
+        checkpoint that stores gate and up as one ``[2I, H]`` matrix, gate rows first."""
         super().__init__(prefix)
         self.hidden_size, self.intermediate_size = int(hidden_size), int(intermediate_size)
+        unknown = set(names or {}) - set(self.ROLES) - {"gate_up"}
+        if unknown:
+            raise ValueError(f"{prefix}: unknown tensor roles {sorted(unknown)}; known: {sorted(self.ROLES)} and 'gate_up'")
+        self.names = {**self.ROLES, **(names or {})}
 
     def weight_specs(self) -> list[WeightSpec]:
         h, i = self.hidden_size, self.intermediate_size
-        return [WeightSpec(self.name("gate_proj.weight"), (i, h), MATRIX),
-                WeightSpec(self.name("up_proj.weight"), (i, h), MATRIX),
-                WeightSpec(self.name("down_proj.weight"), (h, i), MATRIX)]
+        down = WeightSpec(self.name(f"{self.names['down']}.weight"), (h, i), MATRIX)
+        if "gate_up" in self.names:
+            return [WeightSpec(self.name(f"{self.names['gate_up']}.weight"), (2 * i, h), MATRIX), down]
+        return [WeightSpec(self.name(f"{self.names['gate']}.weight"), (i, h), MATRIX),
+                WeightSpec(self.name(f"{self.names['up']}.weight"), (i, h), MATRIX), down]
 
     INTERLEAVE = 16       # rows per block when gate and up are interleaved for the fused kernel
 
     def load(self, fetch: Fetch, runtime: Runtime) -> None:
         super().load(fetch, runtime)
-        gate, up = fetch(self.name("gate_proj.weight")), fetch(self.name("up_proj.weight"))
+        if "gate_up" in self.names:
+            gate, up = fetch(self.name(f"{self.names['gate_up']}.weight")).chunk(2, dim=0)
+        else:
+            gate, up = (fetch(self.name(f"{self.names[role]}.weight")) for role in ("gate", "up"))
         # The layout of the merged matrix is private.  In bfloat16 the rows are interleaved in blocks of 16
         # (gate 0..15, up 0..15, gate 16..31, ...), so that the decode kernel has gate and up of the same
         # columns in one workgroup and applies the gate in its epilogue.
@@ -44,7 +59,7 @@ class SwiGLU(FeedForward):
             self.gate_up = Projection(merged)
         else:
             self.gate_up = Projection.stacked([gate, up])
-        self.down = Projection(fetch(self.name("down_proj.weight")))
+        self.down = Projection(fetch(self.name(f"{self.names['down']}.weight")))
 
     def forward(self, x, step=None):
         if isinstance(x, NormedRows):

@@ -7,7 +7,7 @@ import torch
 
 from somi_inference_amd.cache import RELEASED, CacheError, CacheManager, OutOfPages, PagePool
 from somi_inference_amd.engine import StepEntry, build_step
-from somi_inference_amd.parts import FixedStateSpec, PagedKVSpec
+from somi_inference_amd.parts import PAGE, FixedStateSpec, PagedKVSpec, PagedSpec, PageTensor
 
 
 def manager(num_blocks=20, block_size=4, needs=None, max_requests=8):
@@ -133,8 +133,11 @@ def test_state_slots_and_cache_sharing_runs():
 @pytest.mark.parametrize("seed", range(6))
 def test_random_orders_never_lose_hold_twice_or_free_twice(seed):
     rng = random.Random(seed)
-    needs = [PagedKVSpec(1, 8), PagedKVSpec(1, 8, window=5)]
+    latent = (PageTensor("latent", (PAGE, 6)),)
+    needs = [PagedKVSpec(1, 8), PagedKVSpec(1, 8, window=5), PagedSpec(latent, page_size=3),
+             PagedSpec(latent, window=7, page_size=6)]
     m = manager(num_blocks=12, block_size=4, needs=needs, max_requests=5)
+    assert [g.pool.num_pages for g in m.groups] == [12, 12, 16, 8]
     live, next_id = {}, 0
     for _ in range(400):
         action = rng.random()
@@ -162,7 +165,7 @@ def test_random_orders_never_lose_hold_twice_or_free_twice(seed):
         m.check_invariants()
     for rid in list(live):
         m.free(rid)
-    assert m.free_pages() == [12, 12]
+    assert m.free_pages() == [12, 12, 16, 8]
 
 
 def test_step_arrays_for_a_mixed_batch():
@@ -210,3 +213,43 @@ def test_rollback_gives_back_what_a_failed_step_reserved_and_nothing_else():
     cache.free("a")
     assert cache.free_pages() == [8, 8]
     cache.check_invariants()
+
+
+def test_a_group_stores_what_its_spec_lists_in_pages_of_its_own_size():
+    latent = PagedSpec((PageTensor("latent", (PAGE, 6), torch.float32), PageTensor("gate", (2, PAGE))), page_size=3)
+    needs = [PagedKVSpec(2, 8), latent, PagedKVSpec(2, 8, page_size=3), latent, 1]
+    m = CacheManager(needs, block_size=4, num_blocks=6, max_requests=2, dtype=torch.bfloat16, device="cpu")
+    # keys and values at the engine's page size; the latent group and the k/v layer that asks for pages of 3
+    # share tables (same window, same page size) and hold the pool's 24 tokens in 8 pages
+    assert [(g.window, g.page_size, g.pool.num_pages, g.runs) for g in m.groups] == [(None, 4, 6, [0]), (None, 3, 8, [1, 2, 3])]
+    kv, lat, kv3, lat2, reader = m.layer_caches
+    assert kv.k.shape == (6, 2, 4, 8) and kv.v.shape == (6, 2, 8, 4) and kv.page_size == 4
+    assert lat.tensors["latent"].shape == (8, 3, 6) and lat.tensors["latent"].dtype == torch.float32
+    assert lat.tensors["gate"].shape == (8, 2, 3) and lat.tensors["gate"].dtype == torch.bfloat16
+    assert lat.k is None and lat.page_size == 3
+    assert kv3.k.shape == (8, 2, 3, 8) and kv3.group == lat.group == 1
+    assert lat2.tensors["latent"] is not lat.tensors["latent"]
+    assert reader.tensors["latent"] is lat.tensors["latent"] and not reader.writes and reader.page_size == 3
+    assert CacheManager.page_bytes(needs, 4, torch.bfloat16) == 4 * (2 * 2 * 8 * 2 + (6 * 4 + 2 * 2) + 2 * 2 * 8 * 2 + (6 * 4 + 2 * 2))
+    m.register("r")
+    assert m.pages_needed("r", 7) == [2, 3]
+    m.reserve("r", 7)
+    m.commit("r", 7)
+    assert m.slots(0, "r", 3, 3) == [m.page_list(0, "r")[0] * 4 + 3, m.page_list(0, "r")[1] * 4, m.page_list(0, "r")[1] * 4 + 1]
+    assert m.slots(1, "r", 2, 2) == [m.page_list(1, "r")[0] * 3 + 2, m.page_list(1, "r")[1] * 3]
+    # one more page in group 0 would hold up to token 12, two more in group 1 up to token 15
+    assert m.tokens_within("r", [1, 2]) == 5 and m.tokens_within("r", [0, 0]) == 1
+    assert m.holds(24) and not m.holds(25)
+    step = build_step([StepEntry("r", [1], [0])], _reserved(m, "r", 1), torch.device("cpu"))
+    assert [view.page_size for view in step.paged] == [4, 3]
+    assert step.paged[1].block_table.shape == (1, 3) and step.paged[0].block_table.shape == (1, 2)
+    m.check_invariants()
+    with pytest.raises(ValueError, match="holds no page"):
+        manager(num_blocks=1, block_size=4, needs=[PagedSpec((PageTensor("x", (PAGE,)),), page_size=5)])
+    with pytest.raises(ValueError, match="PAGE exactly once"):
+        PageTensor("x", (3, 4))
+
+
+def _reserved(m, request_id, count):
+    m.reserve(request_id, count)
+    return m
