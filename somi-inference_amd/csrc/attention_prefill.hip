@@ -18,6 +18,7 @@
 // Every key tile is used for all QB query blocks from registers.  Key tiles are aligned to absolute
 // positions (multiples of 32), so a query's arithmetic does not depend on how the prompt was cut.
 #include "common.h"
+#include "attention_prefill_tile.h"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
@@ -242,6 +243,9 @@ attention_prefill_kernel(const bf16* __restrict__ q, int64_t q_stride, const bf1
 #define PREFILL_SHAPE_NARROW 1     // 64 queries a workgroup
 #define PREFILL_SHAPE_SPLIT 2      // 64 queries, two wavefronts share a query block's keys
 #define PREFILL_SHAPE_WIDE 3       // 128 queries
+#define PREFILL_SHAPE_TILE 4       // the 32 x 32 tile kernel: 128 queries a workgroup, two key splits
+#define PREFILL_SHAPE_TILE_WIDE 5  // the 32 x 32 tile kernel: 256 queries a workgroup
+#define PREFILL_TILE_WIDE_GROUPS 512   // from this many 256-query groups on the tile kernel takes 256 queries a workgroup
 #ifndef PREFILL_KEY_SPLIT_BELOW
 #define PREFILL_KEY_SPLIT_BELOW 896   // below this many 64-query workgroups two wavefronts share a query block's keys
                                       // (measured at 7B head counts: 448 workgroups 29 against 33 us, 512 tokens after
@@ -632,7 +636,8 @@ static int launch_prefill(const void* q, int64_t q_stride, const void* kc, const
 // portion out: its tokens are somebody else's); max_entry_len: the longest portion (sizes the grid).  bfloat16 only; head_dim a multiple of 16
 // up to 256; page_size a multiple of 4.  k_cache [pages, nkv, page_size, D], v_cache [pages, nkv, D, page_size];
 // out: [n_tokens, nq * D].  max_context: the longest context a portion ends at (a hint for the launch shape; 0: unknown).
-// shape: 0 lets the launcher choose; 1..3 ask for a launch shape of the LDS kernel (PREFILL_SHAPE_*).
+// shape: 0 lets the launcher choose; 1..3 ask for a launch shape of the 16 x 16 LDS kernel, 4 and 5 for one of the
+// 32 x 32 tile kernel (PREFILL_SHAPE_*).
 extern "C" int somi_attention_prefill(const void* q, int64_t q_stride, const void* k_cache, const void* v_cache,
                                       const int* block_table, int max_blocks, const int* entry_start,
                                       const int* entry_first_pos, const int* entry_len, int n_entries, int max_entry_len, int max_context,
@@ -644,13 +649,24 @@ extern "C" int somi_attention_prefill(const void* q, int64_t q_stride, const voi
     SOMI_REQUIRE(D % 16 == 0 && D >= 16 && D <= 256, "attention_prefill: head_dim %d must be a multiple of 16 up to 256", D);
     SOMI_REQUIRE(page_size > 0 && page_size % 4 == 0, "attention_prefill: page size %d must be a multiple of 4", page_size);
     SOMI_REQUIRE(window >= 0, "attention_prefill: window must be >= 0");
-    SOMI_REQUIRE(shape >= PREFILL_SHAPE_AUTO && shape <= PREFILL_SHAPE_WIDE, "attention_prefill: unknown launch shape %d", shape);
+    SOMI_REQUIRE(shape >= PREFILL_SHAPE_AUTO && shape <= PREFILL_SHAPE_TILE_WIDE, "attention_prefill: unknown launch shape %d", shape);
     SOMI_REQUIRE(n_entries <= 65535 && nq <= 65535, "attention_prefill: too many entries or heads");
     SOMI_REQUIRE(max_entry_len <= 65535 * 128, "attention_prefill: a portion of %d tokens is too long", max_entry_len);
     SOMI_REQUIRE((uintptr_t)q % 16 == 0 && (q_stride * 2) % 16 == 0 && (uintptr_t)k_cache % 16 == 0 &&
                  (uintptr_t)v_cache % 8 == 0 && (uintptr_t)out % 8 == 0,
                  "attention_prefill: q, k, v and out must be 16-byte aligned");
     if (n_entries == 0 || max_entry_len == 0) return 0;
+    // head sizes 64 and 128 over pages of 8 keys or more: the 32 x 32 tile kernel
+    const bool tile_ok = somi_prefill_tile_applies(D, page_size, max_blocks, window) && (uintptr_t)v_cache % 16 == 0;
+    if (shape >= PREFILL_SHAPE_TILE)
+        SOMI_REQUIRE(tile_ok, "attention_prefill: the tile kernel does not take head size %d, pages of %d keys or a block table of %d pages",
+                     D, page_size, max_blocks);
+    if (tile_ok && (shape == PREFILL_SHAPE_AUTO || shape >= PREFILL_SHAPE_TILE)) {
+        const int64_t groups = (int64_t)ceil_div(max_entry_len, 256) * n_entries * nq;
+        const bool wide = shape == PREFILL_SHAPE_AUTO ? groups >= PREFILL_TILE_WIDE_GROUPS : shape == PREFILL_SHAPE_TILE_WIDE;
+        return somi_prefill_tile(q, q_stride, k_cache, v_cache, block_table, max_blocks, entry_start, entry_first_pos, entry_len,
+                                 n_entries, max_entry_len, wide, nq, nkv, D, page_size, window, scale, out, stream);
+    }
 #define SOMI_PREFILL(DT, QB)                                                                                       \
     case DT:                                                                                                       \
         return launch_prefill<DT, QB>(q, q_stride, k_cache, v_cache, block_table, max_blocks, entry_start,         \

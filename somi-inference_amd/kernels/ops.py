@@ -262,7 +262,9 @@ def attention_prefill(q: torch.Tensor, q_stride: int, k_cache: torch.Tensor, v_c
     ([N, nq * D] bfloat16).  entry_start: [E + 1] int32 offsets of the portions in the flat batch;
     entry_first_position: [E] int32.  ``max_context``: the longest context a portion ends at, a hint for the
     launch shape (0: unknown).  ``shape``: 0 lets the launcher choose; 1 (64 queries a workgroup), 2 (the same
-    with a query block's keys split over two wavefronts) or 3 (128 queries) asks for that shape of the LDS kernel.
+    with a query block's keys split over two wavefronts) or 3 (128 queries) asks for that shape of the 16 x 16 LDS
+    kernel; 4 (128 queries, two key splits) or 5 (256 queries) for that shape of the 32 x 32 tile kernel (head sizes 64
+    and 128, pages of 8 keys or more).
     ``entry_len``: [E] int32 lengths that stand for the offsets' own; 0 leaves a portion out (its rows of ``out`` are
     not written)."""
     _need(q, "q", torch.bfloat16)

@@ -391,14 +391,27 @@ def test_attention_decode_refuses_what_it_cannot_do():
         ops.attention_decode(q, 32, kc, vc, i32([[0]]), i32([0]), i32([0]), 2, 0, 0.2, 16, 1, out)
 
 
+def tile_kernel_takes(d, page):
+    """The sizes the 32 x 32 tile kernel of the prefill attention takes (launch shapes 4 and 5)."""
+    return d in (64, 128) and page >= 8 and page & (page - 1) == 0
+
+
 @pytest.mark.parametrize("nq, nkv, d, page, window", [
     (8, 4, 32, 4, 0), (12, 2, 64, 16, 0), (8, 1, 48, 8, 0), (6, 3, 128, 16, 37), (28, 4, 128, 16, 0),
-    (4, 2, 16, 8, 0), (14, 2, 256, 16, 0), (5, 5, 80, 4, 5), (7, 1, 112, 32, 100), (3, 1, 208, 16, 0)])
-@pytest.mark.parametrize("shape", [0, 1, 2, 3], ids=["auto", "narrow", "split", "wide"])
+    (4, 2, 16, 8, 0), (14, 2, 256, 16, 0), (5, 5, 80, 4, 5), (7, 1, 112, 32, 100), (3, 1, 208, 16, 0),
+    (14, 2, 64, 8, 20), (8, 2, 128, 32, 0), (5, 1, 128, 8, 150), (6, 6, 64, 64, 0)])
+@pytest.mark.parametrize("shape", [0, 1, 2, 3, 4, 5], ids=["auto", "narrow", "split", "wide", "tile", "tile-wide"])
 def test_attention_prefill_mfma_against_dense_softmax(nq, nkv, d, page, window, shape):
     """Portions of several requests in one launch: a long one that starts at position 0, one that continues
     after 150 cached tokens, a portion of two tokens, single tokens after 77 and after 0 cached ones.  Each
-    launch shape of the kernel that stages tiles through LDS is asked for in turn."""
+    launch shape of the two kernels that stage tiles through LDS is asked for in turn; the tile kernel refuses the
+    sizes it does not take."""
+    if shape >= 4 and not tile_kernel_takes(d, page):
+        q, kc, vc = rnd(4, nq * d, dtype="bfloat16"), rnd(2, nkv, page, d, dtype="bfloat16"), rnd(2, nkv, d, page, dtype="bfloat16")
+        with pytest.raises(KernelError, match="tile kernel does not take"):
+            ops.attention_prefill(q, nq * d, kc, vc, i32([[1]]), i32([0, 4]), i32([0]), 4, nq, window, d ** -0.5,
+                                  torch.zeros_like(q), shape=shape)
+        return
     cached, new = [0, 150, 30, 77, 0], [203, 130, 2, 1, 1]
     total = [c + n for c, n in zip(cached, new)]
     n_pages = sum((t + page - 1) // page for t in total) + 3
@@ -698,8 +711,50 @@ def test_many_rows_product_into_the_residual_stream(m, n, k, tile):
         torch.testing.assert_close(got.float(), want, atol=0.02 * float(want.abs().max()), rtol=2e-2)
 
 
+@pytest.mark.parametrize("nq, nkv, d, page, window", [(8, 2, 128, 16, 0), (14, 2, 64, 8, 700), (4, 4, 128, 64, 1500)])
+@pytest.mark.parametrize("shape", [0, 4, 5], ids=["auto", "tile", "tile-wide"])
+def test_attention_prefill_tile_kernel_over_long_contexts(nq, nkv, d, page, window, shape):
+    """Many steps of the tile kernel: a prompt of 1,100 tokens from position 0, 300 tokens after 2,000 cached ones
+    (a block table of 144 to 288 pages), a portion that ends inside its first tile, and one whose length is no
+    multiple of anything; with and without a window that the long requests outgrow.  Against the plain kernel."""
+    cached, new = [0, 2000, 5, 31], [1100, 300, 20, 333]
+    total = [c + n for c, n in zip(cached, new)]
+    n_pages = sum((t + page - 1) // page for t in total) + 2
+    perm = torch.randperm(n_pages - 1, generator=torch.Generator().manual_seed(8)).add(1).tolist()
+    tables, at = [], 0
+    for t in total:
+        count = (t + page - 1) // page
+        tables.append(perm[at:at + count])
+        at += count
+    width = max(len(t) for t in tables) + 1
+    block_table = i32([t + [0] * (width - len(t)) for t in tables])
+    kc = torch.full((n_pages, nkv, page, d), float("nan"), dtype=torch.bfloat16, device=DEV)      # what is no key of a request is NaN
+    vc = torch.full((n_pages, nkv, d, page), float("nan"), dtype=torch.bfloat16, device=DEV)
+    for r, t in enumerate(total):
+        keys, values = rnd(t, nkv, d, dtype="bfloat16", seed=50 + r), rnd(t, nkv, d, dtype="bfloat16", seed=60 + r)
+        pos = torch.arange(t, device=DEV)
+        pages = torch.tensor(tables[r], device=DEV)[pos // page]
+        kc[pages, :, pos % page] = keys
+        vc[pages, :, :, pos % page] = values
+    n = sum(new)
+    q = rnd(n, nq * d, dtype="bfloat16", seed=9, scale=1.5)
+    positions, entry, starts = [], [], [0]
+    for e, (c, k) in enumerate(zip(cached, new)):
+        positions += [c + i for i in range(k)]
+        entry += [e] * k
+        starts.append(starts[-1] + k)
+    scale = d ** -0.5
+    want = ops.paged_attention_plain(q, nq * d, kc, vc, block_table, i32(entry), i32(positions), nq, window, scale)
+    assert bool(torch.isfinite(want.float()).all())
+    out = torch.full((n, nq * d), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ops.attention_prefill(q, nq * d, kc, vc, block_table, i32(starts), i32(cached), max(new), nq, window, scale, out,
+                          max_context=max(total), shape=shape)
+    assert bool(torch.isfinite(out.float()).all())
+    torch.testing.assert_close(out.float(), want.float(), atol=2e-2, rtol=2e-2)
+
+
 @pytest.mark.parametrize("nq, nkv, d, page, window", [(8, 2, 64, 16, 0), (6, 3, 128, 16, 21), (4, 1, 32, 8, 0), (14, 2, 256, 16, 0),
-                                                     (5, 5, 80, 4, 9)])
+                                                     (5, 5, 80, 4, 9), (7, 1, 128, 8, 40), (4, 2, 64, 32, 0)])
 def test_attention_ignores_whatever_lies_beyond_a_requests_keys(nq, nkv, d, page, window):
     """Pages are handed out again without being cleared, and pages a window has passed read as page 0.  Everything
     in the cache that is not a visible key of the request is NaN here (the tail of its last page, every other
@@ -748,7 +803,7 @@ def test_attention_ignores_whatever_lies_beyond_a_requests_keys(nq, nkv, d, page
     plain_out = ops.paged_attention_plain(q, nq * d, kc, vc, block_table, i32(entry), i32(positions), nq, window, scale)
     assert bool(torch.isfinite(plain_out.float()).all()), "the plain kernel let a value from outside the visible keys through"
     torch.testing.assert_close(plain_out.float().cpu(), want, atol=2e-2, rtol=2e-2)
-    for shape in (0, 1, 2, 3):
+    for shape in (0, 1, 2, 3) + ((4, 5) if tile_kernel_takes(d, page) else ()):
         out = torch.full((n, nq * d), float("nan"), dtype=torch.bfloat16, device=DEV)
         ops.attention_prefill(q, nq * d, kc, vc, block_table, i32(starts), i32(cached), max(new), nq, window, scale, out,
                               shape=shape)
