@@ -26,6 +26,7 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E bandwidth
 PEAK_FLOPS = {"bfloat16": 2.5e15, "float32": 157.3e12}   # dense MFMA peaks
+POINT_BATCHES = (1, 64, 96, 128)      # decode is also measured at these numbers of requests ("points")
 
 
 # layer sizes of the Qwen2.5 family: (layers, hidden, heads, kv heads, head_dim, intermediate, rms_norm_eps,
@@ -53,7 +54,7 @@ def parse_args() -> argparse.Namespace:
     p.add_argument("--block-size", type=int, default=16)
     p.add_argument("--prefill-tokens", type=int, default=2048)
     p.add_argument("--seed", type=int, default=0)
-    p.add_argument("--no-points", action="store_true", help="skip the batch 1 / batch 64 decode points")
+    p.add_argument("--no-points", action="store_true", help="skip the decode points at other batch sizes (1, 64, 96, 128)")
     p.add_argument("--no-prefill", action="store_true", help="skip the prefill measurement")
     p.add_argument("--no-peaks", action="store_true", help="skip the measurement of the machine's own peaks")
     p.add_argument("--output-file", type=str, default=None, help="Append the result line to a JSONL file.")
@@ -152,7 +153,7 @@ def main() -> int:
     device = torch.device("cuda:0")
     model = random_model(config, seed=args.seed, dtype=args.dtype, draw_on="device")
     elem = 2 if args.dtype == "bfloat16" else 4
-    batches = [args.batch] if args.no_points else sorted({1, args.batch, 64})
+    batches = [args.batch] if args.no_points else sorted({1, args.batch, *POINT_BATCHES})
     # Decoding is measured through the generation loop itself (scheduler, step function, sampler, running ahead of
     # the device).  The scheduler runs the prompts in portions of 2,048 tokens and lets the requests that are done
     # with theirs decode meanwhile, so a request has decoded up to `ramp` tokens before the timed steps begin.
@@ -207,7 +208,7 @@ def main() -> int:
 
     results = {}
     for batch in batches:
-        steps = args.steps if batch == args.batch else max(8, args.steps // 2)
+        steps = args.steps if batch == args.batch else max(8, args.steps // (2 if batch <= 64 else 4))
         warmup = args.warmup if batch == args.batch else max(2, args.warmup // 2)
         results[batch] = decode_run(batch, steps, warmup)
 
@@ -272,7 +273,7 @@ def main() -> int:
         roofline["frac_of_measured"] = round(achieved / peaks["stream_read_gbs"], 4)
     line = {
         "metric": f"decode tok/s at batch {args.batch}, Qwen2.5-{args.sizes.upper()} layer sizes "
-                  f"(plus prefill tok/s at {args.prefill_tokens:,} tokens, batch 1/64 points)",
+                  f"(plus prefill tok/s at {args.prefill_tokens:,} tokens, batch 1/64/96/128 points)",
         "value": round(main_run["tok_s"], 2), "unit": "tokens/s", "n_gpus": 1,
         "steps": main_run["steps"], "warmup": main_run["warmup"], "ms_per_step": round(main_run["ms"], 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
@@ -288,7 +289,7 @@ def main() -> int:
                    "mean_context": round(main_run["mean_ctx"], 1)},
         "roofline": roofline,
         "latency_ms": summarize_ms(main_run["step_ms"]),
-        "points": {f"decode_b{b}": round(r["tok_s"], 2) for b, r in results.items() if b in (1, 64)},
+        "points": {f"decode_b{b}": round(r["tok_s"], 2) for b, r in results.items() if b in POINT_BATCHES},
     }
     if prefill is not None:
         line["prefill"] = prefill

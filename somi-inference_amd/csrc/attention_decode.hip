@@ -42,6 +42,22 @@ __device__ __forceinline__ bf16x8 half_step(const bf16* p) {
     return u.wide;
 }
 
+// The keys of split `split` of a token at position p that sees keys from lo on: the visible range (from the
+// 32-key tile that holds lo) cut into num_splits equal parts of a multiple of 16 keys, at most split_len each.
+// The parts follow the token's own range, not the longest context the launch was sized for, so a launch with
+// more splits than a short context needs (a captured step serves contexts up to its block tables' width) still
+// gives every workgroup a share of the keys.
+__device__ __forceinline__ void decode_split_range(int p, int lo, int split, int split_len, int num_splits, int& begin,
+                                                   int& end) {
+    const int base = lo & ~31;
+    const int span = p - base + 1;
+    int len = ((span + num_splits - 1) / num_splits + 15) & ~15;
+    len = len < split_len ? len : split_len;
+    const int first = base + split * len;
+    begin = lo > first ? lo : first;
+    end = p < first + len - 1 ? p : first + len - 1;
+}
+
 template <int DT>
 __global__ void __launch_bounds__(256)
 attention_decode_kernel(const bf16* __restrict__ q, int64_t q_stride, const bf16* __restrict__ kc,
@@ -67,8 +83,8 @@ attention_decode_kernel(const bf16* __restrict__ q, int64_t q_stride, const bf16
     const int p = positions[t];
     const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
     const int* table = block_table + (int64_t)token_entry[t] * max_blocks;
-    const int begin = lo > split * split_len ? lo : split * split_len;
-    const int end = p < (split + 1) * split_len - 1 ? p : (split + 1) * split_len - 1;      // inclusive
+    int begin, end;                                  // this split's keys, inclusive
+    decode_split_range(p, lo, split, split_len, num_splits, begin, end);
 
     const int hloc = hb * 16 + r;
     const int head = kvh * G + (hloc < G ? hloc : G - 1);
@@ -249,8 +265,8 @@ attention_decode_lds_kernel(const bf16* __restrict__ q, int64_t q_stride, const 
     const int p = positions[t];
     const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
     const int* table = block_table + (int64_t)token_entry[t] * max_blocks;
-    const int begin = lo > split * split_len ? lo : split * split_len;
-    const int end = p < (split + 1) * split_len - 1 ? p : (split + 1) * split_len - 1;      // inclusive
+    int begin, end;                                  // this split's keys, inclusive
+    decode_split_range(p, lo, split, split_len, num_splits, begin, end);
     const int hloc = hb * 16 + r;
     const int head = kvh * G + (hloc < G ? hloc : G - 1);
 

@@ -9,6 +9,7 @@ from . import ops
 SKINNY_MAX_ROWS = 64   # what the skinny MFMA kernel takes
 MID_PASSES_ROWS = 192  # up to here a product with long K and few columns runs the split-K kernel in passes of 64 rows
 SKINNY_ROWS = 64       # up to here the few-rows kernels run; beyond, the many-rows kernel (ops.linear_big)
+RESIDUAL_PASSES_ROWS = 128   # up to here a product into the residual stream with few columns runs in passes of 64 rows
 
 
 def _mid_is_faster(m: int, n: int, k: int) -> bool:
@@ -43,9 +44,22 @@ def linear_residual(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | 
                     next_norm_weight: torch.Tensor | None = None) -> tuple[torch.Tensor, torch.Tensor | None]:
     """h += x @ weight.T (+ bias) in place, by the kernel that :func:`linear` would take for the sizes; see
     :func:`ops.linear_residual`."""
-    if x.shape[0] > ops.FUSED_MAX_ROWS:
+    m, n = x.shape[0], weight.shape[0]
+    if ops.FUSED_MAX_ROWS < m <= RESIDUAL_PASSES_ROWS and n <= 8192:
+        # few columns and little more than 64 rows (the o projection of 65 to 128 requests): the 256-row tiles of the
+        # many-rows kernel are too few to fill the device (28 workgroups at 7B sizes: 61 us), two passes of the
+        # few-rows kernel are not (2 x 14 us)
+        stats, weighted = [], []
+        for at in range(0, m, ops.FUSED_MAX_ROWS):
+            rows = slice(at, at + ops.FUSED_MAX_ROWS)
+            mid = _mid_is_faster(min(ops.FUSED_MAX_ROWS, m - at), n, x.shape[1])
+            part_stats, part_weighted = ops.linear_residual(x[rows], weight, bias, h[rows], next_norm_weight, mid=mid)
+            stats.append(part_stats)
+            weighted.append(part_weighted)
+        return torch.cat(stats, dim=1), (torch.cat(weighted) if next_norm_weight is not None else None)
+    if m > ops.FUSED_MAX_ROWS:
         return ops.linear_big_residual(x, weight, bias, h, next_norm_weight)
-    mid = _mid_is_faster(x.shape[0], weight.shape[0], x.shape[1])
+    mid = _mid_is_faster(m, n, x.shape[1])
     return ops.linear_residual(x, weight, bias, h, next_norm_weight, mid=mid)
 
 

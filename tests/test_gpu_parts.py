@@ -266,7 +266,7 @@ def test_rotary_part_offers_the_reference_table():
     assert inv_freq.cpu().tolist() == pytest.approx([1.0, 1e6 ** -0.25, 1e6 ** -0.5, 1e6 ** -0.75], rel=1e-6)
 
 
-@pytest.mark.parametrize("n_rows", [7, 40, 64, 65, 300])
+@pytest.mark.parametrize("n_rows", [7, 40, 64, 65, 100, 128, 129, 300])
 def test_bfloat16_rows_take_the_add_and_the_norm_inside_the_products(n_rows):
     """Steps in bfloat16, of a few rows (the decode kernels) and of many (the many-rows kernel): a block's last projections arrive at the residual stream uncomputed and are
     added to it by the kernel that computes them; the next norm is applied by the projection that reads the
