@@ -86,20 +86,22 @@ template <int N> __device__ __forceinline__ void big_wait_vmcnt() { asm volatile
 // stage kt frees two slots, which take B of kt + 2 and A of kt + 3.
 // The wide form is persistent: a workgroup walks its die's tiles 32 apart, and the first pieces of the next
 // tile are asked for before the finished tile is stored, so the stores and the first loads overlap.
-template <int BN, int S, int NW, int EPI, bool KTAIL>
+// BM: rows of a tile, 256 (two wavefronts along m) or 128 (one: for 65 to 128 rows, where a 256-row tile would
+// spend half of its products on rows that are not there).
+template <int BM, int BN, int S, int NW, int EPI, bool KTAIL>
 __global__ void __launch_bounds__(NW * 64, 1)
 linear_big_kernel(const BigArgs p) {
     extern __shared__ __attribute__((aligned(1024))) char lds[];
-    constexpr int BM = BIG_BM, BK = BIG_BK, ROW_BYTES = BIG_ROW_BYTES;
+    constexpr int BK = BIG_BK, ROW_BYTES = BIG_ROW_BYTES;
     constexpr int A_BYTES = BM * ROW_BYTES, B_BYTES = BN * ROW_BYTES, STAGE = A_BYTES + B_BYTES;
-    constexpr int WAVES_N = NW / 2;                               // wavefronts: 2 along m, NW / 2 along n
+    constexpr int WAVES_M = BM / 128, WAVES_N = NW / WAVES_M;     // wavefronts along m and along n
     constexpr int WTM = 4, WTN = 2;                               // 32 x 32 products of a wavefront: 128 x 64
-    static_assert(BM / 2 == WTM * 32 && BN / WAVES_N == WTN * 32, "a wavefront owns 128 x 64 of the tile");
+    static_assert(BM == WAVES_M * WTM * 32 && BN / WAVES_N == WTN * 32, "a wavefront owns 128 x 64 of the tile");
     constexpr int LA = BM / 8 / NW, LB = BN / 8 / NW, L = LA + LB;  // direct loads a lane issues per stage (8 rows each)
     constexpr int KK = BK / 16, NM = WTM * WTN, NF = WTM + WTN;
     constexpr bool HALF = S == 5;
     static_assert(HALF || (S == 3 && L % KK == 0), "three whole stages, loads divisible over the sub-steps");
-    static_assert(!HALF || (LA == LB && BN == 256), "halves of equal size");
+    static_assert(!HALF || (LA == LB && BN == 256 && BM == 256), "halves of equal size");
     constexpr int LPS = HALF ? 0 : L / KK;
     constexpr int HB = 256 * ROW_BYTES;                           // bytes of a slot of the wide ring
     constexpr int STG = HALF ? 3 * HB : 0;                        // where the epilogue stages: slots 3 and 4, or the ring
@@ -171,7 +173,7 @@ linear_big_kernel(const BigArgs p) {
 #pragma unroll
     for (int kk = 0; kk < KK; ++kk) {
         const uint32_t f = frow * ROW_BYTES + (((kk * 2 + fk) ^ ((frow >> 1) & 7)) << 4);
-        foffa[kk] = lds_base + f + wm * (BM / 2) * ROW_BYTES;
+        foffa[kk] = lds_base + f + wm * 128 * ROW_BYTES;
         foffb[kk] = lds_base + f + wn * (BN / WAVES_N) * ROW_BYTES;
     }
     // read q of a set, in the order the products need them: a[0], every b, then the other a
@@ -321,7 +323,7 @@ linear_big_kernel(const BigArgs p) {
         if (EPI != BIG_RESIDUAL) {
 #pragma unroll
             for (int i = 0; i < WTM; ++i) {
-                const int sm = m0 + wm * (BM / 2) + i * 32 + ml;
+                const int sm = m0 + wm * 128 + i * 32 + ml;
                 scale[i] = p.row_scale != nullptr ? p.row_scale[sm < M ? sm : M - 1] : 1.f;
             }
             if (EPI == BIG_PLAIN) {
@@ -389,7 +391,7 @@ linear_big_kernel(const BigArgs p) {
                 for (int pass = 0; pass < 32 * LPR / 64; ++pass) {
                     const int row = pass * (64 / LPR) + lane / LPR, piece = lane % LPR;
                     const u32x4 v = *(const u32x4*)(stg + row * SROW + piece * 16);
-                    const int gm = m0 + wm * (BM / 2) + i * 32 + row;
+                    const int gm = m0 + wm * 128 + i * 32 + row;
                     const int gc = out_c0 + piece * 8;
                     if (gm < M) {
                         bf16* dst = p.out + (int64_t)gm * out_n + gc;
@@ -425,7 +427,7 @@ linear_big_kernel(const BigArgs p) {
                     for (int pass = 0; pass < 4; ++pass) {
                         const int row = pass * 8 + (lane >> 3), piece = lane & 7;
                         f32x4 v = *(const f32x4*)(stg + row * SROW + piece * 16);
-                        const int gm = m0 + wm * (BM / 2) + i * 32 + row;
+                        const int gm = m0 + wm * 128 + i * 32 + row;
                         const int gn = wave_n0 + j * 32 + piece * 4;
                         if (gm < M && gn < N) {
                             float* hp = p.h + (int64_t)gm * N + gn;
@@ -463,7 +465,7 @@ linear_big_kernel(const BigArgs p) {
                         float v = sq[pass];
 #pragma unroll
                         for (int off = 4; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
-                        const int gm = m0 + wm * (BM / 2) + i * 32 + pass * 8 + (lane >> 3);
+                        const int gm = m0 + wm * 128 + i * 32 + pass * 8 + (lane >> 3);
                         if ((lane & 7) == 0 && gm < M) p.stats_out[(int64_t)stats_row * p.stats_width + gm] = v;
                     }
                 }
@@ -505,15 +507,19 @@ static bool big_use_wide(int m, int n) {
     return wide <= narrow;
 }
 
-template <int BN, int S, int NW, int EPI, bool KTAIL>
+// The 128-row tile: asked for (tile code BIG_TILE_LOW), or chosen for up to 128 rows.
+#define BIG_TILE_LOW 1
+static bool big_use_low(int m, int tile) { return tile == BIG_TILE_LOW || (tile == 0 && m <= 128); }
+
+template <int BM, int BN, int S, int NW, int EPI, bool KTAIL>
 static int big_launch_one(const BigArgs& args, hipStream_t stream) {
-    const int lds_bytes = S == 5 ? 5 * 256 * BIG_ROW_BYTES : S * (BIG_BM + BN) * BIG_ROW_BYTES;
+    const int lds_bytes = S == 5 ? 5 * 256 * BIG_ROW_BYTES : S * (BM + BN) * BIG_ROW_BYTES;
     static bool raised[64];
     int device = 0;
     hipError_t err = hipGetDevice(&device);
     if (err != hipSuccess || device < 0 || device >= 64) return somi_fail("linear_big: hipGetDevice failed");
     if (!raised[device]) {
-        err = hipFuncSetAttribute((const void*)linear_big_kernel<BN, S, NW, EPI, KTAIL>,
+        err = hipFuncSetAttribute((const void*)linear_big_kernel<BM, BN, S, NW, EPI, KTAIL>,
                                   hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
         if (err != hipSuccess) return somi_fail("linear_big: %d bytes of LDS refused: %s", lds_bytes, hipGetErrorString(err));
         raised[device] = true;
@@ -526,19 +532,25 @@ static int big_launch_one(const BigArgs& args, hipStream_t stream) {
         const int cus_per_die = big_compute_units() / 8 > 0 ? big_compute_units() / 8 : 1;
         per_die = per < cus_per_die ? per : cus_per_die;
     }
-    hipLaunchKernelGGL((linear_big_kernel<BN, S, NW, EPI, KTAIL>), dim3(per_die * 8), dim3(NW * 64), lds_bytes, stream, args);
+    hipLaunchKernelGGL((linear_big_kernel<BM, BN, S, NW, EPI, KTAIL>), dim3(per_die * 8), dim3(NW * 64), lds_bytes, stream, args);
     SOMI_LAUNCH_CHECK("linear_big");
     return 0;
 }
 
 template <int EPI>
 static int big_launch(BigArgs& args, int tile, hipStream_t stream) {
+    const bool ktail = args.K % BIG_BK != 0;
+    if (big_use_low(args.M, tile)) {
+        // up to 128 rows: one row tile of 128, four wavefronts side by side over 256 columns
+        args.tiles_m = ceil_div(args.M, 128);
+        args.tiles_n = ceil_div(args.N, 256);
+        return ktail ? big_launch_one<128, 256, 3, 4, EPI, true>(args, stream) : big_launch_one<128, 256, 3, 4, EPI, false>(args, stream);
+    }
     const bool wide = tile == 0 ? big_use_wide(args.M, args.N) : tile == 256;
     args.tiles_m = ceil_div(args.M, BIG_BM);
     args.tiles_n = ceil_div(args.N, wide ? 256 : 128);
-    const bool ktail = args.K % BIG_BK != 0;
-    if (wide) return ktail ? big_launch_one<256, 5, 8, EPI, true>(args, stream) : big_launch_one<256, 5, 8, EPI, false>(args, stream);
-    return ktail ? big_launch_one<128, 3, 4, EPI, true>(args, stream) : big_launch_one<128, 3, 4, EPI, false>(args, stream);
+    if (wide) return ktail ? big_launch_one<256, 256, 5, 8, EPI, true>(args, stream) : big_launch_one<256, 256, 5, 8, EPI, false>(args, stream);
+    return ktail ? big_launch_one<256, 128, 3, 4, EPI, true>(args, stream) : big_launch_one<256, 128, 3, 4, EPI, false>(args, stream);
 }
 
 static int big_check(const char* what, const void* x, int64_t ldx, const void* w, int64_t ldw, int m, int n, int k) {
@@ -583,8 +595,10 @@ extern "C" int somi_row_scale(const float* stats, int blocks, int width, int m, 
 }
 
 // Workgroup columns that write row statistics in the residual form: the first size of stats_out.
-// tile: 0 lets the launcher choose, 128 or 256 asks for that tile width.
+// tile: 0 lets the launcher choose (the 128-row tile up to 128 rows, else 256-row tiles of the width that fills the
+// device better); 128 or 256 asks for that width of the 256-row tile, 1 for the 128-row tile (128 x 256).
 extern "C" int somi_linear_big_stats_blocks(int m, int n, int tile) {
+    if (big_use_low(m, tile)) return ceil_div(n, 256) * 4;
     const bool wide = tile == 0 ? big_use_wide(m, n) : tile == 256;
     return wide ? ceil_div(n, 256) * 4 : ceil_div(n, 128) * 2;
 }
@@ -596,7 +610,7 @@ extern "C" int somi_linear_big(const void* x, int64_t ldx, const void* w, int64_
     if (big_check("linear_big", x, ldx, w, ldw, m, n, k) != 0) return 1;
     SOMI_REQUIRE(out != nullptr, "linear_big: no output");
     SOMI_REQUIRE(!swiglu || (n % 32 == 0 && bias == nullptr), "linear_big: the gated form needs N a multiple of 32 and no bias");
-    SOMI_REQUIRE(tile == 0 || tile == 128 || tile == 256, "linear_big: tile width %d (0, 128 or 256)", tile);
+    SOMI_REQUIRE(tile == 0 || tile == BIG_TILE_LOW || tile == 128 || tile == 256, "linear_big: tile code %d (0, 1, 128 or 256)", tile);
     BigArgs args = {};
     args.x = (const bf16*)x; args.ldx = ldx; args.w = (const bf16*)w; args.ldw = ldw; args.bias = bias;
     args.M = m; args.N = n; args.K = k; args.out = (bf16*)out;
@@ -614,7 +628,7 @@ extern "C" int somi_linear_big_residual(const void* x, int64_t ldx, const void* 
     SOMI_REQUIRE(h != nullptr, "linear_big_residual: no residual stream");
     SOMI_REQUIRE((weighted == nullptr) == (norm_w == nullptr), "linear_big_residual: the norm's weight and its rows come together");
     SOMI_REQUIRE(stats_out == nullptr || stats_width >= m, "linear_big_residual: row statistics of width %d do not cover %d rows", stats_width, m);
-    SOMI_REQUIRE(tile == 0 || tile == 128 || tile == 256, "linear_big_residual: tile width %d (0, 128 or 256)", tile);
+    SOMI_REQUIRE(tile == 0 || tile == BIG_TILE_LOW || tile == 128 || tile == 256, "linear_big_residual: tile code %d (0, 1, 128 or 256)", tile);
     BigArgs args = {};
     args.x = (const bf16*)x; args.ldx = ldx; args.w = (const bf16*)w; args.ldw = ldw; args.bias = bias;
     args.M = m; args.N = n; args.K = k; args.h = h; args.norm_w = norm_w; args.weighted = (bf16*)weighted;

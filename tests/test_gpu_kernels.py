@@ -627,11 +627,11 @@ def _interleave16(gate, up):
     return torch.stack([gate.view(-1, b, h), up.view(-1, b, h)], dim=1).reshape(-1, h).contiguous()
 
 
-@pytest.mark.parametrize("tile", [0, 128, 256])
+@pytest.mark.parametrize("tile", [0, 1, 128, 256])
 @pytest.mark.parametrize("m,n,k", BIG_SHAPES)
 def test_many_rows_product_plain_with_bias_and_row_scale(m, n, k, tile):
     """x . w^T (+ bias) against F.linear in float32, with tails in M, N and K (K = 200 and 72 end inside a stage,
-    K = 8 is one piece), for both tile widths; then the same with the rows scaled as an RMS norm would."""
+    K = 8 is one piece), for every tile (1: the 128-row tile that up to 128 rows take by themselves); then the same with the rows scaled as an RMS norm would."""
     x, w, bias = rnd(m, k, dtype="bfloat16", seed=1), rnd(n, k, dtype="bfloat16", seed=2, scale=0.3), rnd(n, seed=3)
     want = F.linear(x.float(), w.float(), bias)
     got = ops.linear_big(x, w, bias, tile=tile)
@@ -661,12 +661,12 @@ def test_many_rows_product_reads_strided_rows_and_refuses_what_it_cannot_take():
         ops.linear_big(rnd(70, 64, dtype="bfloat16"), rnd(8, 32, dtype="bfloat16"))
     with pytest.raises(KernelError, match="bfloat16"):
         ops.linear_big(rnd(70, 64), rnd(8, 64))
-    with pytest.raises(KernelError, match="tile width"):
+    with pytest.raises(KernelError, match="tile code"):
         ops.linear_big(rnd(70, 64, dtype="bfloat16"), rnd(8, 64, dtype="bfloat16"), tile=64)
 
 
-@pytest.mark.parametrize("tile", [128, 256])
-@pytest.mark.parametrize("m,inter,k", [(65, 16, 64), (130, 272, 200), (512, 1040, 192), (2048, 48, 72)])
+@pytest.mark.parametrize("tile", [0, 1, 128, 256])
+@pytest.mark.parametrize("m,inter,k", [(65, 16, 64), (100, 528, 136), (130, 272, 200), (512, 1040, 192), (2048, 48, 72)])
 def test_many_rows_product_with_the_gate_in_its_end(m, inter, k, tile):
     x = rnd(m, k, dtype="bfloat16", seed=6)
     gate, up = rnd(inter, k, dtype="bfloat16", seed=7, scale=0.2), rnd(inter, k, dtype="bfloat16", seed=8, scale=0.2)
@@ -683,8 +683,8 @@ def test_many_rows_product_with_the_gate_in_its_end(m, inter, k, tile):
     torch.testing.assert_close(got.float(), want, atol=0.02 * float(want.abs().max()) + 1e-3, rtol=2e-2)
 
 
-@pytest.mark.parametrize("tile", [0, 128, 256])
-@pytest.mark.parametrize("m,n,k", [(65, 132, 64), (300, 520, 200), (1024, 72, 1032), (257, 256, 136)])
+@pytest.mark.parametrize("tile", [0, 1, 128, 256])
+@pytest.mark.parametrize("m,n,k", [(65, 132, 64), (128, 600, 264), (300, 520, 200), (1024, 72, 1032), (257, 256, 136)])
 def test_many_rows_product_into_the_residual_stream(m, n, k, tile):
     """h += x . w^T + bias in float32, with the next norm's weighted rows and the rows' sums of squares; feeding
     those into the scaled product gives the product of the normed rows."""
