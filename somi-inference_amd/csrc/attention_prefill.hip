@@ -234,7 +234,7 @@ attention_prefill_kernel(const bf16* __restrict__ q, int64_t q_stride, const bf1
 //   different banks); V tile: [D channels][32 + 4 keys] (a row is 18 dwords: the 16 channels that an 8-byte
 //   read serves at once fall into different pairs of the 32 banks; with 20 dwords a row the counters showed
 //   twice the conflicts).
-#define PREFILL_LDS_PAGES 28672    // block-table entries of the visible range that LDS holds at most (112 KB beside the tiles)
+#define PREFILL_LDS_TOTAL (96 * 1024)   // LDS of a workgroup, tiles (static) and page list (dynamic) together, that a launch may ask for
 #ifndef PREFILL_WIDE_GROUPS
 #define PREFILL_WIDE_GROUPS 600    // from this many 128-query groups on, workgroups take 128 queries, else 64 (measured: 448 groups 72 against 82 us with 64 queries, 672 groups 136 against 119)
 #endif
@@ -563,6 +563,9 @@ attention_prefill_lds_kernel(const bf16* __restrict__ q, int64_t q_stride, const
 
 // Block-table entries a workgroup of the LDS kernel may list: the pages of its visible range (everything
 // before its last query, or a window and the workgroup's 128 queries) and a 32-key tile's overhang.
+// Static LDS of the LDS kernel: two buffers of KS key tiles [32][D + 8] and value tiles [D][36], bfloat16.
+static int prefill_lds_static(int D, int ks) { return 2 * ks * (32 * (D + 8) + D * 36) * 2; }
+
 static int prefill_page_entries(int max_blocks, int page_size, int window) {
     int entries = max_blocks + 16;                   // + the overhang of a step of two 32-key tiles, pages of 4 keys
     if (window > 0) entries = min(entries, (window + 128 + 128) / page_size + 16);
@@ -593,9 +596,10 @@ static int launch_prefill_lds(const void* q, int64_t q_stride, const void* kc, c
         hipLaunchKernelGGL((attention_prefill_lds_kernel<DT, 2, 1>), grid, dim3(256), page_list, stream, (const bf16*)q,
                            q_stride, (const bf16*)kc, (const bf16*)vc, block_table, max_blocks, entry_start,
                            entry_first_pos, entry_len, nq, nkv, page_size, window, scale * 1.44269504088896341f, (bf16*)out);
-    } else if (shape == PREFILL_SHAPE_AUTO
-                   ? (int64_t)grid.x * grid.y * grid.z < PREFILL_KEY_SPLIT_BELOW && reach >= PREFILL_KEY_SPLIT_REACH
-                   : shape == PREFILL_SHAPE_SPLIT) {
+    } else if ((shape == PREFILL_SHAPE_AUTO
+                    ? (int64_t)grid.x * grid.y * grid.z < PREFILL_KEY_SPLIT_BELOW && reach >= PREFILL_KEY_SPLIT_REACH
+                    : shape == PREFILL_SHAPE_SPLIT) &&
+               (int)page_list + prefill_lds_static(DT * 16, 2) <= PREFILL_LDS_TOTAL) {
         // few workgroups with many tiles each: the keys of a query block are split over two wavefronts
         if (page_list > 16 * 1024)
             (void)hipFuncSetAttribute((const void*)attention_prefill_lds_kernel<DT, 1, 2>,
@@ -684,7 +688,8 @@ extern "C" int somi_attention_prefill(const void* q, int64_t q_stride, const voi
     // head sizes 32..128 stage keys and values through LDS; the others (LDS would not hold two tiles, or a
     // tile is smaller than the workgroup's loads) keep them in registers per wavefront, and so do page sizes
     // that are no power of two and block tables too wide for the LDS copy of a request's pages
-    const bool lds_ok = (page_size & (page_size - 1)) == 0 && prefill_page_entries(max_blocks, page_size, window) <= PREFILL_LDS_PAGES;
+    const bool lds_ok = (page_size & (page_size - 1)) == 0 &&
+                        prefill_page_entries(max_blocks, page_size, window) * 4 + prefill_lds_static(D, 1) <= PREFILL_LDS_TOTAL;
     switch (D / 16) {
         SOMI_PREFILL(1, 4); SOMI_PREFILL_LDS(2); SOMI_PREFILL_LDS(3); SOMI_PREFILL_LDS(4); SOMI_PREFILL_LDS(5);
         SOMI_PREFILL_LDS(6); SOMI_PREFILL_LDS(7); SOMI_PREFILL_LDS(8); SOMI_PREFILL(9, 2); SOMI_PREFILL(10, 2);

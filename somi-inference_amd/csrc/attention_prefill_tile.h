@@ -4,7 +4,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
-#define SOMI_PREFILL_TILE_LDS_MAX (144 * 1024)   // dynamic LDS a workgroup of the kernel may ask for
+#define SOMI_PREFILL_TILE_LDS_MAX (112 * 1024)   // dynamic LDS a workgroup of the kernel may ask for (launches with 106 KB are tested)
 
 // Dynamic LDS of a launch with qblk query blocks and ks key splits a workgroup.
 int somi_prefill_tile_lds(int D, int qblk, int ks, int max_blocks, int page_size, int window);

@@ -753,6 +753,43 @@ def test_attention_prefill_tile_kernel_over_long_contexts(nq, nkv, d, page, wind
     torch.testing.assert_close(out.float(), want.float(), atol=2e-2, rtol=2e-2)
 
 
+@pytest.mark.parametrize("width, first", [(10_000, 150_000), (13_000, 200_000), (25_000, 390_000)])
+def test_attention_prefill_under_very_wide_block_tables(width, first):
+    """Contexts of hundreds of thousands of tokens: block tables of 10,000 pages (the tile kernel with a long list
+    of pages in LDS), of 13,000 (beyond what it holds beside its tiles: the 16 x 16 kernel with the list in dynamic
+    LDS) and of 25,000 (beyond that too: the kernel that reads the table from memory).  A portion of 130 tokens at
+    position `first` beside one of 70 from position 0; the logical pages share a pool of 500 physical ones, which
+    the plain kernel reads through the same table.  Queries are enlarged so that a few of the keys carry the sum."""
+    nq, nkv, d, page = 4, 2, 128, 16
+    cached, new = [first, 0], [130, 70]
+    pool = 500
+    columns = torch.arange(width)
+    block_table = torch.stack([1 + (columns * 7 + r) % pool for r in range(2)]).to(torch.int32).to(DEV)
+    kc = rnd(pool + 1, nkv, page, d, dtype="bfloat16", seed=71)
+    vc = rnd(pool + 1, nkv, d, page, dtype="bfloat16", seed=72)
+    n = sum(new)
+    q = rnd(n, nq * d, dtype="bfloat16", seed=73, scale=3.0)
+    positions, entry, starts = [], [], [0]
+    for e, (c, k) in enumerate(zip(cached, new)):
+        positions += [c + i for i in range(k)]
+        entry += [e] * k
+        starts.append(starts[-1] + k)
+    assert (max(positions) // page) < width
+    scale = d ** -0.5
+    want = ops.paged_attention_plain(q, nq * d, kc, vc, block_table, i32(entry), i32(positions), nq, 0, scale)
+    assert float(want.float().abs().max()) > 0.5, "the sums are flat: a wrong key would not show"
+    out = torch.full((n, nq * d), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ops.attention_prefill(q, nq * d, kc, vc, block_table, i32(starts), i32(cached), max(new), nq, 0, scale, out,
+                          max_context=first + 130)
+    torch.testing.assert_close(out.float(), want.float(), atol=3e-2, rtol=3e-2)
+    # single tokens at the far end, with the keys split over workgroups
+    last = [starts[1] - 1, n - 1]
+    dec = torch.full((n, nq * d), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ops.attention_decode(q, nq * d, kc, vc, block_table, i32(entry), i32(positions), nq, 0, scale, 2048, (first + 130 + 2047) // 2048,
+                         dec, token_list=i32(last))
+    torch.testing.assert_close(dec[last].float(), want[last].float(), atol=3e-2, rtol=3e-2)
+
+
 @pytest.mark.parametrize("nq, nkv, d, page, window", [(8, 2, 64, 16, 0), (6, 3, 128, 16, 21), (4, 1, 32, 8, 0), (14, 2, 256, 16, 0),
                                                      (5, 5, 80, 4, 9), (7, 1, 128, 8, 40), (4, 2, 64, 32, 0)])
 def test_attention_ignores_whatever_lies_beyond_a_requests_keys(nq, nkv, d, page, window):
