@@ -367,12 +367,14 @@ static int launch_tile(const void* q, int64_t q_stride, const void* kc, const vo
                        int max_entry_len, int nq, int nkv, int page_size, int window, float scale, void* out,
                        hipStream_t stream) {
     const int lds = somi_prefill_tile_lds(D, QBLK, KS, max_blocks, page_size, window);
-    static int lds_allowed = 0;                  // the largest dynamic LDS this kernel has been allowed so far
-    if (lds > lds_allowed) {
+    static int lds_allowed[64];                  // per device: the largest dynamic LDS this kernel has been allowed so far
+    int device = 0;
+    if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) return somi_fail("attention_prefill_tile: hipGetDevice failed");
+    if (lds > lds_allowed[device]) {
         const hipError_t err = hipFuncSetAttribute((const void*)prefill_tile_kernel<D, QBLK, KS>,
                                                    hipFuncAttributeMaxDynamicSharedMemorySize, lds);
         if (err != hipSuccess) return somi_fail("attention_prefill_tile: %d bytes of LDS refused: %s", lds, hipGetErrorString(err));
-        lds_allowed = lds;
+        lds_allowed[device] = lds;
     }
     const dim3 grid(nq, n_entries, ceil_div(max_entry_len, QBLK * 32));
     hipLaunchKernelGGL((prefill_tile_kernel<D, QBLK, KS>), grid, dim3(QBLK * KS * 64), lds, stream, (const bf16*)q, q_stride,
