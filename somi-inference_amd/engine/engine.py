@@ -111,7 +111,7 @@ class Engine:
             tokens = draw(
                 logits,
                 [p.request.sampling_params for p in sampled],
-                token_histories=[p.request.all_tokens for p in sampled],
+                token_histories=[p.request.tokens for p in sampled],
                 seeds=[p.request.seed for p in sampled],
                 counters=[len(p.request.output_tokens) for p in sampled],
             )

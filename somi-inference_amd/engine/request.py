@@ -3,8 +3,10 @@
 
 from __future__ import annotations
 
+from collections.abc import Sequence
 from dataclasses import dataclass, field
 from enum import Enum
+from itertools import chain, islice
 from typing import Hashable
 
 from ..sampling.params import SamplingParams
@@ -16,7 +18,45 @@ class RequestStatus(Enum):
     FINISHED = "finished"
 
 
-@dataclass
+class TokenView(Sequence):
+    """A request's prompt and output tokens as one sequence, without copying them (a request of thousands of tokens
+    is looked at in every step)."""
+
+    __slots__ = ("prompt", "output")
+
+    def __init__(self, prompt: list[int], output: list[int]) -> None:
+        self.prompt, self.output = prompt, output
+
+    def __len__(self) -> int:
+        return len(self.prompt) + len(self.output)
+
+    def __iter__(self):
+        return chain(self.prompt, self.output)
+
+    def __getitem__(self, index):
+        if isinstance(index, slice):
+            start, stop, step = index.indices(len(self))
+            if step != 1:
+                return list(self)[index]
+            split = len(self.prompt)
+            if stop <= split:
+                return self.prompt[start:stop]
+            if start >= split:
+                return self.output[start - split:stop - split]
+            return self.prompt[start:] + self.output[:stop - split]
+        if index < 0:
+            index += len(self)
+        split = len(self.prompt)
+        return self.prompt[index] if index < split else self.output[index - split]
+
+    def __eq__(self, other) -> bool:
+        return len(self) == len(other) and all(a == b for a, b in zip(self, other))
+
+    def __repr__(self) -> str:
+        return f"TokenView({list(islice(self, 8))}{'...' if len(self) > 8 else ''}, {len(self)} tokens)"
+
+
+@dataclass(eq=False)          # a request is itself: queues look it up by identity, not by comparing token lists
 class Request:
     request_id: Hashable
     prompt_tokens: list[int]
@@ -38,6 +78,15 @@ class Request:
     @property
     def all_tokens(self) -> list[int]:
         return self.prompt_tokens + self.output_tokens
+
+    @property
+    def tokens(self) -> TokenView:
+        """Prompt and output tokens as one sequence (a view, not a copy)."""
+        return TokenView(self.prompt_tokens, self.output_tokens)
+
+    @property
+    def num_tokens(self) -> int:
+        return len(self.prompt_tokens) + len(self.output_tokens)
 
     @property
     def num_pending(self) -> int:

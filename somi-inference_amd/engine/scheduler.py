@@ -160,46 +160,45 @@ class Scheduler:
             return count
         return count - count % self.granule
 
-    def _fit(self, request: Request, want: int, taken: list[int]) -> int:
-        """Largest portion <= want whose pages are free after what this step already took."""
+    def _fit(self, request: Request, want: int, taken: list[int]) -> tuple[int, list[int]]:
+        """Largest portion <= want whose pages are free after what this step already took, and the pages it
+        takes in each group."""
         free = [f - t for f, t in zip(self.cache.free_pages(), taken)]
         count = self._whole(request, want)
         while count > 0:
             need = self.cache.pages_needed(request.request_id, count)
             if all(n <= f for n, f in zip(need, free)):
-                return count
+                return count, need
             # shrink to the end of the last page that still fits
             count = self._whole(request, min(count - 1, self.cache.tokens_within(request.request_id, free)))
-        return 0
+        return 0, [0] * len(free)
 
     def schedule(self) -> SchedulerOutput:
         output = SchedulerOutput()
         budget = self.max_num_batched_tokens
         taken = [0] * len(self.cache.groups)
 
-        def take(request: Request, count: int) -> None:
+        def take(request: Request, count: int, need: list[int]) -> None:
             nonlocal budget
-            need = self.cache.pages_needed(request.request_id, count)
             for g, n in enumerate(need):
                 taken[g] += n
             start = request.num_computed
-            tokens = request.all_tokens[start:start + count]
-            output.portions.append(ScheduledPortion(request, start, tokens,
-                                                    samples=start + count == len(request.all_tokens)))
+            output.portions.append(ScheduledPortion(request, start, request.tokens[start:start + count],
+                                                    samples=start + count == request.num_tokens))
             budget -= count
 
         # 1. running requests: those that decode first, then those with prompt left
         order = [r for r in self.running if r.num_pending == 1] + [r for r in self.running if r.num_pending > 1]
         for request in order:
-            if request not in self.running or budget <= 0:
-                continue
+            if request.status is not RequestStatus.RUNNING or budget <= 0:
+                continue                     # preempted in this step, or nothing left to give
             want = self._whole(request, min(request.num_pending, self.chunk, budget))
             if want == 0:
                 continue                     # what is left of the budget does not hold a granule: next step
             while True:
-                count = self._fit(request, want, taken)
+                count, need = self._fit(request, want, taken)
                 if count > 0:
-                    take(request, count)
+                    take(request, count, need)
                     break
                 if self.running[-1] is request and len(self.running) == 1:
                     raise SchedulerError(
@@ -222,7 +221,7 @@ class Scheduler:
             if want == 0:
                 break
             self.cache.register(request.request_id)
-            count = self._fit(request, want, taken)
+            count, need = self._fit(request, want, taken)
             if count < want:
                 self.cache.free(request.request_id)     # the pages of its first portion are not free: wait
                 break
@@ -230,5 +229,5 @@ class Scheduler:
             request.status = RequestStatus.RUNNING
             self.running.append(request)
             output.admitted.append(request)
-            take(request, count)
+            take(request, count, need)
         return output
