@@ -51,8 +51,8 @@ template <int MT, int NS, int MODE, typename TO, bool SWIGLU, bool TAIL, bool RO
 __global__ void __launch_bounds__(FUSED_MAX_WAVES * 64)
 linear_fused_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, const float* __restrict__ bias,
                     TO* __restrict__ out, float* __restrict__ h, const float* __restrict__ norm_w, float eps,
-                    const float* __restrict__ stats_in, int stats_blocks, float* __restrict__ stats_out,
-                    bf16* __restrict__ xnext, int M, int N, int K, FusedRope rope) {
+                    const float* __restrict__ stats_in, int stats_blocks, int stats_stride,
+                    float* __restrict__ stats_out, bf16* __restrict__ xnext, int M, int N, int K, FusedRope rope) {
     extern __shared__ __attribute__((aligned(16))) char lds[];
     __shared__ float row_scale[64];
     __shared__ float part[FUSED_MAX_WAVES * 4 * 16 * MT];
@@ -138,7 +138,8 @@ linear_fused_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, cons
     u32x4 A[NL], B[NL];
     if (mine_n >= 1) issue(A, 0);                    // the first loads are under way while what follows is fetched
     if (mine_n >= 2) issue(B, 1);
-    // The rows' scales come from the producer's partial sums of squares [stats_blocks][ROWS], added in a fixed
+    // The rows' scales come from the producer's partial sums of squares [stats_blocks][ROWS] (stats_stride floats
+    // from one workgroup's sums to the next: these rows may be some of the rows of a longer table), added in a fixed
     // order: lane l of wavefront v adds the rows MT (l % 16) .. + MT - 1 (one load) of the workgroups
     // 4 v + l / 16, that + 4 waves, ...; then a thread per row adds those sums in order.  The first loads go
     // out here, before the weight stream, and are only looked at after it.
@@ -146,7 +147,7 @@ linear_fused_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, cons
     float early[EARLY][MT];
     const int stats_group = wave * 4 + g, stats_groups = waves * 4;
     auto stats_load = [&](float (&to)[MT], int block) {
-        const float* from = stats_in + (int64_t)block * ROWS + r * MT;
+        const float* from = stats_in + (int64_t)block * stats_stride + r * MT;
         if (block < stats_blocks) {
             __builtin_memcpy(&to[0], __builtin_assume_aligned(from, MT == 3 ? 4 : 4 * MT), 4 * MT);
         } else {
@@ -397,8 +398,8 @@ static int fused_waves(int K) {
 template <int MT, int NS, int MODE, typename TO, bool SW, bool TL, bool ROPE>
 static void fused_launch_kernel(const void* x, const void* w, const float* bias, void* out, float* h,
                                 const float* norm_w, float eps, const float* stats_in, int stats_blocks,
-                                float* stats_out, void* xnext, int M, int N, int K, const FusedRope& rope,
-                                hipStream_t stream) {
+                                int stats_stride, float* stats_out, void* xnext, int M, int N, int K,
+                                const FusedRope& rope, hipStream_t stream) {
     const int waves = fused_waves(K);
     const dim3 grid(ROPE ? (rope.nq + 2 * rope.nkv) * (rope.D / 32) : ceil_div(N, 16 * NS)), block(waves * 64);
     const size_t smem = fused_lds(MT, NS, waves);
@@ -406,21 +407,22 @@ static void fused_launch_kernel(const void* x, const void* w, const float* bias,
         (void)hipFuncSetAttribute((const void*)linear_fused_kernel<MT, NS, MODE, TO, SW, TL, ROPE>,
                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     hipLaunchKernelGGL((linear_fused_kernel<MT, NS, MODE, TO, SW, TL, ROPE>), grid, block, smem, stream,
-                       (const bf16*)x, (const bf16*)w, bias, (TO*)out, h, norm_w, eps, stats_in, stats_blocks, stats_out,
-                       (bf16*)xnext, M, N, K, rope);
+                       (const bf16*)x, (const bf16*)w, bias, (TO*)out, h, norm_w, eps, stats_in, stats_blocks,
+                       stats_stride > 0 ? stats_stride : 16 * MT, stats_out, (bf16*)xnext, M, N, K, rope);
 }
 
 template <int NS, int MODE, typename TO, bool SW, bool ROPE = false>
 static int fused_launch(const void* x, const void* w, const float* bias, void* out, float* h, const float* norm_w,
                         float eps, const float* stats_in, int stats_blocks, float* stats_out, void* xnext, int M, int N,
-                        int K, hipStream_t stream, const FusedRope& rope = FusedRope{}) {
+                        int K, hipStream_t stream, const FusedRope& rope = FusedRope{}, int stats_stride = 0) {
     const bool tail = K % FUSED_CK != 0;
 #define SOMI_FUSED(MT)                                                                                               \
     if (tail) fused_launch_kernel<MT, NS, MODE, TO, SW, true, ROPE>(x, w, bias, out, h, norm_w, eps, stats_in,          \
-                                                                    stats_blocks, stats_out, xnext, M, N, K, rope,    \
-                                                                    stream);                                          \
+                                                                    stats_blocks, stats_stride, stats_out, xnext, M, \
+                                                                    N, K, rope, stream);                              \
     else fused_launch_kernel<MT, NS, MODE, TO, SW, false, ROPE>(x, w, bias, out, h, norm_w, eps, stats_in,             \
-                                                                stats_blocks, stats_out, xnext, M, N, K, rope, stream); \
+                                                                stats_blocks, stats_stride, stats_out, xnext, M, N,  \
+                                                                K, rope, stream);                                     \
     break
     switch (ceil_div(M, 16)) {
         case 1: SOMI_FUSED(1);
@@ -484,8 +486,9 @@ extern "C" int somi_linear_scaled(const void* x, float eps, const float* stats, 
 // first; with stats == null x is used as it is.  q: [M, nq D] bfloat16, out, rotated; k (rotated) and v go to
 // their pages: k_cache [pages, nkv, page_size, D], v_cache [pages, nkv, D, page_size], slot of row m =
 // page * page_size + offset or -1.  positions: [M] int32; inv_freq: [D / 2] float32 (the whole head is
-// rotated).  D must be a multiple of 32, M <= 64.
-extern "C" int somi_linear_rope_store(const void* x, float eps, const float* stats, int stats_blocks, const void* w,
+// rotated).  D must be a multiple of 32, M <= 64.  stats_stride: floats from one workgroup's sums to the next where
+// the M rows are some of the rows of a longer table (a multiple of 4), or 0 for 16 ceil(M / 16).
+extern "C" int somi_linear_rope_store(const void* x, float eps, const float* stats, int stats_blocks, int stats_stride, const void* w,
                                       const float* bias, void* q, const int* positions, const int* slots,
                                       const float* inv_freq, void* k_cache, void* v_cache, int nq, int nkv, int D,
                                       int page_size, int M, int K, hipStream_t stream) {
@@ -498,11 +501,13 @@ extern "C" int somi_linear_rope_store(const void* x, float eps, const float* sta
                  "linear_rope_store: q, positions, slots, inv_freq and the caches are needed");
     SOMI_REQUIRE((uintptr_t)q % 8 == 0 && (uintptr_t)k_cache % 8 == 0, "linear_rope_store: q and the k cache must be 8-byte aligned");
     SOMI_REQUIRE(!stats || (stats_blocks > 0 && (uintptr_t)stats % 16 == 0), "linear_rope_store: bad row statistics");
+    SOMI_REQUIRE(stats_stride == 0 || (stats_stride % 4 == 0 && stats_stride >= 16 * ceil_div(M, 16)),
+                 "linear_rope_store: a stride of %d floats does not hold the sums of %d rows", stats_stride, M);
     if (M == 0) return 0;
     const FusedRope rope{positions, slots, inv_freq, (bf16*)k_cache, (bf16*)v_cache, nq, nkv, D, page_size};
     if (stats)
         return fused_launch<2, FUSED_SCALED, bf16, false, true>(x, w, bias, q, nullptr, nullptr, eps, stats, stats_blocks,
-                                                                nullptr, nullptr, M, N, K, stream, rope);
+                                                                nullptr, nullptr, M, N, K, stream, rope, stats_stride);
     return fused_launch<2, 0, bf16, false, true>(x, w, bias, q, nullptr, nullptr, 0.f, nullptr, 0, nullptr, nullptr, M, N, K,
                                                  stream, rope);
 }

@@ -13,7 +13,11 @@ MAX_SPLITS = 1024               # what the merge kernel holds
 DECODE_PORTION = 8              # portions of at most this many tokens take the decode kernel (engine.batch.SHORT_ENTRY)
 
 
-def decode_splits(num_tokens: int, groups: int, max_context: int, page_size: int = 0) -> tuple[int, int]:
+UNIT_HEAD_DIM = 128             # workgroups per compute unit: UNIT_HEAD_DIM / head size, at least one
+
+
+def decode_splits(num_tokens: int, groups: int, max_context: int, page_size: int = 0,
+                  head_dim: int = 128) -> tuple[int, int]:
     """(split_len, num_splits): how the keys of a request are cut over workgroups so that
     ``num_tokens * groups * num_splits`` is about the number of compute units.  Boundaries are multiples of
     MIN_SPLIT in absolute positions.  With ``page_size`` a split is no longer than what the kernel that stages
@@ -22,7 +26,8 @@ def decode_splits(num_tokens: int, groups: int, max_context: int, page_size: int
     against 6.8 at 3,9xx tokens)."""
     max_context = max(1, max_context)
     most = (max_context + MIN_SPLIT - 1) // MIN_SPLIT
-    splits = max(1, min(ops.compute_units() // max(1, num_tokens * groups), most, MAX_SPLITS))
+    workgroups = ops.compute_units() * max(1, UNIT_HEAD_DIM // max(1, head_dim))
+    splits = max(1, min(workgroups // max(1, num_tokens * groups), most, MAX_SPLITS))
     split_len = ((max_context + splits - 1) // splits + MIN_SPLIT - 1) // MIN_SPLIT * MIN_SPLIT
     if page_size > 0:
         longest = ops.library().somi_attention_decode_lds_split(int(page_size))
@@ -60,11 +65,11 @@ def paged_attention(qkv: torch.Tensor, num_heads: int, k_cache: torch.Tensor, v_
                               step.entry_first_position, step.max_entry_len, num_heads, window, scale, out,
                               max_context=step.max_context, entry_len=step.long_entry_len if short else None)
         if short:
-            split_len, num_splits = decode_splits(short, groups, step.max_context, k_cache.shape[2])
+            split_len, num_splits = decode_splits(short, groups, step.max_context, k_cache.shape[2], head_dim)
             ops.attention_decode(qkv, qkv.shape[1], k_cache, v_cache, block_table, step.token_entry, step.positions,
                                  num_heads, window, scale, split_len, num_splits, out, token_list=step.short_tokens)
         return out
-    split_len, num_splits = decode_splits(step.num_tokens, groups, step.max_context, k_cache.shape[2])
+    split_len, num_splits = decode_splits(step.num_tokens, groups, step.max_context, k_cache.shape[2], head_dim)
     ops.attention_decode(qkv, qkv.shape[1], k_cache, v_cache, block_table, step.token_entry, step.positions,
                          num_heads, window, scale, split_len, num_splits, out)
     return out

@@ -50,9 +50,11 @@ def linear_residual(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | 
         # many-rows kernel are too few to fill the device (28 workgroups at 7B sizes: 61 us), two passes of the
         # few-rows kernel are not (2 x 14 us)
         stats, weighted = [], []
+        # one kernel for every pass, the short last one too: the passes' statistics have one row per workgroup and
+        # are laid side by side
+        mid = _mid_is_faster(ops.FUSED_MAX_ROWS, n, x.shape[1])
         for at in range(0, m, ops.FUSED_MAX_ROWS):
             rows = slice(at, at + ops.FUSED_MAX_ROWS)
-            mid = _mid_is_faster(min(ops.FUSED_MAX_ROWS, m - at), n, x.shape[1])
             part_stats, part_weighted = ops.linear_residual(x[rows], weight, bias, h[rows], next_norm_weight, mid=mid)
             stats.append(part_stats)
             weighted.append(part_weighted)

@@ -338,6 +338,9 @@ def _stats_width(rows: int) -> int:
     return 16 * ((rows + 15) // 16)
 
 
+stats_width = _stats_width          # columns of the row statistics of this many rows
+
+
 def _big_operands(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, what: str) -> tuple[int, int, int]:
     """Checks what the many-rows kernel assumes of its operands; x may be a view with a row stride of its own."""
     for t, name in ((x, "input"), (weight, "weight")):
@@ -477,21 +480,26 @@ def linear_scaled(x: torch.Tensor, eps: float, stats: torch.Tensor, weight: torc
 
 def linear_rope_store(x: torch.Tensor, eps: float, stats: torch.Tensor | None, weight: torch.Tensor,
                       bias: torch.Tensor | None, positions: torch.Tensor, slots: torch.Tensor, inv_freq: torch.Tensor,
-                      nq: int, nkv: int, head_dim: int, k_cache: torch.Tensor, v_cache: torch.Tensor) -> torch.Tensor:
+                      nq: int, nkv: int, head_dim: int, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                      out: torch.Tensor | None = None) -> torch.Tensor:
     """The q/k/v product of at most 64 bfloat16 rows with the rotary encoding of q and k and the store of k and v
     into their cache pages in its end -> q [M, nq * D], rotated.  weight: [(nq + 2 nkv) * D, K], q heads, k
     heads, v heads.  With ``stats`` x holds ``norm_weight * h`` and the sums are scaled per row as in
-    :func:`linear_scaled`; without, x is used as it is.  The whole head is rotated (inv_freq: [D / 2]); D must be
-    a multiple of 32."""
+    :func:`linear_scaled` (``stats`` may be the columns of these rows in the table of more rows); without, x is
+    used as it is.  The whole head is rotated (inv_freq: [D / 2]); D must be a multiple of 32."""
     _need(x, "linear input", torch.bfloat16)
     m, k = x.shape
     _need(weight, "q/k/v weight", torch.bfloat16, ((nq + 2 * nkv) * head_dim, k))
     if bias is not None:
         _need(bias, "q/k/v bias", torch.float32, (weight.shape[0],))
+    stats_stride = 0
     if stats is not None:
-        _need(stats, "row statistics", torch.float32)
-        if stats.dim() != 2 or stats.shape[1] != _stats_width(m):
-            raise KernelError(f"linear_rope_store: row statistics must be [blocks, {_stats_width(m)}], got {tuple(stats.shape)}")
+        if not isinstance(stats, torch.Tensor) or not stats.is_cuda or stats.dtype != torch.float32:
+            raise KernelError("linear_rope_store: row statistics must be a float32 tensor on the GPU")
+        if stats.dim() != 2 or stats.shape[1] != _stats_width(m) or stats.stride(1) != 1 or stats.stride(0) % 4:
+            raise KernelError(f"linear_rope_store: row statistics must be [blocks, {_stats_width(m)}] with rows of "
+                              f"consecutive floats, got {tuple(stats.shape)} with strides {stats.stride()}")
+        stats_stride = stats.stride(0)
     _need(positions, "positions", torch.int32, (m,))
     _need(slots, "slot mapping", torch.int32, (m,))
     _need(inv_freq, "inv_freq", torch.float32, (head_dim // 2,))
@@ -499,9 +507,13 @@ def linear_rope_store(x: torch.Tensor, eps: float, stats: torch.Tensor | None, w
     if k_cache.dim() != 4 or k_cache.shape[1] != nkv or k_cache.shape[3] != head_dim:
         raise KernelError(f"linear_rope_store: cache shape {tuple(k_cache.shape)} != [pages, {nkv}, page, {head_dim}]")
     _need(v_cache, "v cache", torch.bfloat16, _v_shape(k_cache))
-    q = torch.empty((m, nq * head_dim), dtype=torch.bfloat16, device=x.device)
+    if out is None:
+        q = torch.empty((m, nq * head_dim), dtype=torch.bfloat16, device=x.device)
+    else:
+        _need(out, "q", torch.bfloat16, (m, nq * head_dim))
+        q = out
     _check(library().somi_linear_rope_store(_ptr(x), ctypes.c_float(eps), _ptr(stats),
-                                            stats.shape[0] if stats is not None else 0, _ptr(weight), _ptr(bias),
+                                            stats.shape[0] if stats is not None else 0, stats_stride, _ptr(weight), _ptr(bias),
                                             _ptr(q), _ptr(positions), _ptr(slots), _ptr(inv_freq), _ptr(k_cache),
                                             _ptr(v_cache), nq, nkv, head_dim, k_cache.shape[2], m, k, _stream()))
     return q

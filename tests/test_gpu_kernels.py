@@ -555,6 +555,29 @@ def test_products_fused_with_the_residual_add_and_the_norm(m, hidden, n_out, int
         ops.linear_residual(rnd(65, inter, dtype="bfloat16"), w1, None, rnd(65, hidden), mid=mid)
 
 
+@pytest.mark.parametrize("m", [65, 70, 96, 128])
+@pytest.mark.parametrize("n, k", [(192, 8200), (136, 264)])
+def test_product_into_the_stream_of_65_to_128_rows(m, n, k):
+    """The chooser's passes of 64 rows (with a long K: of the kernel that splits K, the short last pass too), their
+    statistics side by side, and the product that reads them."""
+    from somi_inference_amd.kernels import linear as chooser
+    x = rnd(m, k, dtype="bfloat16", seed=1)
+    w1, b1 = rnd(n, k, dtype="bfloat16", seed=2, scale=0.1), rnd(n, seed=3)
+    h = rnd(m, n, seed=4, scale=2.0)
+    norm_w = 1.0 + rnd(n, seed=5, scale=0.1)
+    want_h = h + F.linear(x.float(), w1.float(), b1)
+    got_h = h.clone()
+    stats, weighted = chooser.linear_residual(x, w1, b1, got_h, norm_w)
+    torch.testing.assert_close(got_h, want_h, atol=2e-5 * float(want_h.abs().max()) * math.sqrt(k), rtol=1e-5)
+    assert stats.shape[1] == 16 * ((m + 15) // 16)
+    torch.testing.assert_close(stats.sum(dim=0)[:m], got_h.pow(2).sum(dim=1), rtol=1e-5, atol=1e-6)
+    assert torch.equal(weighted, (norm_w * got_h).to(torch.bfloat16))
+    w2 = rnd(80, n, dtype="bfloat16", seed=6, scale=0.05)
+    got = chooser.linear_scaled(weighted, 1e-5, stats, w2)
+    want = F.linear(plain_rms(got_h, norm_w, 1e-5), w2.float())
+    torch.testing.assert_close(got.float(), want, atol=float(want.abs().max()) * 2 ** -6, rtol=2 ** -6)
+
+
 @pytest.mark.parametrize("scaled", [True, False], ids=["normed", "as-is"])
 @pytest.mark.parametrize("m, nq, nkv, d, hidden, page", [(1, 4, 2, 32, 64, 16), (9, 12, 2, 64, 200, 8), (16, 3, 3, 128, 520, 4),
                                                          (24, 6, 2, 96, 264, 8), (37, 5, 1, 96, 1000, 16), (64, 28, 4, 128, 3584, 16)])
@@ -607,6 +630,17 @@ def test_qkv_product_with_the_rotation_and_the_cache_store(m, nq, nkv, d, hidden
     ops.rope_kv_store(qkv, positions, slots, inv_freq, d, nq, nkv, d, kc2, vc2)
     # the same sums in the same order, rounded at the same places: the same bits
     assert torch.equal(q, qkv[:, :nq * d]) and torch.equal(kc, kc2) and torch.equal(vc, vc2)
+    if scaled:
+        # the rows' sums as some columns of the table of more rows, q into a given tensor: the same bits again
+        table = torch.full((3, 64 + stats.shape[1] + 16), 1e9, device=DEV)
+        table[:, 64:64 + stats.shape[1]] = stats
+        kc3, vc3, q3 = torch.zeros_like(kc), torch.zeros_like(vc), torch.full_like(q, 3.0)
+        assert ops.linear_rope_store(x, eps, table[:, 64:64 + stats.shape[1]], w, b, positions, slots, inv_freq, nq, nkv, d,
+                                     kc3, vc3, out=q3) is q3
+        assert torch.equal(q, q3) and torch.equal(kc, kc3) and torch.equal(vc, vc3)
+        with pytest.raises(KernelError, match="consecutive floats"):
+            ops.linear_rope_store(x, eps, table[:, 1:2 * stats.shape[1]:2][:, :stats.shape[1]], w, b, positions, slots,
+                                  inv_freq, nq, nkv, d, kc3, vc3)
     with pytest.raises(KernelError, match="multiple of 32"):
         ops.linear_rope_store(x, eps, stats, rnd(4 * 48, hidden, dtype="bfloat16"), None, positions, slots,
                               plain.rope_inv_freq(48, theta).to(DEV), 2, 1, 48,

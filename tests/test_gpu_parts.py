@@ -108,6 +108,39 @@ def test_attention_part_whole_and_in_portions(dtype, nq, nkv, d, hidden, window)
         close(torch.cat(outs), want, dtype)
 
 
+@pytest.mark.parametrize("n_rows", [40, 64, 65, 81, 100, 128, 129])
+def test_attention_part_reads_rows_still_to_be_normed(n_rows):
+    """bfloat16 rows as a product into the residual stream leaves them (weighted, with their sums of squares): up to 64
+    the q/k/v product norms, rotates and stores them in one kernel, up to 128 in passes of 64 that cut through a
+    request, beyond by the many-rows kernels.  Three requests' prompts in one step."""
+    from somi_inference_amd.parts.linear import NormedRows
+    nq, nkv, d, hidden = 8, 2, 32, 72
+    attn, w, cache, cfg = attention_setup("bfloat16", nq, nkv, d, hidden, block_size=8)
+    ffn = SwiGLU("m", hidden_size=hidden, intermediate_size=96)
+    wf = load_random(ffn, "bfloat16", scale=4.0)
+    norm = RMSNorm("n", hidden_size=hidden, eps=1e-5)
+    wn = load_random(norm, "bfloat16")
+    h0 = torch.randn(n_rows, hidden, device=DEV)
+    x0 = norm.forward(h0)
+    stream = ResidualStream(h0.clone())
+    stream.add(ffn.forward(x0))
+    lazy = stream.normed(norm, lazy=True)
+    assert isinstance(lazy, NormedRows)
+    sizes = [n_rows // 2, n_rows // 3, n_rows - n_rows // 2 - n_rows // 3]
+    for i, size in enumerate(sizes):
+        cache.register(i)
+        cache.reserve(i, size)
+    step = build_step([StepEntry(i, [0] * size, []) for i, size in enumerate(sizes)], cache, DEV)
+    got = rows(attn.forward(lazy, step, cache.layer_caches[0]))
+    h1 = h0.cpu() + plain.swiglu(x0.float().cpu(), wf["m.gate_proj.weight"], wf["m.up_proj.weight"], wf["m.down_proj.weight"])
+    x1 = plain.rms_norm(h1, wn["n.weight"], 1e-5)
+    at = 0
+    for size in sizes:
+        want = plain.attention_block(x1[at:at + size], w, "a", cfg, torch.arange(size), None)
+        close(got[at:at + size], want, "bfloat16")
+        at += size
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_attention_part_far_key_among_hundreds_and_window_edge(dtype):
     """One query and one far key are made to agree strongly, so that key alone decides the output:
