@@ -368,7 +368,7 @@ linear_fused_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, cons
             float total = 0.f;
             for (int s = 0; s < NS; ++s)
                 for (int gg = 0; gg < 4; ++gg) total += part[(s * MT + mt) * 64 + gg * 16 + rr];
-            stats_out[blockIdx.x * ROWS + threadIdx.x] = total;
+            stats_out[(int64_t)blockIdx.x * stats_stride + threadIdx.x] = total;
         }
     }
 }
@@ -450,16 +450,20 @@ extern "C" int somi_linear_residual_blocks(int M, int N) { return ceil_div(N, 16
 // h[m, n] += x[m, :] . w[n, :] (+ bias[n]).  x: [M, K] bfloat16; w: [N, K] bfloat16; bias: [N] float32 or null;
 // h: [M, N] float32, in and out; stats: [somi_linear_residual_blocks(M, N)][16 ceil(M / 16)] float32, out: per
 // workgroup and row the sum of squares of the new h over the workgroup's columns (rows from M on: 0); xnext:
-// [M, N] bfloat16, out, = norm_w[n] * h[m, n] (norm_w: [N] float32), or null.  M <= 64.
+// [M, N] bfloat16, out, = norm_w[n] * h[m, n] (norm_w: [N] float32), or null.  M <= 64.  stats_stride: floats from
+// one workgroup's sums to the next where they are columns of the table of more rows (a multiple of 4), or 0.
 extern "C" int somi_linear_residual(const void* x, const void* w, const float* bias, float* h, float* stats,
-                                    const float* norm_w, void* xnext, int M, int N, int K, hipStream_t stream) {
+                                    int stats_stride, const float* norm_w, void* xnext, int M, int N, int K,
+                                    hipStream_t stream) {
     if (fused_check(x, w, M, N, K)) return 1;
     SOMI_REQUIRE(h && stats, "linear_residual: h and stats are needed");
     SOMI_REQUIRE(!xnext || norm_w, "linear_residual: the next rows need the norm's weight");
+    SOMI_REQUIRE(stats_stride == 0 || (stats_stride % 4 == 0 && stats_stride >= 16 * ceil_div(M, 16)),
+                 "linear_residual: a stride of %d floats does not hold the sums of %d rows", stats_stride, M);
     if (M == 0) return 0;
     if (fused_strips(M, N, false) >= 2)
-        return fused_launch<2, FUSED_RESIDUAL, float, false>(x, w, bias, nullptr, h, norm_w, 0.f, nullptr, 0, stats, xnext, M, N, K, stream);
-    return fused_launch<1, FUSED_RESIDUAL, float, false>(x, w, bias, nullptr, h, norm_w, 0.f, nullptr, 0, stats, xnext, M, N, K, stream);
+        return fused_launch<2, FUSED_RESIDUAL, float, false>(x, w, bias, nullptr, h, norm_w, 0.f, nullptr, 0, stats, xnext, M, N, K, stream, FusedRope{}, stats_stride);
+    return fused_launch<1, FUSED_RESIDUAL, float, false>(x, w, bias, nullptr, h, norm_w, 0.f, nullptr, 0, stats, xnext, M, N, K, stream, FusedRope{}, stats_stride);
 }
 
 // out = s * (x . w^T) (+ bias) with the row scales s[m] = 1 / sqrt(sum of stats[:, m] / K + eps), or with swiglu

@@ -38,6 +38,7 @@ struct MidFusion {
     const float* norm_w;      // residual: the next norm's weight [N], or null
     bf16* xnext;              // residual: [M, N] = bfloat16(norm_w * h), or null
     float* stats_out;         // residual: [column tiles][16 MT] sums of squares of the new h over the tile's columns
+    int stats_stride;         // floats from one row of either table to the next, or 0 for 16 MT
     const float* stats_in;    // scaled: [stats_blocks][16 MT] partial sums of squares of the rows that were normed
     int stats_blocks;
     float eps;
@@ -383,8 +384,9 @@ linear_mid_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, const 
         return;
     }
     MidAhead<MT, NS, FUSE> ahead;
-    mid_fetch_ahead(ahead, fusion, M, N, bias, n0, 16 * MT, 0);
-    mid_finish<MT, NS, TO, SWIGLU, FUSE>(acc, ahead, bias, out, fusion, M, N, K, n0, tile, 16 * MT, 0);
+    const int stats_stride = fusion.stats_stride > 0 ? fusion.stats_stride : 16 * MT;
+    mid_fetch_ahead(ahead, fusion, M, N, bias, n0, stats_stride, 0);
+    mid_finish<MT, NS, TO, SWIGLU, FUSE>(acc, ahead, bias, out, fusion, M, N, K, n0, tile, stats_stride, 0);
 }
 
 // Adds the partial sums of the splits in split order and applies the epilogue: one workgroup per column tile
@@ -395,7 +397,8 @@ linear_mid_reduce_kernel(const float* __restrict__ partial, const float* __restr
                          int M, int N, int K, int splits, MidFusion fusion) {
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, tile = blockIdx.x, mt = blockIdx.y;
     MidAhead<1, NS, FUSE> ahead;
-    mid_fetch_ahead(ahead, fusion, M, N, bias, tile * (64 * NS), 16 * MT, 16 * mt);
+    const int stats_stride = fusion.stats_stride > 0 ? fusion.stats_stride : 16 * MT;
+    mid_fetch_ahead(ahead, fusion, M, N, bias, tile * (64 * NS), stats_stride, 16 * mt);
     f32x4 acc[NS][1];
 #pragma unroll
     for (int s = 0; s < NS; ++s) acc[s][0] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -404,7 +407,7 @@ linear_mid_reduce_kernel(const float* __restrict__ partial, const float* __restr
 #pragma unroll
         for (int s = 0; s < NS; ++s) acc[s][0] += *reinterpret_cast<const f32x4*>(theirs + (s * MT + mt) * 256);
     }
-    mid_finish<1, NS, TO, SWIGLU, FUSE>(acc, ahead, bias, out, fusion, M, N, K, tile * (64 * NS), tile, 16 * MT, 16 * mt);
+    mid_finish<1, NS, TO, SWIGLU, FUSE>(acc, ahead, bias, out, fusion, M, N, K, tile * (64 * NS), tile, stats_stride, 16 * mt);
 }
 
 template <int MT, int NS, int CK, int DEPTH, typename TO, bool SW, bool TL, int FUSE>
@@ -542,13 +545,17 @@ extern "C" int somi_linear_mid_residual_tiles(int M, int N, int K) {
 
 // The product into the residual stream, as somi_linear_residual (linear_fused.hip) for up to 64 rows:
 // h[m, n] += x[m, :] . w[n, :] (+ bias[n]) in float32; stats: [somi_linear_mid_residual_tiles()][16 ceil(M / 16)]
-// float32 sums of squares of the new h per column tile and row; xnext: [M, N] = bfloat16(norm_w * h), or null.
+// float32 sums of squares of the new h per column tile and row (stats_stride: floats from one tile's sums to the
+// next where they are columns of the table of more rows, a multiple of 4, or 0); xnext: [M, N] = bfloat16(norm_w * h),
+// or null.
 extern "C" int somi_linear_mid_residual(const void* x, const void* w, const float* bias, float* h, float* stats,
-                                        const float* norm_w, void* xnext, int M, int N, int K, float* workspace,
-                                        int64_t workspace_floats, hipStream_t stream) {
+                                        int stats_stride, const float* norm_w, void* xnext, int M, int N, int K,
+                                        float* workspace, int64_t workspace_floats, hipStream_t stream) {
     if (mid_check(x, w, SOMI_BF16, M, N, K)) return 1;
     SOMI_REQUIRE(h && stats, "linear_mid_residual: h and stats are needed");
     SOMI_REQUIRE(!xnext || norm_w, "linear_mid_residual: the next rows need the norm's weight");
+    SOMI_REQUIRE(stats_stride == 0 || (stats_stride % 4 == 0 && stats_stride >= 16 * ceil_div(M, 16)),
+                 "linear_mid_residual: a stride of %d floats does not hold the sums of %d rows", stats_stride, M);
     if (M == 0) return 0;
     int strips, splits;
     mid_shape(M, N, K, false, workspace ? workspace_floats : 0, &strips, &splits);
@@ -557,6 +564,7 @@ extern "C" int somi_linear_mid_residual(const void* x, const void* w, const floa
     fusion.norm_w = norm_w;
     fusion.xnext = (bf16*)xnext;
     fusion.stats_out = stats;
+    fusion.stats_stride = stats_stride;
     return mid_dispatch<MID_RESIDUAL>(x, w, bias, nullptr, SOMI_BF16, M, N, K, strips, splits, false, workspace, fusion, stream);
 }
 

@@ -29,6 +29,13 @@ def prefers_mid_passes(m: int, n: int, k: int) -> bool:
     return SKINNY_ROWS < m <= MID_PASSES_ROWS and k >= 8192 and n <= 8192
 
 
+def residual_in_passes(m: int, n: int) -> bool:
+    """A product into the residual stream with few columns and little more than 64 rows (o and down of 65 to 128
+    requests) runs as passes of the few-rows kernels: the 256-row tiles of the many-rows kernel are too few to
+    fill the device there (28 workgroups at 7B sizes: 61 us for o, two passes of the few-rows kernel 2 x 14 us)."""
+    return ops.FUSED_MAX_ROWS < m <= RESIDUAL_PASSES_ROWS and n <= 8192
+
+
 def linear_swiglu(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
     """silu(x @ gate.T) * (x @ up.T) for bfloat16 rows; weight: [2 I, K], gate and up rows interleaved in blocks
     of 16."""
@@ -45,20 +52,22 @@ def linear_residual(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | 
     """h += x @ weight.T (+ bias) in place, by the kernel that :func:`linear` would take for the sizes; see
     :func:`ops.linear_residual`."""
     m, n = x.shape[0], weight.shape[0]
-    if ops.FUSED_MAX_ROWS < m <= RESIDUAL_PASSES_ROWS and n <= 8192:
-        # few columns and little more than 64 rows (the o projection of 65 to 128 requests): the 256-row tiles of the
-        # many-rows kernel are too few to fill the device (28 workgroups at 7B sizes: 61 us), two passes of the
-        # few-rows kernel are not (2 x 14 us)
-        stats, weighted = [], []
+    if residual_in_passes(m, n):
         # one kernel for every pass, the short last one too: the passes' statistics have one row per workgroup and
-        # are laid side by side
-        mid = _mid_is_faster(ops.FUSED_MAX_ROWS, n, x.shape[1])
+        # lie side by side in one table
+        k = x.shape[1]
+        mid = _mid_is_faster(ops.FUSED_MAX_ROWS, n, k)
+        stats = torch.empty((ops.residual_stats_blocks(ops.FUSED_MAX_ROWS, n, k, mid), ops.stats_width(m)),
+                            dtype=torch.float32, device=x.device)
+        weighted = None
+        if next_norm_weight is not None:
+            weighted = torch.empty((m, n), dtype=torch.bfloat16, device=x.device)
         for at in range(0, m, ops.FUSED_MAX_ROWS):
-            rows = slice(at, at + ops.FUSED_MAX_ROWS)
-            part_stats, part_weighted = ops.linear_residual(x[rows], weight, bias, h[rows], next_norm_weight, mid=mid)
-            stats.append(part_stats)
-            weighted.append(part_weighted)
-        return torch.cat(stats, dim=1), (torch.cat(weighted) if next_norm_weight is not None else None)
+            upto = min(at + ops.FUSED_MAX_ROWS, m)
+            ops.linear_residual(x[at:upto], weight, bias, h[at:upto], next_norm_weight, mid=mid,
+                                stats_out=stats[:, at:at + ops.stats_width(upto - at)],
+                                weighted_out=weighted[at:upto] if weighted is not None else None)
+        return stats, weighted
     if m > ops.FUSED_MAX_ROWS:
         return ops.linear_big_residual(x, weight, bias, h, next_norm_weight)
     mid = _mid_is_faster(m, n, x.shape[1])

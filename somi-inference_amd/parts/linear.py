@@ -80,6 +80,8 @@ class Projection:
 
     def deferred(self, x: torch.Tensor) -> "torch.Tensor | DeferredProduct":
         """The product, or a promise of it where the residual stream can compute and add it in one kernel."""
-        if x.dtype == torch.bfloat16 and self.fusable(x.shape[0]) and x.data_ptr() % 16 == 0:
+        rows = x.shape[0]
+        if (x.dtype == torch.bfloat16 and x.data_ptr() % 16 == 0 and self.fusable(min(rows, ops.FUSED_MAX_ROWS))
+                and (self.fusable(rows) or linear_kernels.residual_in_passes(rows, self.out_features))):
             return DeferredProduct(self, x)
         return self(x)
