@@ -140,6 +140,7 @@ def main() -> int:
 
     from somi_inference_amd.config import Qwen2Config
     from somi_inference_amd.engine import Engine, Request, Scheduler, StepEntry
+    from somi_inference_amd.engine.engine import full_collections_deferred
     from somi_inference_amd.models import make_runner, random_model
     from somi_inference_amd.sampling import Sampler, SamplingParams
 
@@ -158,7 +159,8 @@ def main() -> int:
     # the device).  The scheduler runs the prompts in portions of 2,048 tokens and lets the requests that are done
     # with theirs decode meanwhile, so a request has decoded up to `ramp` tokens before the timed steps begin.
     portion = 2048
-    ramp = max(batches) * ((args.context + portion - 1) // portion) + 8
+    # (beyond 128 requests the decoding tokens take a visible share of a step's 2,048: a prompt then needs one portion more)
+    ramp = max(batches) * ((args.context + portion - 1) // portion + (1 if max(batches) > 128 else 0)) + 8
     pages_per_request = (args.context + ramp + args.block_size - 1) // args.block_size + 1
     num_blocks = max(max(batches) * pages_per_request,
                      (args.prefill_tokens + args.block_size - 1) // args.block_size + 1)
@@ -184,20 +186,21 @@ def main() -> int:
         runner.capture_decode_graphs(batch, args.context + ramp)
         for request in requests:
             engine.add_request(request)
-        while scheduler.waiting or any(r.num_computed < len(r.prompt_tokens) for r in requests):
-            engine.step()
-        for _ in range(warmup):
-            engine.step()
-        sync()
-        cached_before = sum(runner.cache.num_tokens(r.request_id) for r in requests)
-        marks = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
-        marks[0].record()
-        start = time.perf_counter()
-        for i in range(steps):
-            engine.step()
-            marks[i + 1].record()
-        sync()
-        seconds = time.perf_counter() - start
+        with full_collections_deferred():          # as Engine.run() steps its requests
+            while scheduler.waiting or any(r.num_computed < len(r.prompt_tokens) for r in requests):
+                engine.step()
+            for _ in range(warmup):
+                engine.step()
+            sync()
+            cached_before = sum(runner.cache.num_tokens(r.request_id) for r in requests)
+            marks = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
+            marks[0].record()
+            start = time.perf_counter()
+            for i in range(steps):
+                engine.step()
+                marks[i + 1].record()
+            sync()
+            seconds = time.perf_counter() - start
         cached_after = sum(runner.cache.num_tokens(r.request_id) for r in requests)
         assert cached_after - cached_before == batch * steps, "a timed step was not a decode step of every request"
         step_ms = [marks[i].elapsed_time(marks[i + 1]) for i in range(steps)]

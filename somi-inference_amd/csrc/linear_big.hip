@@ -72,6 +72,11 @@ struct BigArgs {
     bf16* weighted;                   // [M, N] = bfloat16(norm_w * h) or null
     float* stats_out;                 // [tiles_n * waves along n][stats_width] or null
     int stats_width;
+    // residual with K split over workgroups (tiles of three whole stages only): each split leaves its sums in
+    // partial [splits][M][N] and big_split_reduce_kernel does what the epilogue would have done
+    float* partial;                   // or null: one workgroup walks the whole K
+    int splits, kt_per;               // workgroups per tile and stages of K each of them walks
+    int stats_rows;                   // rows of stats_out (one per 64 columns of the tiles)
 };
 
 template <int N> __device__ __forceinline__ void big_wait_vmcnt() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
@@ -112,14 +117,16 @@ linear_big_kernel(const BigArgs p) {
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave / WAVES_N, wn = wave % WAVES_N;
     const int M = p.M, N = p.N, K = p.K;
-    const int KT = (K + BK - 1) / BK;
+    const int splits = HALF ? 1 : p.splits;                      // workgroups that share a tile's K
+    int KT = (K + BK - 1) / BK;                                   // stages this workgroup walks, from kt_first on
+    int kt_first = 0;
     const int lrow = lane >> 3, lpos = lane & 7;
     const int frow = lane & 31, fk = lane >> 5;
     const int ml = lane & 31, nh = lane >> 5;
 
     // tiles of this workgroup: the die (blockIdx % 8) owns a contiguous range of tiles with the row tiles of a
     // column tile next to each other; its workgroups take them 32 (wide, persistent) apart, or one each
-    const int total = p.tiles_m * p.tiles_n, per = (total + 7) / 8;
+    const int total = p.tiles_m * p.tiles_n * splits, per = (total + 7) / 8;
     const int die_first = (blockIdx.x & 7) * per, die_end = die_first + per < total ? die_first + per : total;
     const int stride = HALF ? (int)(gridDim.x >> 3) : per;
     int logical = die_first + (blockIdx.x >> 3);
@@ -135,11 +142,19 @@ linear_big_kernel(const BigArgs p) {
     for (int i = 0; i < LA; ++i) piece_a[i] = lpos ^ ((((wave * LA + i) * 8 + lrow) >> 1) & 7);
 #pragma unroll
     for (int i = 0; i < LB; ++i) piece_b[i] = lpos ^ ((((wave * LB + i) * 8 + lrow) >> 1) & 7);
-    auto aim = [&](int tile) {                 // point the loads at a tile
+    auto aim = [&](int item) {                 // point the loads at a tile (and, with K split, at this split's stages)
+        const int tile = item / splits;
         const int tn = tile / p.tiles_m, tm = tile % p.tiles_m;
         const int mlim = M - tm * BM, nlim = N - tn * BN;
         xa = (const char*)(p.x + (int64_t)tm * BM * p.ldx);
         wb = (const char*)(p.w + (int64_t)tn * BN * p.ldw);
+        if (!HALF && splits > 1) {
+            kt_first = (item % splits) * p.kt_per;
+            const int left = (K + BK - 1) / BK - kt_first;
+            KT = left < p.kt_per ? left : p.kt_per;
+            xa += (int64_t)kt_first * ROW_BYTES;
+            wb += (int64_t)kt_first * ROW_BYTES;
+        }
 #pragma unroll
         for (int i = 0; i < LA; ++i) {
             const int row = (wave * LA + i) * 8 + lrow;
@@ -157,7 +172,7 @@ linear_big_kernel(const BigArgs p) {
         kt = kt < KT ? kt : KT - 1;
         const char* src = (is_b ? wb + offb[i] : xa + offa[i]) + (int64_t)kt * ROW_BYTES;
         if (KTAIL) {
-            if (kt * BK + (is_b ? piece_b[i] : piece_a[i]) * 8 >= K) src = (const char*)big_zero_piece;
+            if ((kt_first + kt) * BK + (is_b ? piece_b[i] : piece_a[i]) * 8 >= K) src = (const char*)big_zero_piece;
         }
         char* dst = lds + at + (wave * (is_b ? LB : LA) + i) * 1024;
         __builtin_amdgcn_global_load_lds((const BIG_GLOBAL void*)src, (BIG_LDS void*)dst, 16, 0, 0);
@@ -204,7 +219,8 @@ linear_big_kernel(const BigArgs p) {
     }
 
     while (true) {
-        const int tn = logical / p.tiles_m, tm = logical % p.tiles_m;
+        const int tile = logical / splits;
+        const int tn = tile / p.tiles_m, tm = tile % p.tiles_m;
         const int m0 = tm * BM, n0 = tn * BN;
         const int next = logical + stride;
         const bool has_next = HALF && next < die_end;
@@ -429,7 +445,16 @@ linear_big_kernel(const BigArgs p) {
                         f32x4 v = *(const f32x4*)(stg + row * SROW + piece * 16);
                         const int gm = m0 + wm * 128 + i * 32 + row;
                         const int gn = wave_n0 + j * 32 + piece * 4;
-                        if (gm < M && gn < N) {
+                        if (!HALF && p.partial != nullptr) {
+                            // K is split: this workgroup's sums go to its plane of the workspace as they are
+                            if (gm < M && gn < N) {
+                                float* pp = p.partial + ((int64_t)(logical % splits) * M + gm) * N + gn;
+                                if ((N & 3) == 0 && gn + 4 <= N) *(f32x4*)pp = v;
+                                else
+                                    for (int c = 0; c < 4; ++c)
+                                        if (gn + c < N) pp[c] = v[c];
+                            }
+                        } else if (gm < M && gn < N) {
                             float* hp = p.h + (int64_t)gm * N + gn;
                             if (aligned && gn + 4 <= N) {
                                 f32x4 hv = *(const f32x4*)hp;
@@ -458,7 +483,7 @@ linear_big_kernel(const BigArgs p) {
                     }
                     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
                 }
-                if (p.stats_out != nullptr) {
+                if (p.stats_out != nullptr && (HALF || p.partial == nullptr)) {
                     // the 8 lanes of a row add their squares in a fixed order
 #pragma unroll
                     for (int pass = 0; pass < 4; ++pass) {
@@ -480,6 +505,82 @@ linear_big_kernel(const BigArgs p) {
 #pragma unroll
             for (int i = 0; i < LA; ++i) issue_piece(q, q, i);
         logical = next;
+    }
+}
+
+// The end of the residual form where K was split: h += sum over the splits (in split order) + bias, the next norm's
+// weighted rows and the sums of squares, laid out as the unsplit kernel's (one row of the statistics per 64
+// columns).  A workgroup takes 16 rows x 256 columns; the 16 lanes of a row read 256 consecutive bytes of a plane.
+__global__ void __launch_bounds__(256)
+big_split_reduce_kernel(const BigArgs p) {
+    const int row = threadIdx.x >> 4, cg = threadIdx.x & 15;
+    const int gm = blockIdx.y * 16 + row;
+    const int M = p.M, N = p.N;
+    const bool whole = (N & 3) == 0 && ((uintptr_t)p.h & 15) == 0 && (p.weighted == nullptr || ((uintptr_t)p.weighted & 7) == 0);
+    float sq[4] = {0.f, 0.f, 0.f, 0.f};
+    if (gm < M) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const int gn = blockIdx.x * 256 + q * 64 + cg * 4;
+            if (gn >= N) continue;
+            const bool four = whole && gn + 4 <= N;
+            f32x4 sum = {0.f, 0.f, 0.f, 0.f};
+            const float* pp = p.partial + (int64_t)gm * N + gn;
+            const int64_t plane = (int64_t)M * N;
+            if (four) {
+                // four planes' loads in flight at a time, added in split order
+                int s = 0;
+                for (; s + 4 <= p.splits; s += 4) {
+                    const f32x4 a = *(const f32x4*)(pp + s * plane), b = *(const f32x4*)(pp + (s + 1) * plane);
+                    const f32x4 c = *(const f32x4*)(pp + (s + 2) * plane), d = *(const f32x4*)(pp + (s + 3) * plane);
+                    sum += a;
+                    sum += b;
+                    sum += c;
+                    sum += d;
+                }
+                for (; s < p.splits; ++s) sum += *(const f32x4*)(pp + s * plane);
+            } else {
+                for (int s = 0; s < p.splits; ++s)
+                    for (int c = 0; c < 4; ++c)
+                        if (gn + c < N) sum[c] += pp[s * plane + c];
+            }
+            float* hp = p.h + (int64_t)gm * N + gn;
+            if (four) {
+                f32x4 hv = *(const f32x4*)hp;
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    hv[c] += sum[c] + (p.bias != nullptr ? p.bias[gn + c] : 0.f);
+                    sq[q] += hv[c] * hv[c];
+                }
+                *(f32x4*)hp = hv;
+                if (p.weighted != nullptr) {
+                    bf16x4 wv;
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) wv[c] = (bf16)(p.norm_w[gn + c] * hv[c]);
+                    *(bf16x4*)(p.weighted + (int64_t)gm * N + gn) = wv;
+                }
+            } else {
+                for (int c = 0; c < 4; ++c)
+                    if (gn + c < N) {
+                        const float hv = hp[c] + sum[c] + (p.bias != nullptr ? p.bias[gn + c] : 0.f);
+                        hp[c] = hv;
+                        sq[q] += hv * hv;
+                        if (p.weighted != nullptr) p.weighted[(int64_t)gm * N + gn + c] = (bf16)(p.norm_w[gn + c] * hv);
+                    }
+            }
+        }
+    }
+    if (p.stats_out != nullptr) {
+        // the 16 lanes of a row add their squares in a fixed order; every lane takes part
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            float v = sq[q];
+#pragma unroll
+            for (int off = 8; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+            // columns past N inside the last tile: a row of zeros, as the unsplit kernel leaves it
+            if (cg == 0 && gm < M && blockIdx.x * 4 + q < p.stats_rows)
+                p.stats_out[(int64_t)(blockIdx.x * 4 + q) * p.stats_width + gm] = v;
+        }
     }
 }
 
@@ -526,7 +627,7 @@ static int big_launch_one(const BigArgs& args, hipStream_t stream) {
     }
     // one workgroup per tile; the wide form is persistent: at most one workgroup per compute unit, a multiple of 8
     // (the dies), each walking its die's tiles
-    const int per = ceil_div(args.tiles_m * args.tiles_n, 8);
+    const int per = ceil_div(args.tiles_m * args.tiles_n * args.splits, 8);
     int per_die = per;
     if (S == 5) {
         const int cus_per_die = big_compute_units() / 8 > 0 ? big_compute_units() / 8 : 1;
@@ -534,21 +635,56 @@ static int big_launch_one(const BigArgs& args, hipStream_t stream) {
     }
     hipLaunchKernelGGL((linear_big_kernel<BM, BN, S, NW, EPI, KTAIL>), dim3(per_die * 8), dim3(NW * 64), lds_bytes, stream, args);
     SOMI_LAUNCH_CHECK("linear_big");
+    if (EPI == BIG_RESIDUAL && args.partial != nullptr) {
+        hipLaunchKernelGGL(big_split_reduce_kernel, dim3(ceil_div(args.N, 256), ceil_div(args.M, 16)), dim3(256), 0, stream, args);
+        SOMI_LAUNCH_CHECK("linear_big: reduce");
+    }
     return 0;
 }
 
+// How many workgroups share a tile's K in the residual form (tiles of three whole stages): as many as give about
+// every compute unit a workgroup, with at least BIG_SPLIT_MIN_STAGES stages each, within the workspace; 1 where the
+// tiles alone fill half of the device.  (7B down projection at 192 rows: 28 tiles of 256 x 128, 296 stages: 227 us
+// unsplit, 62 in 9 splits.)
+#define BIG_SPLIT_MIN_STAGES 8
+static int big_splits(int tiles, int m, int n, int k, int64_t workspace_floats) {
+    const int cus = big_compute_units();
+    const int stages = ceil_div(k, BIG_BK);
+    if (workspace_floats <= 0 || tiles * 2 > cus) return 1;
+    int64_t splits = cus / tiles;
+    if (splits > stages / BIG_SPLIT_MIN_STAGES) splits = stages / BIG_SPLIT_MIN_STAGES;
+    if (splits > workspace_floats / ((int64_t)m * n)) splits = workspace_floats / ((int64_t)m * n);
+    if (splits <= 1) return 1;
+    const int per = ceil_div(stages, (int)splits);
+    return ceil_div(stages, per);                    // no split without stages
+}
+
 template <int EPI>
-static int big_launch(BigArgs& args, int tile, hipStream_t stream) {
+static int big_launch(BigArgs& args, int tile, hipStream_t stream, float* workspace = nullptr, int64_t workspace_floats = 0) {
     const bool ktail = args.K % BIG_BK != 0;
+    args.splits = 1;
+    args.partial = nullptr;
+    auto split_k = [&]() {                     // the tiles are set: share their K where they are few
+        if (EPI != BIG_RESIDUAL || workspace == nullptr) return;
+        args.splits = big_splits(args.tiles_m * args.tiles_n, args.M, args.N, args.K, workspace_floats);
+        if (args.splits > 1) {
+            args.kt_per = ceil_div(ceil_div(args.K, BIG_BK), args.splits);
+            args.partial = workspace;
+        }
+    };
     if (big_use_low(args.M, tile)) {
         // up to 128 rows: one row tile of 128, four wavefronts side by side over 256 columns
         args.tiles_m = ceil_div(args.M, 128);
         args.tiles_n = ceil_div(args.N, 256);
+        args.stats_rows = args.tiles_n * 4;
+        split_k();
         return ktail ? big_launch_one<128, 256, 3, 4, EPI, true>(args, stream) : big_launch_one<128, 256, 3, 4, EPI, false>(args, stream);
     }
     const bool wide = tile == 0 ? big_use_wide(args.M, args.N) : tile == 256;
     args.tiles_m = ceil_div(args.M, BIG_BM);
     args.tiles_n = ceil_div(args.N, wide ? 256 : 128);
+    args.stats_rows = wide ? args.tiles_n * 4 : args.tiles_n * 2;
+    if (!wide) split_k();
     if (wide) return ktail ? big_launch_one<256, 256, 5, 8, EPI, true>(args, stream) : big_launch_one<256, 256, 5, 8, EPI, false>(args, stream);
     return ktail ? big_launch_one<256, 128, 3, 4, EPI, true>(args, stream) : big_launch_one<256, 128, 3, 4, EPI, false>(args, stream);
 }
@@ -603,6 +739,13 @@ extern "C" int somi_linear_big_stats_blocks(int m, int n, int tile) {
     return wide ? ceil_div(n, 256) * 4 : ceil_div(n, 128) * 2;
 }
 
+// Workgroups that share a tile's K in somi_linear_big_residual with this much workspace (1: K is not split).
+extern "C" int somi_linear_big_splits(int m, int n, int k, int tile, int64_t workspace_floats) {
+    if (big_use_low(m, tile)) return big_splits(ceil_div(m, 128) * ceil_div(n, 256), m, n, k, workspace_floats);
+    const bool wide = tile == 0 ? big_use_wide(m, n) : tile == 256;
+    return wide ? 1 : big_splits(ceil_div(m, BIG_BM) * ceil_div(n, 128), m, n, k, workspace_floats);
+}
+
 // out = s * (x . w^T) + bias -> bfloat16 [M, N]; with swiglu w is [N, K] with gate and up rows interleaved in blocks
 // of 16 and out is [M, N / 2] = silu(s g) * (s u).  row_scale (or null): s [M], see somi_row_scale.
 extern "C" int somi_linear_big(const void* x, int64_t ldx, const void* w, int64_t ldw, const float* bias, void* out,
@@ -620,10 +763,13 @@ extern "C" int somi_linear_big(const void* x, int64_t ldx, const void* w, int64_
 
 // h += x . w^T + bias, float32 in place [M, N].  norm_w / weighted (or null): weighted = bfloat16(norm_w * h);
 // stats_out (or null): [somi_linear_big_stats_blocks(m, n, tile)][stats_width] sums of squares of the new h, each over
-// the 64 columns of one wavefront.
+// the 64 columns of one wavefront.  workspace (or null): workspace_floats of float32, 16-byte aligned, that let the
+// 128-row tile split K over workgroups where the tiles alone leave most of the device idle (somi_linear_big_splits
+// says how many ways; the 256 x 128 tiles do the same); calls that share a workspace must not overlap.
 extern "C" int somi_linear_big_residual(const void* x, int64_t ldx, const void* w, int64_t ldw, const float* bias, float* h,
                                         const float* norm_w, void* weighted, float* stats_out, int stats_width,
-                                        int m, int n, int k, int tile, hipStream_t stream) {
+                                        int m, int n, int k, int tile, float* workspace, int64_t workspace_floats,
+                                        hipStream_t stream) {
     if (big_check("linear_big_residual", x, ldx, w, ldw, m, n, k) != 0) return 1;
     SOMI_REQUIRE(h != nullptr, "linear_big_residual: no residual stream");
     SOMI_REQUIRE((weighted == nullptr) == (norm_w == nullptr), "linear_big_residual: the norm's weight and its rows come together");
@@ -633,5 +779,7 @@ extern "C" int somi_linear_big_residual(const void* x, int64_t ldx, const void* 
     args.x = (const bf16*)x; args.ldx = ldx; args.w = (const bf16*)w; args.ldw = ldw; args.bias = bias;
     args.M = m; args.N = n; args.K = k; args.h = h; args.norm_w = norm_w; args.weighted = (bf16*)weighted;
     args.stats_out = stats_out; args.stats_width = stats_width;
-    return big_launch<BIG_RESIDUAL>(args, tile, stream);
+    SOMI_REQUIRE(workspace == nullptr || (((uintptr_t)workspace & 15) == 0 && workspace_floats >= 0),
+                 "linear_big_residual: the workspace must be aligned to 16 bytes");
+    return big_launch<BIG_RESIDUAL>(args, tile, stream, workspace, workspace_floats);
 }

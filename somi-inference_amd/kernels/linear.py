@@ -7,7 +7,7 @@ import torch
 from . import ops
 
 SKINNY_MAX_ROWS = 64   # what the skinny MFMA kernel takes
-MID_PASSES_ROWS = 192  # up to here a product with long K and few columns runs the split-K kernel in passes of 64 rows
+MID_PASSES_ROWS = 128  # up to here a product with long K and few columns runs the split-K kernel in passes of 64 rows
 SKINNY_ROWS = 64       # up to here the few-rows kernels run; beyond, the many-rows kernel (ops.linear_big)
 RESIDUAL_PASSES_ROWS = 128   # up to here a product into the residual stream with few columns runs in passes of 64 rows
 
@@ -25,7 +25,9 @@ def _mid_is_faster(m: int, n: int, k: int) -> bool:
 def prefers_mid_passes(m: int, n: int, k: int) -> bool:
     """More than SKINNY_ROWS rows, but few enough that a product with a long K and few columns (down) runs faster
     as passes of the split-K kernel over 64 rows each than on the 256-row tiles of the many-rows kernel, which are
-    too few to fill the device there (7B down projection: 62 to 67 us at 65 to 128 rows, 99 at 192, against 157)."""
+    too few to fill the device there (7B down projection: 62 to 67 us at 65 to 128 rows against 157).  The product
+    into the residual stream has ways of its own (passes that add into the stream up to 128 rows, the many-rows
+    kernel with K split over workgroups beyond); this is for a product that is kept."""
     return SKINNY_ROWS < m <= MID_PASSES_ROWS and k >= 8192 and n <= 8192
 
 

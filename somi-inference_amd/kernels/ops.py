@@ -394,11 +394,13 @@ def linear_big(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None 
 
 
 def linear_big_residual(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, h: torch.Tensor,
-                        next_norm_weight: torch.Tensor | None = None, tile: int = 0
+                        next_norm_weight: torch.Tensor | None = None, tile: int = 0, split_k: bool = True
                         ) -> tuple[torch.Tensor, torch.Tensor | None]:
     """h += x @ weight.T (+ bias) in float32, in place, for any number of rows.  Returns the row statistics
     ``[blocks, 16 ceil(M / 16)]`` (sums of squares of the new h, each over the 64 columns of one wavefront) and,
-    with ``next_norm_weight``, the rows ``bfloat16(next_norm_weight * h)``: what :func:`linear_big` scales."""
+    with ``next_norm_weight``, the rows ``bfloat16(next_norm_weight * h)``: what :func:`linear_big` scales.
+    ``split_k``: the 128-row tile may split K over workgroups (through the device's workspace) where its tiles alone
+    would leave most of the device idle."""
     m, n, k = _big_operands(x, weight, bias, "linear_big_residual")
     _need(h, "residual stream", torch.float32, (m, n))
     lib = library()
@@ -408,10 +410,17 @@ def linear_big_residual(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tenso
     if next_norm_weight is not None:
         _need(next_norm_weight, "norm weight", torch.float32, (n,))
         weighted = torch.empty((m, n), dtype=torch.bfloat16, device=x.device)
+    workspace = _mid_workspace(x.device) if split_k else None
     _check(lib.somi_linear_big_residual(_ptr(x), ctypes.c_int64(x.stride(0)), _ptr(weight), ctypes.c_int64(weight.stride(0)),
                                         _ptr(bias), _ptr(h), _ptr(next_norm_weight), _ptr(weighted), _ptr(stats),
-                                        stats.shape[1], m, n, k, int(tile), _stream()))
+                                        stats.shape[1], m, n, k, int(tile), _ptr(workspace),
+                                        ctypes.c_int64(workspace.numel() if workspace is not None else 0), _stream()))
     return stats, weighted
+
+
+def linear_big_splits(m: int, n: int, k: int, tile: int = 0) -> int:
+    """Workgroups that share a tile's K in :func:`linear_big_residual` for these sizes (1: K is not split)."""
+    return library().somi_linear_big_splits(m, n, k, int(tile), ctypes.c_int64(MID_WORKSPACE_FLOATS))
 
 
 def residual_stats_blocks(m: int, n: int, k: int, mid: bool) -> int:

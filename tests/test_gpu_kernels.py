@@ -745,6 +745,38 @@ def test_many_rows_product_into_the_residual_stream(m, n, k, tile):
         torch.testing.assert_close(got.float(), want, atol=0.02 * float(want.abs().max()), rtol=2e-2)
 
 
+@pytest.mark.parametrize("tile", [1, 0, 128], ids=["128-row", "chosen", "256x128"])
+@pytest.mark.parametrize("m,n,k", [(100, 520, 2056), (128, 264, 4096), (65, 130, 1024), (7, 72, 3000), (300, 96, 1032),
+                                   (260, 300, 2056), (513, 200, 1536)])
+def test_many_rows_product_into_the_stream_with_k_split_over_workgroups(m, n, k, tile):
+    """Few tiles and a long K: the 128-row tile and the 256 x 128 tile split K over workgroups, and a second kernel
+    adds the splits' sums into the stream and leaves the weighted rows and the sums of squares as the unsplit kernel
+    does (K that ends inside a stage, N that is no multiple of 4 or of the tile, rows that do not fill a tile,
+    several row tiles)."""
+    assert ops.linear_big_splits(m, n, k, tile=tile) > 1
+    x, w, bias = rnd(m, k, dtype="bfloat16", seed=9), rnd(n, k, dtype="bfloat16", seed=10, scale=0.2), rnd(n, seed=11)
+    h0 = rnd(m, n, seed=12)
+    norm_w = rnd(n, seed=13).abs() + 0.5
+    want_h = h0 + F.linear(x.float(), w.float(), bias)
+    tol = dict(atol=2e-4 * float(want_h.abs().max()) + 1e-4, rtol=1e-4)
+    h = h0.clone()
+    stats, weighted = ops.linear_big_residual(x, w, bias, h, norm_w, tile=tile)
+    torch.testing.assert_close(h, want_h, **tol)
+    assert torch.equal(weighted, (norm_w * h).to(torch.bfloat16))
+    torch.testing.assert_close(stats[:, :m].sum(0), h.pow(2).sum(1), rtol=1e-4, atol=1e-3)
+    whole = h0.clone()
+    whole_stats, whole_weighted = ops.linear_big_residual(x, w, bias, whole, norm_w, tile=tile, split_k=False)
+    assert whole_stats.shape == stats.shape
+    torch.testing.assert_close(h, whole, **tol)
+    torch.testing.assert_close(stats[:, :m], whole_stats[:, :m], rtol=1e-3, atol=1e-3)
+    again = h0.clone()                                   # the workspace is used again: the same bits
+    ops.linear_big_residual(x, w, bias, again, norm_w, tile=tile)
+    assert torch.equal(again, h)
+    no_bias = h0.clone()
+    assert ops.linear_big_residual(x, w, None, no_bias, tile=tile)[1] is None
+    torch.testing.assert_close(no_bias, h0 + F.linear(x.float(), w.float()), **tol)
+
+
 @pytest.mark.parametrize("nq, nkv, d, page, window", [(8, 2, 128, 16, 0), (14, 2, 64, 8, 700), (4, 4, 128, 64, 1500)])
 @pytest.mark.parametrize("shape", [0, 4, 5], ids=["auto", "tile", "tile-wide"])
 def test_attention_prefill_tile_kernel_over_long_contexts(nq, nkv, d, page, window, shape):

@@ -357,3 +357,30 @@ def test_portions_come_in_multiples_of_the_granule_except_the_one_that_ends_the_
     assert portions[:3] == [8, 8, 2] and all(n == 1 for n in portions[3:])
     with pytest.raises(SchedulerError, match="granule"):
         Scheduler(cache, max_concurrent=1, max_num_batched_tokens=8, chunk=3, granule=4)
+
+
+def test_full_collections_wait_while_requests_are_stepped_and_come_back_after():
+    import gc
+    before = gc.get_threshold()
+    seen = []
+
+    class Watching(ScriptedRunner):
+        def step(self, entries):
+            seen.append(gc.get_threshold())
+            if len(seen) == 3 and self.fail:
+                raise RuntimeError("a step that fails")
+            return super().step(entries)
+
+    cache = make_cache()
+    scheduler = Scheduler(cache, max_concurrent=4, max_num_batched_tokens=64)
+    runner = Watching(cache)
+    runner.fail = False
+    engine = Engine(runner, scheduler, ScriptedSampler({0: [7, 8, 9]}), None)
+    engine.run(deque([(0, request(0, 5, 3))]))
+    assert seen and all(t[:2] == before[:2] and t[2] > 1_000_000 for t in seen)
+    assert gc.get_threshold() == before
+    runner.fail = True
+    del seen[:]
+    with pytest.raises(RuntimeError, match="a step that fails"):
+        engine.run(deque([(0, request(0, 5, 3))]))
+    assert gc.get_threshold() == before and not cache.live_requests()
