@@ -75,7 +75,8 @@ struct BigArgs {
     // residual with K split over workgroups (tiles of three whole stages only): each split leaves its sums in
     // partial [splits][M][N] and big_split_reduce_kernel does what the epilogue would have done
     float* partial;                   // or null: one workgroup walks the whole K
-    int splits, kt_per;               // workgroups per tile and stages of K each of them walks
+    int splits;                       // workgroups per tile: split s walks the stages s, s + splits, s + 2 splits, ...
+                                      // (the splits of a tile run side by side and so read neighbouring lines of a row)
     int stats_rows;                   // rows of stats_out (one per 64 columns of the tiles)
 };
 
@@ -118,8 +119,9 @@ linear_big_kernel(const BigArgs p) {
     const int wm = wave / WAVES_N, wn = wave % WAVES_N;
     const int M = p.M, N = p.N, K = p.K;
     const int splits = HALF ? 1 : p.splits;                      // workgroups that share a tile's K
-    int KT = (K + BK - 1) / BK;                                   // stages this workgroup walks, from kt_first on
+    int KT = (K + BK - 1) / BK;                                   // stages this workgroup walks: kt_first, kt_first + splits, ...
     int kt_first = 0;
+    const int64_t stage_bytes = (int64_t)ROW_BYTES * splits;      // from one of its stages to the next
     const int lrow = lane >> 3, lpos = lane & 7;
     const int frow = lane & 31, fk = lane >> 5;
     const int ml = lane & 31, nh = lane >> 5;
@@ -149,9 +151,8 @@ linear_big_kernel(const BigArgs p) {
         xa = (const char*)(p.x + (int64_t)tm * BM * p.ldx);
         wb = (const char*)(p.w + (int64_t)tn * BN * p.ldw);
         if (!HALF && splits > 1) {
-            kt_first = (item % splits) * p.kt_per;
-            const int left = (K + BK - 1) / BK - kt_first;
-            KT = left < p.kt_per ? left : p.kt_per;
+            kt_first = item % splits;
+            KT = ((K + BK - 1) / BK - kt_first + splits - 1) / splits;
             xa += (int64_t)kt_first * ROW_BYTES;
             wb += (int64_t)kt_first * ROW_BYTES;
         }
@@ -170,9 +171,9 @@ linear_big_kernel(const BigArgs p) {
     // the last one (it lands in a slot that is never read again)
     auto issue = [&](bool is_b, int kt, int at, int i) {
         kt = kt < KT ? kt : KT - 1;
-        const char* src = (is_b ? wb + offb[i] : xa + offa[i]) + (int64_t)kt * ROW_BYTES;
+        const char* src = (is_b ? wb + offb[i] : xa + offa[i]) + kt * stage_bytes;
         if (KTAIL) {
-            if ((kt_first + kt) * BK + (is_b ? piece_b[i] : piece_a[i]) * 8 >= K) src = (const char*)big_zero_piece;
+            if ((kt_first + kt * splits) * BK + (is_b ? piece_b[i] : piece_a[i]) * 8 >= K) src = (const char*)big_zero_piece;
         }
         char* dst = lds + at + (wave * (is_b ? LB : LA) + i) * 1024;
         __builtin_amdgcn_global_load_lds((const BIG_GLOBAL void*)src, (BIG_LDS void*)dst, 16, 0, 0);
@@ -667,10 +668,7 @@ static int big_launch(BigArgs& args, int tile, hipStream_t stream, float* worksp
     auto split_k = [&]() {                     // the tiles are set: share their K where they are few
         if (EPI != BIG_RESIDUAL || workspace == nullptr) return;
         args.splits = big_splits(args.tiles_m * args.tiles_n, args.M, args.N, args.K, workspace_floats);
-        if (args.splits > 1) {
-            args.kt_per = ceil_div(ceil_div(args.K, BIG_BK), args.splits);
-            args.partial = workspace;
-        }
+        if (args.splits > 1) args.partial = workspace;
     };
     if (big_use_low(args.M, tile)) {
         // up to 128 rows: one row tile of 128, four wavefronts side by side over 256 columns
