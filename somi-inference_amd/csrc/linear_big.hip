@@ -68,6 +68,7 @@ struct BigArgs {
     const float* row_scale;           // [M] the rows' scales s, or null
     // residual
     float* h;                         // [M, N] float32, in and out
+    int overwrite;                    // h is out only: h = x . w^T + bias (float32 results of many rows: logits)
     const float* norm_w;              // [N] or null
     bf16* weighted;                   // [M, N] = bfloat16(norm_w * h) or null
     float* stats_out;                 // [tiles_n * waves along n][stats_width] or null
@@ -458,7 +459,7 @@ linear_big_kernel(const BigArgs p) {
                         } else if (gm < M && gn < N) {
                             float* hp = p.h + (int64_t)gm * N + gn;
                             if (aligned && gn + 4 <= N) {
-                                f32x4 hv = *(const f32x4*)hp;
+                                f32x4 hv = p.overwrite ? f32x4{0.f, 0.f, 0.f, 0.f} : *(const f32x4*)hp;
 #pragma unroll
                                 for (int c = 0; c < 4; ++c) {
                                     hv[c] += v[c] + (p.bias != nullptr ? p.bias[gn + c] : 0.f);
@@ -474,7 +475,7 @@ linear_big_kernel(const BigArgs p) {
                             } else {
                                 for (int c = 0; c < 4; ++c)
                                     if (gn + c < N) {
-                                        const float hv = hp[c] + v[c] + (p.bias != nullptr ? p.bias[gn + c] : 0.f);
+                                        const float hv = (p.overwrite ? 0.f : hp[c]) + v[c] + (p.bias != nullptr ? p.bias[gn + c] : 0.f);
                                         hp[c] = hv;
                                         sq[pass] += hv * hv;
                                         if (p.weighted != nullptr) p.weighted[(int64_t)gm * N + gn + c] = (bf16)(p.norm_w[gn + c] * hv);
@@ -547,7 +548,7 @@ big_split_reduce_kernel(const BigArgs p) {
             }
             float* hp = p.h + (int64_t)gm * N + gn;
             if (four) {
-                f32x4 hv = *(const f32x4*)hp;
+                f32x4 hv = p.overwrite ? f32x4{0.f, 0.f, 0.f, 0.f} : *(const f32x4*)hp;
 #pragma unroll
                 for (int c = 0; c < 4; ++c) {
                     hv[c] += sum[c] + (p.bias != nullptr ? p.bias[gn + c] : 0.f);
@@ -563,7 +564,7 @@ big_split_reduce_kernel(const BigArgs p) {
             } else {
                 for (int c = 0; c < 4; ++c)
                     if (gn + c < N) {
-                        const float hv = hp[c] + sum[c] + (p.bias != nullptr ? p.bias[gn + c] : 0.f);
+                        const float hv = (p.overwrite ? 0.f : hp[c]) + sum[c] + (p.bias != nullptr ? p.bias[gn + c] : 0.f);
                         hp[c] = hv;
                         sq[q] += hv * hv;
                         if (p.weighted != nullptr) p.weighted[(int64_t)gm * N + gn + c] = (bf16)(p.norm_w[gn + c] * hv);
@@ -780,4 +781,17 @@ extern "C" int somi_linear_big_residual(const void* x, int64_t ldx, const void* 
     SOMI_REQUIRE(workspace == nullptr || (((uintptr_t)workspace & 15) == 0 && workspace_floats >= 0),
                  "linear_big_residual: the workspace must be aligned to 16 bytes");
     return big_launch<BIG_RESIDUAL>(args, tile, stream, workspace, workspace_floats);
+}
+
+// out = x . w^T + bias -> float32 [M, N] (logits of many rows, which must not pass through bfloat16): the residual
+// form's end writing its sums instead of adding them, without the norm's by-products.
+extern "C" int somi_linear_big_f32(const void* x, int64_t ldx, const void* w, int64_t ldw, const float* bias, float* out,
+                                   int m, int n, int k, int tile, hipStream_t stream) {
+    if (big_check("linear_big_f32", x, ldx, w, ldw, m, n, k) != 0) return 1;
+    SOMI_REQUIRE(out != nullptr, "linear_big_f32: no output");
+    SOMI_REQUIRE(tile == 0 || tile == BIG_TILE_LOW || tile == 128 || tile == 256, "linear_big_f32: tile code %d (0, 1, 128 or 256)", tile);
+    BigArgs args = {};
+    args.x = (const bf16*)x; args.ldx = ldx; args.w = (const bf16*)w; args.ldw = ldw; args.bias = bias;
+    args.M = m; args.N = n; args.K = k; args.h = out; args.overwrite = 1;
+    return big_launch<BIG_RESIDUAL>(args, tile, stream);
 }

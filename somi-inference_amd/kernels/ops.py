@@ -418,6 +418,19 @@ def linear_big_residual(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tenso
     return stats, weighted
 
 
+def linear_big_f32(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None, tile: int = 0,
+                   out: torch.Tensor | None = None) -> torch.Tensor:
+    """x @ weight.T (+ bias) as float32 for any number of bfloat16 rows (logits of many rows at once: the weight is
+    read once, and no result passes through bfloat16)."""
+    m, n, k = _big_operands(x, weight, bias, "linear_big_f32")
+    if out is None:
+        out = torch.empty((m, n), dtype=torch.float32, device=x.device)
+    _need(out, "linear_big_f32 out", torch.float32, (m, n))
+    _check(library().somi_linear_big_f32(_ptr(x), ctypes.c_int64(x.stride(0)), _ptr(weight), ctypes.c_int64(weight.stride(0)),
+                                         _ptr(bias), _ptr(out), m, n, k, int(tile), _stream()))
+    return out
+
+
 def linear_big_splits(m: int, n: int, k: int, tile: int = 0) -> int:
     """Workgroups that share a tile's K in :func:`linear_big_residual` for these sizes (1: K is not split)."""
     return library().somi_linear_big_splits(m, n, k, int(tile), ctypes.c_int64(MID_WORKSPACE_FLOATS))

@@ -745,6 +745,25 @@ def test_many_rows_product_into_the_residual_stream(m, n, k, tile):
         torch.testing.assert_close(got.float(), want, atol=0.02 * float(want.abs().max()), rtol=2e-2)
 
 
+@pytest.mark.parametrize("tile", [0, 1, 128, 256])
+@pytest.mark.parametrize("m,n,k", [(65, 130, 64), (128, 1000, 264), (300, 521, 200), (257, 72, 1032)])
+def test_many_rows_product_in_float32(m, n, k, tile):
+    """x . w^T (+ bias) written as float32 (logits of many rows): against F.linear, closer than a bfloat16 result could
+    be; and through the chooser, which takes it for more than 64 rows."""
+    from somi_inference_amd.kernels import linear as chooser
+    x, w, bias = rnd(m, k, dtype="bfloat16", seed=1), rnd(n, k, dtype="bfloat16", seed=2, scale=0.3), rnd(n, seed=3)
+    want = F.linear(x.float(), w.float(), bias)
+    tol = dict(atol=2e-5 * float(want.abs().max()) * math.sqrt(k), rtol=1e-5)
+    out = torch.full((m, n), 7.0, device=DEV)                    # what was there is not added to
+    got = ops.linear_big_f32(x, w, bias, tile=tile, out=out)
+    assert got is out and got.dtype == torch.float32
+    torch.testing.assert_close(got, want, **tol)
+    torch.testing.assert_close(ops.linear_big_f32(x, w, tile=tile), F.linear(x.float(), w.float()), **tol)
+    if tile == 0:
+        chosen = chooser.linear(x, w, bias, out_dtype=torch.float32)
+        assert chosen.dtype == torch.float32 and torch.equal(chosen, got)
+
+
 @pytest.mark.parametrize("tile", [1, 0, 128], ids=["128-row", "chosen", "256x128"])
 @pytest.mark.parametrize("m,n,k", [(100, 520, 2056), (128, 264, 4096), (65, 130, 1024), (7, 72, 3000), (300, 96, 1032),
                                    (260, 300, 2056), (513, 200, 1536)])
