@@ -8,10 +8,13 @@
 //   plain     out = s[m] * (x . w^T) + bias             (bfloat16; s: the row scale of an RMS norm, or 1)
 //   swiglu    out = silu(s g) * (s u), g and u the gate and up products    (models/qwen2.py:226-229)
 //   residual  h += x . w^T + bias in float32, in place (models/qwen2.py:333-339), leaving what the next
-//             norm needs: bfloat16(norm_w * h) and the rows' sums of squares in partial sums
+//             norm needs: bfloat16(norm_w * h) and the rows' sums of squares in partial sums; the same end
+//             writes float32 results as they are (logits of many rows: somi_linear_big_f32).  Where the
+//             tiles of this form are few (o and down of some hundred rows), the workgroups of a tile share
+//             its K, each leaving its sums in a plane of a workspace, and a second kernel does the end.
 //
 // How it maps to gfx950:
-//   * a workgroup owns a 256 x 256 or 256 x 128 tile of the output and walks K in stages of 64 (one
+//   * a workgroup owns a 256 x 256 or 256 x 128 tile of the output (128 x 256 for up to 128 rows) and walks K in stages of 64 (one
 //     128-byte line per row: the L2 serves whole lines, half-used lines cost as much as full ones);
 //   * both operands come by direct-to-LDS loads of 16 bytes a lane into a ring of stages (two for the wide
 //     tile: 2 x 64 KB; three for the narrow one: 3 x 48 KB).  The 16-byte piece c of row r lies at piece
