@@ -515,77 +515,68 @@ linear_big_kernel(const BigArgs p) {
 
 // The end of the residual form where K was split: h += sum over the splits (in split order) + bias, the next norm's
 // weighted rows and the sums of squares, laid out as the unsplit kernel's (one row of the statistics per 64
-// columns).  A workgroup takes 16 rows x 256 columns; the 16 lanes of a row read 256 consecutive bytes of a plane.
+// columns).  A workgroup takes 16 rows x 64 columns (blockIdx.x counts the rows of the statistics); the 16 lanes of
+// a row read 256 consecutive bytes of a plane.
 __global__ void __launch_bounds__(256)
 big_split_reduce_kernel(const BigArgs p) {
     const int row = threadIdx.x >> 4, cg = threadIdx.x & 15;
-    const int gm = blockIdx.y * 16 + row;
+    const int gm = blockIdx.y * 16 + row, gn = blockIdx.x * 64 + cg * 4;
     const int M = p.M, N = p.N;
     const bool whole = (N & 3) == 0 && ((uintptr_t)p.h & 15) == 0 && (p.weighted == nullptr || ((uintptr_t)p.weighted & 7) == 0);
-    float sq[4] = {0.f, 0.f, 0.f, 0.f};
-    if (gm < M) {
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            const int gn = blockIdx.x * 256 + q * 64 + cg * 4;
-            if (gn >= N) continue;
-            const bool four = whole && gn + 4 <= N;
-            f32x4 sum = {0.f, 0.f, 0.f, 0.f};
-            const float* pp = p.partial + (int64_t)gm * N + gn;
-            const int64_t plane = (int64_t)M * N;
-            if (four) {
-                // four planes' loads in flight at a time, added in split order
-                int s = 0;
-                for (; s + 4 <= p.splits; s += 4) {
-                    const f32x4 a = *(const f32x4*)(pp + s * plane), b = *(const f32x4*)(pp + (s + 1) * plane);
-                    const f32x4 c = *(const f32x4*)(pp + (s + 2) * plane), d = *(const f32x4*)(pp + (s + 3) * plane);
-                    sum += a;
-                    sum += b;
-                    sum += c;
-                    sum += d;
-                }
-                for (; s < p.splits; ++s) sum += *(const f32x4*)(pp + s * plane);
-            } else {
-                for (int s = 0; s < p.splits; ++s)
-                    for (int c = 0; c < 4; ++c)
-                        if (gn + c < N) sum[c] += pp[s * plane + c];
+    float sq = 0.f;
+    if (gm < M && gn < N) {
+        const bool four = whole && gn + 4 <= N;
+        f32x4 sum = {0.f, 0.f, 0.f, 0.f};
+        const float* pp = p.partial + (int64_t)gm * N + gn;
+        const int64_t plane = (int64_t)M * N;
+        if (four) {
+            // four planes' loads in flight at a time, added in split order
+            int s = 0;
+            for (; s + 4 <= p.splits; s += 4) {
+                const f32x4 a = *(const f32x4*)(pp + s * plane), b = *(const f32x4*)(pp + (s + 1) * plane);
+                const f32x4 c = *(const f32x4*)(pp + (s + 2) * plane), d = *(const f32x4*)(pp + (s + 3) * plane);
+                sum += a;
+                sum += b;
+                sum += c;
+                sum += d;
             }
-            float* hp = p.h + (int64_t)gm * N + gn;
-            if (four) {
-                f32x4 hv = p.overwrite ? f32x4{0.f, 0.f, 0.f, 0.f} : *(const f32x4*)hp;
-#pragma unroll
-                for (int c = 0; c < 4; ++c) {
-                    hv[c] += sum[c] + (p.bias != nullptr ? p.bias[gn + c] : 0.f);
-                    sq[q] += hv[c] * hv[c];
-                }
-                *(f32x4*)hp = hv;
-                if (p.weighted != nullptr) {
-                    bf16x4 wv;
-#pragma unroll
-                    for (int c = 0; c < 4; ++c) wv[c] = (bf16)(p.norm_w[gn + c] * hv[c]);
-                    *(bf16x4*)(p.weighted + (int64_t)gm * N + gn) = wv;
-                }
-            } else {
+            for (; s < p.splits; ++s) sum += *(const f32x4*)(pp + s * plane);
+        } else {
+            for (int s = 0; s < p.splits; ++s)
                 for (int c = 0; c < 4; ++c)
-                    if (gn + c < N) {
-                        const float hv = (p.overwrite ? 0.f : hp[c]) + sum[c] + (p.bias != nullptr ? p.bias[gn + c] : 0.f);
-                        hp[c] = hv;
-                        sq[q] += hv * hv;
-                        if (p.weighted != nullptr) p.weighted[(int64_t)gm * N + gn + c] = (bf16)(p.norm_w[gn + c] * hv);
-                    }
+                    if (gn + c < N) sum[c] += pp[s * plane + c];
+        }
+        float* hp = p.h + (int64_t)gm * N + gn;
+        if (four) {
+            f32x4 hv = p.overwrite ? f32x4{0.f, 0.f, 0.f, 0.f} : *(const f32x4*)hp;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                hv[c] += sum[c] + (p.bias != nullptr ? p.bias[gn + c] : 0.f);
+                sq += hv[c] * hv[c];
             }
+            *(f32x4*)hp = hv;
+            if (p.weighted != nullptr) {
+                bf16x4 wv;
+#pragma unroll
+                for (int c = 0; c < 4; ++c) wv[c] = (bf16)(p.norm_w[gn + c] * hv[c]);
+                *(bf16x4*)(p.weighted + (int64_t)gm * N + gn) = wv;
+            }
+        } else {
+            for (int c = 0; c < 4; ++c)
+                if (gn + c < N) {
+                    const float hv = (p.overwrite ? 0.f : hp[c]) + sum[c] + (p.bias != nullptr ? p.bias[gn + c] : 0.f);
+                    hp[c] = hv;
+                    sq += hv * hv;
+                    if (p.weighted != nullptr) p.weighted[(int64_t)gm * N + gn + c] = (bf16)(p.norm_w[gn + c] * hv);
+                }
         }
     }
     if (p.stats_out != nullptr) {
-        // the 16 lanes of a row add their squares in a fixed order; every lane takes part
+        // the 16 lanes of a row add their squares in a fixed order; every lane takes part.  Columns past N inside
+        // the last tile give a row of zeros, as the unsplit kernel leaves it.
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            float v = sq[q];
-#pragma unroll
-            for (int off = 8; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
-            // columns past N inside the last tile: a row of zeros, as the unsplit kernel leaves it
-            if (cg == 0 && gm < M && blockIdx.x * 4 + q < p.stats_rows)
-                p.stats_out[(int64_t)(blockIdx.x * 4 + q) * p.stats_width + gm] = v;
-        }
+        for (int off = 8; off > 0; off >>= 1) sq += __shfl_xor(sq, off, 64);
+        if (cg == 0 && gm < M) p.stats_out[(int64_t)blockIdx.x * p.stats_width + gm] = sq;
     }
 }
 
@@ -641,7 +632,7 @@ static int big_launch_one(const BigArgs& args, hipStream_t stream) {
     hipLaunchKernelGGL((linear_big_kernel<BM, BN, S, NW, EPI, KTAIL>), dim3(per_die * 8), dim3(NW * 64), lds_bytes, stream, args);
     SOMI_LAUNCH_CHECK("linear_big");
     if (EPI == BIG_RESIDUAL && args.partial != nullptr) {
-        hipLaunchKernelGGL(big_split_reduce_kernel, dim3(ceil_div(args.N, 256), ceil_div(args.M, 16)), dim3(256), 0, stream, args);
+        hipLaunchKernelGGL(big_split_reduce_kernel, dim3(args.stats_rows, ceil_div(args.M, 16)), dim3(256), 0, stream, args);
         SOMI_LAUNCH_CHECK("linear_big: reduce");
     }
     return 0;

@@ -31,11 +31,16 @@ def prefers_mid_passes(m: int, n: int, k: int) -> bool:
     return SKINNY_ROWS < m <= MID_PASSES_ROWS and k >= 8192 and n <= 8192
 
 
-def residual_in_passes(m: int, n: int) -> bool:
-    """A product into the residual stream with few columns and little more than 64 rows (o and down of 65 to 128
-    requests) runs as passes of the few-rows kernels: the 256-row tiles of the many-rows kernel are too few to
-    fill the device there (28 workgroups at 7B sizes: 61 us for o, two passes of the few-rows kernel 2 x 14 us)."""
-    return ops.FUSED_MAX_ROWS < m <= RESIDUAL_PASSES_ROWS and n <= 8192
+RESIDUAL_PASSES_MAX_K = 8192     # below this K
+
+
+def residual_in_passes(m: int, n: int, k: int) -> bool:
+    """A product into the residual stream with few columns, a short K and little more than 64 rows (o of 65 to 128
+    requests) runs as passes of the few-rows kernel: the tiles of the many-rows kernel are too few to fill the
+    device there, and with so short a K sharing it among workgroups does not pay (7B sizes, 128 rows, inside decode
+    steps: two passes 2 x 12 us, the many-rows kernel with K split 35 + 12).  A long K (down) is what that split is
+    for: steps of 80 / 96 / 128 requests are 3.4 / 2.5 / 2.4 % shorter with it than with passes."""
+    return ops.FUSED_MAX_ROWS < m <= RESIDUAL_PASSES_ROWS and n <= 8192 and k < RESIDUAL_PASSES_MAX_K
 
 
 def linear_swiglu(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
@@ -54,7 +59,7 @@ def linear_residual(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | 
     """h += x @ weight.T (+ bias) in place, by the kernel that :func:`linear` would take for the sizes; see
     :func:`ops.linear_residual`."""
     m, n = x.shape[0], weight.shape[0]
-    if residual_in_passes(m, n):
+    if residual_in_passes(m, n, x.shape[1]):
         # one kernel for every pass, the short last one too: the passes' statistics have one row per workgroup and
         # lie side by side in one table
         k = x.shape[1]

@@ -82,6 +82,6 @@ class Projection:
         """The product, or a promise of it where the residual stream can compute and add it in one kernel."""
         rows = x.shape[0]
         if (x.dtype == torch.bfloat16 and x.data_ptr() % 16 == 0 and self.fusable(min(rows, ops.FUSED_MAX_ROWS))
-                and (self.fusable(rows) or linear_kernels.residual_in_passes(rows, self.out_features))):
+                and (self.fusable(rows) or rows <= linear_kernels.RESIDUAL_PASSES_ROWS)):
             return DeferredProduct(self, x)
         return self(x)
