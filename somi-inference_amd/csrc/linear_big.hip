@@ -82,6 +82,7 @@ struct BigArgs {
     int splits;                       // workgroups per tile: split s walks the stages s, s + splits, s + 2 splits, ...
                                       // (the splits of a tile run side by side and so read neighbouring lines of a row)
     int stats_rows;                   // rows of stats_out (one per 64 columns of the tiles)
+    int reduce_plain;                 // the splits' sums end as the plain form does: out = s * sum + bias in bfloat16
 };
 
 template <int N> __device__ __forceinline__ void big_wait_vmcnt() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
@@ -580,6 +581,47 @@ big_split_reduce_kernel(const BigArgs p) {
     }
 }
 
+// The end of the plain form where K was split: out = s[m] * (sum over the splits, in split order) + bias -> bfloat16.
+// A workgroup takes 16 rows x 64 columns, as big_split_reduce_kernel does.
+__global__ void __launch_bounds__(256)
+big_split_reduce_plain_kernel(const BigArgs p) {
+    const int row = threadIdx.x >> 4, cg = threadIdx.x & 15;
+    const int gm = blockIdx.y * 16 + row, gn = blockIdx.x * 64 + cg * 4;
+    const int M = p.M, N = p.N;
+    if (gm >= M || gn >= N) return;
+    const bool four = (N & 3) == 0 && ((uintptr_t)p.out & 7) == 0 && gn + 4 <= N;
+    f32x4 sum = {0.f, 0.f, 0.f, 0.f};
+    const float* pp = p.partial + (int64_t)gm * N + gn;
+    const int64_t plane = (int64_t)M * N;
+    if (four) {
+        int s = 0;
+        for (; s + 4 <= p.splits; s += 4) {
+            const f32x4 a = *(const f32x4*)(pp + s * plane), b = *(const f32x4*)(pp + (s + 1) * plane);
+            const f32x4 c = *(const f32x4*)(pp + (s + 2) * plane), d = *(const f32x4*)(pp + (s + 3) * plane);
+            sum += a;
+            sum += b;
+            sum += c;
+            sum += d;
+        }
+        for (; s < p.splits; ++s) sum += *(const f32x4*)(pp + s * plane);
+    } else {
+        for (int s = 0; s < p.splits; ++s)
+            for (int c = 0; c < 4; ++c)
+                if (gn + c < N) sum[c] += pp[s * plane + c];
+    }
+    const float scale = p.row_scale != nullptr ? p.row_scale[gm] : 1.f;
+    bf16* op = p.out + (int64_t)gm * N + gn;
+    if (four) {
+        bf16x4 v;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) v[c] = (bf16)(scale * sum[c] + (p.bias != nullptr ? p.bias[gn + c] : 0.f));
+        *(bf16x4*)op = v;
+    } else {
+        for (int c = 0; c < 4; ++c)
+            if (gn + c < N) op[c] = (bf16)(scale * sum[c] + (p.bias != nullptr ? p.bias[gn + c] : 0.f));
+    }
+}
+
 // ---------------------------------------------------------------------- host side
 static int big_compute_units() {
     static int cached[64];
@@ -632,7 +674,10 @@ static int big_launch_one(const BigArgs& args, hipStream_t stream) {
     hipLaunchKernelGGL((linear_big_kernel<BM, BN, S, NW, EPI, KTAIL>), dim3(per_die * 8), dim3(NW * 64), lds_bytes, stream, args);
     SOMI_LAUNCH_CHECK("linear_big");
     if (EPI == BIG_RESIDUAL && args.partial != nullptr) {
-        hipLaunchKernelGGL(big_split_reduce_kernel, dim3(args.stats_rows, ceil_div(args.M, 16)), dim3(256), 0, stream, args);
+        if (args.reduce_plain)
+            hipLaunchKernelGGL(big_split_reduce_plain_kernel, dim3(ceil_div(args.N, 64), ceil_div(args.M, 16)), dim3(256), 0, stream, args);
+        else
+            hipLaunchKernelGGL(big_split_reduce_kernel, dim3(args.stats_rows, ceil_div(args.M, 16)), dim3(256), 0, stream, args);
         SOMI_LAUNCH_CHECK("linear_big: reduce");
     }
     return 0;
@@ -740,9 +785,11 @@ extern "C" int somi_linear_big_splits(int m, int n, int k, int tile, int64_t wor
 }
 
 // out = s * (x . w^T) + bias -> bfloat16 [M, N]; with swiglu w is [N, K] with gate and up rows interleaved in blocks
-// of 16 and out is [M, N / 2] = silu(s g) * (s u).  row_scale (or null): s [M], see somi_row_scale.
+// of 16 and out is [M, N / 2] = silu(s g) * (s u).  row_scale (or null): s [M], see somi_row_scale.  workspace (or
+// null): as in somi_linear_big_residual, for the plain form (q/k/v of some hundred rows: 72 tiles at 7B sizes).
 extern "C" int somi_linear_big(const void* x, int64_t ldx, const void* w, int64_t ldw, const float* bias, void* out,
-                               int m, int n, int k, const float* row_scale, int swiglu, int tile, hipStream_t stream) {
+                               int m, int n, int k, const float* row_scale, int swiglu, int tile, float* workspace,
+                               int64_t workspace_floats, hipStream_t stream) {
     if (big_check("linear_big", x, ldx, w, ldw, m, n, k) != 0) return 1;
     SOMI_REQUIRE(out != nullptr, "linear_big: no output");
     SOMI_REQUIRE(!swiglu || (n % 32 == 0 && bias == nullptr), "linear_big: the gated form needs N a multiple of 32 and no bias");
@@ -751,6 +798,13 @@ extern "C" int somi_linear_big(const void* x, int64_t ldx, const void* w, int64_
     args.x = (const bf16*)x; args.ldx = ldx; args.w = (const bf16*)w; args.ldw = ldw; args.bias = bias;
     args.M = m; args.N = n; args.K = k; args.out = (bf16*)out;
     args.row_scale = row_scale;
+    SOMI_REQUIRE(workspace == nullptr || (((uintptr_t)workspace & 15) == 0 && workspace_floats >= 0),
+                 "linear_big: the workspace must be aligned to 16 bytes");
+    if (!swiglu && workspace != nullptr && somi_linear_big_splits(m, n, k, tile, workspace_floats) > 1) {
+        // the workgroups of a tile share its K and leave float32 sums; the reduce scales, adds the bias and rounds
+        args.reduce_plain = 1;
+        return big_launch<BIG_RESIDUAL>(args, tile, stream, workspace, workspace_floats);
+    }
     return swiglu ? big_launch<BIG_SWIGLU>(args, tile, stream) : big_launch<BIG_PLAIN>(args, tile, stream);
 }
 

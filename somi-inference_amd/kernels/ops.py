@@ -366,13 +366,14 @@ def big_supported(x: torch.Tensor, weight: torch.Tensor) -> bool:
 
 def linear_big(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None, *, swiglu: bool = False,
                eps: float = 0.0, stats: torch.Tensor | None = None, tile: int = 0,
-               out: torch.Tensor | None = None) -> torch.Tensor:
+               out: torch.Tensor | None = None, split_k: bool = True) -> torch.Tensor:
     """s * (x @ weight.T) (+ bias) -> bfloat16 for any number of rows, on 256-row tiles of the matrix cores.
     With ``stats`` ([blocks, width >= M] partial sums of squares, from :func:`linear_big_residual` or
     :func:`linear_residual`) the rows are scaled by s = 1 / sqrt(stats.sum(0) / K + eps): the product of
     RMS-normed rows when x holds ``norm_weight * h``.  With ``swiglu`` weight is [2 I, K] with gate and up rows
     interleaved in blocks of 16 and the result is silu(s g) * (s u) -> [M, I].  ``tile``: 0 lets the launcher
-    choose the tile width, 128 or 256 asks for it."""
+    choose the tile width, 128 or 256 asks for it.  ``split_k``: the ungated form may share a tile's K among
+    workgroups (through the device's workspace) where its tiles alone would leave most of the device idle."""
     m, n, k = _big_operands(x, weight, bias, "linear_big")
     if swiglu and (n % 32 or bias is not None):
         raise KernelError(f"linear_big: the gated form needs an even number of 16-row blocks and no bias, got N = {n}")
@@ -388,8 +389,11 @@ def linear_big(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None 
     if out is None:
         out = torch.empty((m, cols), dtype=torch.bfloat16, device=x.device)
     _need(out, "linear_big out", torch.bfloat16, (m, cols))
+    workspace = _mid_workspace(x.device) if split_k and not swiglu else None
     _check(library().somi_linear_big(_ptr(x), ctypes.c_int64(x.stride(0)), _ptr(weight), ctypes.c_int64(weight.stride(0)),
-                                     _ptr(bias), _ptr(out), m, n, k, _ptr(row_scale), 1 if swiglu else 0, int(tile), _stream()))
+                                     _ptr(bias), _ptr(out), m, n, k, _ptr(row_scale), 1 if swiglu else 0, int(tile),
+                                     _ptr(workspace), ctypes.c_int64(workspace.numel() if workspace is not None else 0),
+                                     _stream()))
     return out
 
 

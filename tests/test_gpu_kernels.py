@@ -745,6 +745,31 @@ def test_many_rows_product_into_the_residual_stream(m, n, k, tile):
         torch.testing.assert_close(got.float(), want, atol=0.02 * float(want.abs().max()), rtol=2e-2)
 
 
+@pytest.mark.parametrize("tile", [1, 0, 128], ids=["128-row", "chosen", "256x128"])
+@pytest.mark.parametrize("m,n,k", [(100, 520, 2056), (65, 130, 1024), (300, 96, 1032), (260, 300, 2056), (513, 200, 1536)])
+def test_many_rows_product_plain_with_k_split_over_workgroups(m, n, k, tile):
+    """The plain form where its tiles are few and K is long (q/k/v of some hundred rows): the workgroups of a tile
+    share its K, and a second kernel scales the rows, adds the bias and rounds.  Against float32 formulas and the
+    unsplit kernel, with and without the rows' scales."""
+    assert ops.linear_big_splits(m, n, k, tile=tile) > 1
+    x, w, bias = rnd(m, k, dtype="bfloat16", seed=1), rnd(n, k, dtype="bfloat16", seed=2, scale=0.3), rnd(n, seed=3)
+    want = F.linear(x.float(), w.float(), bias)
+    tol = dict(atol=0.02 * float(want.abs().max()), rtol=2e-2)
+    got = ops.linear_big(x, w, bias, tile=tile)
+    assert got.dtype == torch.bfloat16
+    torch.testing.assert_close(got.float(), want, **tol)
+    whole = ops.linear_big(x, w, bias, tile=tile, split_k=False)
+    torch.testing.assert_close(got.float(), whole.float(), atol=float(want.abs().max()) * 2 ** -7, rtol=2 ** -7)
+    torch.testing.assert_close(ops.linear_big(x, w, tile=tile).float(), F.linear(x.float(), w.float()), **tol)
+    eps, width = 1e-5, 16 * ((m + 15) // 16)
+    stats = torch.zeros(2, width, device=DEV)
+    stats[:, :m] = torch.rand(2, m, device=DEV) * k * 4
+    s = torch.rsqrt(stats[:, :m].sum(0) / k + eps)[:, None]
+    scaled = ops.linear_big(x, w, bias, eps=eps, stats=stats, tile=tile)
+    want_scaled = s * (x.float() @ w.float().t()) + bias
+    torch.testing.assert_close(scaled.float(), want_scaled, atol=0.02 * float(want_scaled.abs().max()), rtol=2e-2)
+
+
 @pytest.mark.parametrize("tile", [0, 1, 128, 256])
 @pytest.mark.parametrize("m,n,k", [(65, 130, 64), (128, 1000, 264), (300, 521, 200), (257, 72, 1032)])
 def test_many_rows_product_in_float32(m, n, k, tile):
