@@ -235,7 +235,10 @@ __device__ __forceinline__ float lanes4_sum(float v) {
     return __uint_as_float(b[0]) + __uint_as_float(b[1]);
 }
 
-#define DECODE_LDS_PAGES 512
+// Pages of a split that the LDS copy of the block table holds: a table of 512 pages (8,192 keys in pages of 16, what a
+// captured step of requests at 4,096 to 8,192 tokens allows) is one split, with four workgroups of head size 128 still
+// fitting a compute unit's LDS (38 KB each).
+#define DECODE_LDS_PAGES 768
 template <int DT>
 __global__ void __launch_bounds__(256)
 attention_decode_lds_kernel(const bf16* __restrict__ q, int64_t q_stride, const bf16* __restrict__ kc,

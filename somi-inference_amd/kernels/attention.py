@@ -6,27 +6,29 @@ import torch
 
 from . import ops
 
-# The decode kernel aims at one workgroup per compute unit (whole decode steps at 4,096 keys, 7B sizes, 256 units:
-# 8 / 16 / 32 / 64 requests 3.42 / 3.99 / 5.27 / 7.20 ms against 3.43 / 4.05 / 5.39 / 7.29 with two per unit; fewer are slower).
+# The decode kernel aims at two workgroups per compute unit, more for small heads (a workgroup keeps three 32-key tiles
+# in flight, whose bytes go with the head size): whole decode steps at 4,096 keys, 7B sizes, 256 units, take 4.05 / 5.28 /
+# 6.28 ms at 16 / 32 / 48 requests against 4.13 / 5.35 / 6.32 with one per unit; at 64 requests one workgroup each
+# (no split) is 2.5 % slower than two, from 128 on the requests alone give two per unit and nothing is split (the
+# merge kernel goes: 128 requests 4.9 % faster than with a forced split).
 MIN_SPLIT = 64                  # keys per split at least (a multiple of the 16-key tile)
 MAX_SPLITS = 1024               # what the merge kernel holds
 DECODE_PORTION = 8              # portions of at most this many tokens take the decode kernel (engine.batch.SHORT_ENTRY)
-
-
-UNIT_HEAD_DIM = 128             # workgroups per compute unit: UNIT_HEAD_DIM / head size, at least one
+UNIT_HEAD_DIM = 128             # workgroups per compute unit: UNIT_HEAD_DIM / head size, at least MIN_PER_UNIT
+MIN_PER_UNIT = 2
 
 
 def decode_splits(num_tokens: int, groups: int, max_context: int, page_size: int = 0,
                   head_dim: int = 128) -> tuple[int, int]:
     """(split_len, num_splits): how the keys of a request are cut over workgroups so that
-    ``num_tokens * groups * num_splits`` is about the number of compute units.  Boundaries are multiples of
+    ``num_tokens * groups * num_splits`` is about MIN_PER_UNIT times the number of compute units.  Boundaries are multiples of
     MIN_SPLIT in absolute positions.  With ``page_size`` a split is no longer than what the kernel that stages
     tiles through LDS takes (its list of a split's pages is in LDS): contexts beyond that are cut further instead
     of falling to the slower kernel (64 requests at 4,1xx tokens in tables 512 pages wide: 8.2 ms a step before,
     against 6.8 at 3,9xx tokens)."""
     max_context = max(1, max_context)
     most = (max_context + MIN_SPLIT - 1) // MIN_SPLIT
-    workgroups = ops.compute_units() * max(1, UNIT_HEAD_DIM // max(1, head_dim))
+    workgroups = ops.compute_units() * max(MIN_PER_UNIT, UNIT_HEAD_DIM // max(1, head_dim))
     splits = max(1, min(workgroups // max(1, num_tokens * groups), most, MAX_SPLITS))
     split_len = ((max_context + splits - 1) // splits + MIN_SPLIT - 1) // MIN_SPLIT * MIN_SPLIT
     if page_size > 0:
