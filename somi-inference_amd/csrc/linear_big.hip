@@ -740,30 +740,33 @@ static int big_check(const char* what, const void* x, int64_t ldx, const void* w
 }
 
 // s[m] = 1 / sqrt(sum_b stats[b][m] / k + eps): the scale an RMS norm gives row m, from the partial sums of squares
-// that the residual forms leave (here and in linear_fused.hip).  A workgroup takes 32 rows; thread (row, e) adds the
-// blocks b = e, e + 8, e + 16, ... in that order, and the eight sums of a row are added as a fixed tree, so a row's
-// scale does not depend on how many rows there are.
+// that the residual forms leave (here and in linear_fused.hip).  A workgroup takes 8 rows; thread (row, e) adds the
+// blocks b = e, e + 32, e + 64, ... in that order, and the 32 sums of a row are added as a fixed tree, so a row's
+// scale does not depend on how many rows there are.  (Some hundred blocks of a few-rows producer, 128 rows: 8 us with
+// 32 rows a workgroup, where four workgroups walked 28 blocks a thread.)
+#define ROW_SCALE_ROWS 8
 __global__ void __launch_bounds__(256)
 row_scale_kernel(const float* __restrict__ stats, int blocks, int width, int m, float inv_k, float eps, float* __restrict__ out) {
-    __shared__ float parts[8][33];
-    const int r = threadIdx.x & 31, e = threadIdx.x >> 5;
-    const int row = blockIdx.x * 32 + r;
+    __shared__ float parts[32][ROW_SCALE_ROWS + 1];
+    const int r = threadIdx.x & (ROW_SCALE_ROWS - 1), e = threadIdx.x / ROW_SCALE_ROWS;
+    const int row = blockIdx.x * ROW_SCALE_ROWS + r;
     float part = 0.f;
     if (row < m)
-        for (int b = e; b < blocks; b += 8) part += stats[(int64_t)b * width + row];
+        for (int b = e; b < blocks; b += 32) part += stats[(int64_t)b * width + row];
     parts[e][r] = part;
     __syncthreads();
-    if (e == 0 && row < m) {
-        const float sum = ((parts[0][r] + parts[1][r]) + (parts[2][r] + parts[3][r])) +
-                          ((parts[4][r] + parts[5][r]) + (parts[6][r] + parts[7][r]));
-        out[row] = rsqrtf(sum * inv_k + eps);
+    // pairs 16 apart, then 8, 4, 2, 1: the same tree for every row
+    for (int half = 16; half > 0; half >>= 1) {
+        if (e < half) parts[e][r] += parts[e + half][r];
+        __syncthreads();
     }
+    if (e == 0 && row < m) out[row] = rsqrtf(parts[0][r] * inv_k + eps);
 }
 
 extern "C" int somi_row_scale(const float* stats, int blocks, int width, int m, int k, float eps, float* out, hipStream_t stream) {
     SOMI_REQUIRE(stats != nullptr && out != nullptr && blocks > 0 && m > 0 && width >= m && k > 0,
                  "row_scale: bad arguments (blocks=%d width=%d m=%d k=%d)", blocks, width, m, k);
-    hipLaunchKernelGGL(row_scale_kernel, dim3(ceil_div(m, 32)), dim3(256), 0, stream, stats, blocks, width, m, 1.f / (float)k, eps, out);
+    hipLaunchKernelGGL(row_scale_kernel, dim3(ceil_div(m, ROW_SCALE_ROWS)), dim3(256), 0, stream, stats, blocks, width, m, 1.f / (float)k, eps, out);
     SOMI_LAUNCH_CHECK("row_scale");
     return 0;
 }
