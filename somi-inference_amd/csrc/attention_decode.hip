@@ -258,10 +258,13 @@ attention_decode_lds_kernel(const bf16* __restrict__ q, int64_t q_stride, const 
     __shared__ __attribute__((aligned(16))) bf16 vs[2][D * VROW];
     __shared__ int pages[DECODE_LDS_PAGES];
 
-    const int ti = blockIdx.x;
+    // the key/value heads of a token are neighbours in the grid: they start together and walk the same pages at the
+    // same pace, so that the 4 KB pieces of a page that they read (one per head, next to each other) are asked for
+    // at about the same time (steps of 96 to 256 requests 1 to 2 % shorter than with the tokens as neighbours)
+    const int ti = blockIdx.y;
     const int t = token_list ? token_list[ti] : ti;
     const int G = nq / nkv, HB = (G + 15) / 16;
-    const int kvh = blockIdx.y / HB, hb = blockIdx.y % HB;
+    const int kvh = blockIdx.x / HB, hb = blockIdx.x % HB;
     const int split = blockIdx.z;
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, r = lane & 15, g = lane >> 4;
 
@@ -516,9 +519,10 @@ static int launch_decode(const void* q, int64_t q_stride, const void* kc, const 
     const int G = nq / nkv, HB = (G + 15) / 16;
     const size_t smem = (size_t)(waves * DT * 256 + waves * 32) * sizeof(float);
     const bool pow2_pages = (page_size & (page_size - 1)) == 0;
-    if (DT >= 2 && DT <= 8 && pow2_pages && split_len / page_size + 2 + 8 <= DECODE_LDS_PAGES)   // + a tile's overhang
+    if (DT >= 2 && DT <= 8 && pow2_pages && n_list <= 65535 &&
+        split_len / page_size + 2 + 8 <= DECODE_LDS_PAGES)                                        // + a tile's overhang
         // head sizes 32..128: keys and values staged through LDS (two tiles fit)
-        hipLaunchKernelGGL((attention_decode_lds_kernel<(DT >= 2 && DT <= 8 ? DT : 2)>), dim3(n_list, nkv * HB, num_splits),
+        hipLaunchKernelGGL((attention_decode_lds_kernel<(DT >= 2 && DT <= 8 ? DT : 2)>), dim3(nkv * HB, n_list, num_splits),
                            dim3(256), 0, stream, (const bf16*)q, q_stride, (const bf16*)kc, (const bf16*)vc, block_table,
                            max_blocks, token_list, token_entry, positions, nq, nkv, page_size, window, scale, split_len,
                            num_splits, (bf16*)out, part_acc, part_ml);
