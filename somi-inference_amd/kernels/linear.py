@@ -12,14 +12,21 @@ SKINNY_ROWS = 64       # up to here the few-rows kernels run; beyond, the many-r
 RESIDUAL_PASSES_ROWS = 128   # up to here a product into the residual stream with few columns runs in passes of 64 rows
 
 
+LONG_K = 8192            # a K that the split-K kernel cuts into eight pieces of sixteen chunks
+FEW_COLUMNS_PER_UNIT = 32     # up to this many columns per compute unit the few-rows kernel has two workgroups a unit at most
+MANY_COLUMNS_PER_UNIT = 64    # from this many on its workgroups come in several rounds, each reading all of x again
+
+
 def _mid_is_faster(m: int, n: int, k: int) -> bool:
-    """Measured inside decode steps at 7B layer sizes: from 17 rows on, the kernel that shares x inside a
-    workgroup and splits K over workgroups wins where K is long and the columns are few (down: 26 + 5 us
-    against 38 at 32 rows, 34 + 5 against 53 at 64) and where there are very many columns (gate_up: steps of
-    20 to 32 requests 1.7 % shorter, 58 + 8 us against 79 at 64 rows)."""
+    """From 17 rows on, the kernel that shares x inside a workgroup and splits K over workgroups wins where K is
+    long and the columns are few for the device (7B down projection on 256 units: 26 + 5 us against 38 at 32 rows,
+    34 + 5 against 53 at 64) and where there are very many columns (gate_up: steps of 20 to 32 requests 1.7 %
+    shorter, 58 + 8 us against 79 at 64 rows).  Measured inside decode steps at 7B layer sizes; the bounds on the
+    columns go with the device's compute units."""
     if m <= 16:
         return False
-    return (k >= 8192 and n <= 8192) or n >= 16384
+    units = ops.compute_units()
+    return (k >= LONG_K and n <= FEW_COLUMNS_PER_UNIT * units) or n >= MANY_COLUMNS_PER_UNIT * units
 
 
 def prefers_mid_passes(m: int, n: int, k: int) -> bool:
@@ -28,10 +35,10 @@ def prefers_mid_passes(m: int, n: int, k: int) -> bool:
     too few to fill the device there (7B down projection: 62 to 67 us at 65 to 128 rows against 157).  The product
     into the residual stream has ways of its own (passes that add into the stream up to 128 rows, the many-rows
     kernel with K split over workgroups beyond); this is for a product that is kept."""
-    return SKINNY_ROWS < m <= MID_PASSES_ROWS and k >= 8192 and n <= 8192
+    return SKINNY_ROWS < m <= MID_PASSES_ROWS and k >= LONG_K and n <= FEW_COLUMNS_PER_UNIT * ops.compute_units()
 
 
-RESIDUAL_PASSES_MAX_K = 8192     # below this K
+RESIDUAL_PASSES_MAX_K = LONG_K   # below this K
 
 
 def residual_in_passes(m: int, n: int, k: int) -> bool:
@@ -40,7 +47,8 @@ def residual_in_passes(m: int, n: int, k: int) -> bool:
     device there, and with so short a K sharing it among workgroups does not pay (7B sizes, 128 rows, inside decode
     steps: two passes 2 x 12 us, the many-rows kernel with K split 35 + 12).  A long K (down) is what that split is
     for: steps of 80 / 96 / 128 requests are 3.4 / 2.5 / 2.4 % shorter with it than with passes."""
-    return ops.FUSED_MAX_ROWS < m <= RESIDUAL_PASSES_ROWS and n <= 8192 and k < RESIDUAL_PASSES_MAX_K
+    return (ops.FUSED_MAX_ROWS < m <= RESIDUAL_PASSES_ROWS and n <= FEW_COLUMNS_PER_UNIT * ops.compute_units()
+            and k < RESIDUAL_PASSES_MAX_K)
 
 
 def linear_swiglu(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:

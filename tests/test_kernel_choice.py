@@ -45,7 +45,7 @@ def test_a_split_is_no_longer_than_the_page_list_in_lds_holds(device_of_256_unit
     assert choice.decode_splits(256, 4, 16384, 0, 128) == (16384, 1)
 
 
-def test_rows_of_a_product_into_the_stream_choose_their_kernel():
+def test_rows_of_a_product_into_the_stream_choose_their_kernel(device_of_256_units):
     # o of 65 to 128 requests (short K, few columns) runs in passes of the few-rows kernel; down (long K) does not
     assert products.residual_in_passes(96, 3584, 3584) and products.residual_in_passes(128, 3584, 3584)
     assert not products.residual_in_passes(96, 3584, 18944)
@@ -54,6 +54,9 @@ def test_rows_of_a_product_into_the_stream_choose_their_kernel():
     # a kept product with a long K and few columns: passes of the split-K kernel up to 128 rows
     assert products.prefers_mid_passes(100, 3584, 18944) and not products.prefers_mid_passes(129, 3584, 18944)
     assert not products.prefers_mid_passes(100, 37888, 3584)
+    # the few-rows choice between the kernel that splits K and the one that does not goes with the device's units
+    assert products._mid_is_faster(32, 3584, 18944) and products._mid_is_faster(64, 37888, 3584)
+    assert not products._mid_is_faster(16, 3584, 18944) and not products._mid_is_faster(64, 4608, 3584)
 
 
 def test_token_view_reads_prompt_and_output_as_one_sequence_without_copying():
