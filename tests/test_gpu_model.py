@@ -220,12 +220,43 @@ def test_step_contract_errors(model_folders):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", NAMES)
+def test_decode_steps_of_many_requests_against_the_plain_implementation(name, dtype, peaky_folders, oracle):
+    """70, 100, 150 and 260 requests decoding together (the products of 65 to 128 rows in passes and on the 128-row
+    tile, beyond on 256-row tiles with K shared by workgroups, logits of many rows in one pass): four steps each,
+    through the captured graphs, and after the last one the logits of a handful of requests, short and long ones,
+    against the plain implementation."""
+    vocab, bs = TINY[name]["config"].vocab_size, TINY[name]["block_size"]
+    pages = 270 * ((40 + 4 + bs - 1) // bs + 1)
+    runner, _ = make_engine(peaky_folders[name], dtype, bs, pages, max_requests=270)
+    for batch in (70, 100, 150, 260):
+        ids = [f"m{batch}_{i}" for i in range(batch)]
+        tokens = [token_ids(vocab, 2 + (i * 11) % 39, 500 + batch + i) for i in range(batch)]
+        for rid, prompt in zip(ids, tokens):
+            runner.begin(rid)
+            runner.step([StepEntry(rid, prompt[:-1], [])])
+        for step in range(4):
+            logits = runner.step([StepEntry(rid, [seq[-1]], [0]) for rid, seq in zip(ids, tokens)])
+            if step < 3:
+                for seq, token in zip(tokens, logits.argmax(dim=-1).tolist()):
+                    seq.append(int(token))
+        logits = logits.cpu()
+        for i in (0, 1, batch // 3, 64, batch - 2, batch - 1):
+            assert_close(logits[i], oracle("peaky", name, tokens[i])[-1], dtype,
+                         f"{name} {dtype}: request {i} of {batch} after {len(tokens[i])} tokens")
+        for rid in ids:
+            runner.end(rid)
+    runner.cache.check_invariants()
+    assert runner.cache.free_pages() == [pages] * len(runner.cache.groups)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_captured_decode_steps_replay_like_eager_steps(dtype, model_folders):
     """Decode steps are captured as HIP graphs per number of rows (4, 48 and 80 here, the entries padded up to
-    them).  Batches of 3, 40 and 70 requests (the largest
-    takes the library matrix product inside the graph, the others the kernels that fuse norm, rotation and
-    residual add into the products) are replayed several times, with eager work and synchronisations in
-    between, and every replay is compared with the same step run without graphs."""
+    them).  Batches of 3, 40 and 70 requests (the largest takes the products of more than 64 rows inside the
+    graph, the others the few-rows kernels that fuse norm, rotation and residual add into the products) are
+    replayed several times, with eager work and synchronisations in between, and every replay is compared with
+    the same step run without graphs."""
     from somi_inference_amd.models import load_model, make_runner
     from somi_inference_amd.engine import ModelRunner
     from somi_inference_amd.cache import CacheManager
