@@ -151,3 +151,31 @@ def test_greedy_and_seeded_temperature_generation(dtype, wide, plain_side):
     assert heavy >= 4, "the distributions are flat: a draw says little about the logits"
     assert llm.kv_manager.free_pages() == [48]
     json.dumps(sampled)      # plain lists of ints
+
+
+def test_many_requests_decode_together_at_the_real_width(wide):
+    """150 and 260 requests in one decode step in bfloat16: at these widths the products into the stream and the
+    q/k/v product share a tile's K among workgroups, and the logits of all rows come from one pass over the output
+    matrix.  The logits of a handful of requests against the plain implementation."""
+    folder, cfg, weights = wide
+    llm = LLM(folder, dtype="bfloat16", block_size=16, num_blocks=300, max_concurrent=270, eos_token_id=-1)
+    runner = llm.runner
+    for batch in (150, 260):
+        ids = [f"w{batch}_{i}" for i in range(batch)]
+        tokens = [token_ids(VOCAB, 2 + (i * 5) % 11, 900 + batch + i) for i in range(batch)]
+        for rid, prompt in zip(ids, tokens):
+            runner.begin(rid)
+            runner.step([StepEntry(rid, prompt[:-1], [])])
+        for step in range(2):
+            logits = runner.step([StepEntry(rid, [seq[-1]], [0]) for rid, seq in zip(ids, tokens)])
+            if step == 0:
+                for seq, token in zip(tokens, logits.argmax(dim=-1).tolist()):
+                    seq.append(int(token))
+        logits = logits.cpu()
+        assert logits.shape == (batch, VOCAB) and logits.dtype == torch.float32
+        for i in (0, 64, 129, batch - 1):
+            want = plain.model_logits(cfg, weights, tokens[i])[-1]
+            assert_close(logits[i], want, "bfloat16", f"request {i} of {batch} after {len(tokens[i])} tokens")
+        for rid in ids:
+            runner.end(rid)
+    assert llm.kv_manager.free_pages() == [300]
