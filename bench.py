@@ -26,7 +26,7 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E bandwidth
 PEAK_FLOPS = {"bfloat16": 2.5e15, "float32": 157.3e12}   # dense MFMA peaks
-POINT_BATCHES = (1, 64, 96, 128)      # decode is also measured at these numbers of requests ("points")
+POINT_BATCHES = (1, 64, 96, 128, 256)      # decode is also measured at these numbers of requests ("points")
 
 
 # layer sizes of the Qwen2.5 family: (layers, hidden, heads, kv heads, head_dim, intermediate, rms_norm_eps,
@@ -54,7 +54,7 @@ def parse_args() -> argparse.Namespace:
     p.add_argument("--block-size", type=int, default=16)
     p.add_argument("--prefill-tokens", type=int, default=2048)
     p.add_argument("--seed", type=int, default=0)
-    p.add_argument("--no-points", action="store_true", help="skip the decode points at other batch sizes (1, 64, 96, 128)")
+    p.add_argument("--no-points", action="store_true", help="skip the decode points at other batch sizes (1, 64, 96, 128, 256)")
     p.add_argument("--no-prefill", action="store_true", help="skip the prefill measurement")
     p.add_argument("--no-peaks", action="store_true", help="skip the measurement of the machine's own peaks")
     p.add_argument("--output-file", type=str, default=None, help="Append the result line to a JSONL file.")
@@ -276,7 +276,7 @@ def main() -> int:
         roofline["frac_of_measured"] = round(achieved / peaks["stream_read_gbs"], 4)
     line = {
         "metric": f"decode tok/s at batch {args.batch}, Qwen2.5-{args.sizes.upper()} layer sizes "
-                  f"(plus prefill tok/s at {args.prefill_tokens:,} tokens, batch 1/64/96/128 points)",
+                  f"(plus prefill tok/s at {args.prefill_tokens:,} tokens, batch 1/64/96/128/256 points)",
         "value": round(main_run["tok_s"], 2), "unit": "tokens/s", "n_gpus": 1,
         "steps": main_run["steps"], "warmup": main_run["warmup"], "ms_per_step": round(main_run["ms"], 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
