@@ -179,6 +179,79 @@ def test_decoder_layer_with_zero_projections_is_identity():
     torch.testing.assert_close(P.decoder_layer(h, w, 0, cfg, torch.arange(5)), h)
 
 
+def _layer_with_constant_attention(h=8, i=12, nq=2, nkv=1, d=4):
+    """One layer whose attention term does not depend on its input: q/k/v matrices and the q/k biases are
+    zero, the value bias and o_proj are random, so every softmax is uniform over equal values and the term is
+    c = o_proj(bv repeated for the query heads).  The feed-forward weights are random."""
+    cfg, w = _tiny_weights(h=h, i=i, nq=nq, nkv=nkv, d=d)
+    p = "model.layers.0.self_attn"
+    for name in ("q_proj", "k_proj", "v_proj"):
+        w[f"{p}.{name}.weight"] = torch.zeros_like(w[f"{p}.{name}.weight"])
+    w[f"{p}.q_proj.bias"] = torch.zeros(nq * d)
+    w[f"{p}.k_proj.bias"] = torch.zeros(nkv * d)
+    bv = w[f"{p}.v_proj.bias"]
+    c = w[f"{p}.o_proj.weight"] @ bv.view(nkv, d).repeat_interleave(nq // nkv, dim=0).reshape(nq * d)
+    return cfg, w, c
+
+
+def test_each_norm_weight_sits_before_its_own_half_of_the_layer():
+    """/root/reference/somi_inference/models/qwen2.py:333-339: input_layernorm feeds the attention,
+    post_attention_layernorm feeds the feed-forward.  A zero input_layernorm weight makes the attention's input
+    zero, so the attention term is the constant o_proj(repeat(bv)) (biases only) whatever h is, and the
+    feed-forward still sees h + that constant; a zero post_attention_layernorm weight makes the feed-forward
+    term vanish (swiglu(0) = 0) and leaves h + attention.  With the two weights swapped both fail."""
+    cfg, w = _tiny_weights()
+    p = "model.layers.0"
+    h, positions = torch.randn(5, 8), torch.arange(5)
+    norm2 = torch.linspace(0.5, 1.5, 8)
+    bv = w[f"{p}.self_attn.v_proj.bias"]
+    constant = w[f"{p}.self_attn.o_proj.weight"] @ bv.view(1, 4).repeat_interleave(2, dim=0).reshape(8)
+    assert constant.abs().max() > 1e-3
+
+    first_off = dict(w)
+    first_off[f"{p}.input_layernorm.weight"] = torch.zeros(8)
+    first_off[f"{p}.post_attention_layernorm.weight"] = norm2
+    mid = h + constant
+    x = norm2 * mid * torch.rsqrt(mid.pow(2).mean(-1, keepdim=True) + 1e-6)
+    mlp = (F.silu(x @ w[f"{p}.mlp.gate_proj.weight"].t()) * (x @ w[f"{p}.mlp.up_proj.weight"].t())) \
+        @ w[f"{p}.mlp.down_proj.weight"].t()
+    torch.testing.assert_close(P.decoder_layer(h, first_off, 0, cfg, positions), mid + mlp, atol=1e-5, rtol=1e-5)
+
+    second_off = dict(w)
+    second_off[f"{p}.input_layernorm.weight"] = torch.linspace(1.5, 0.5, 8)
+    second_off[f"{p}.post_attention_layernorm.weight"] = torch.zeros(8)
+    got = P.decoder_layer(h, second_off, 0, cfg, positions)
+    normed = second_off[f"{p}.input_layernorm.weight"] * h * torch.rsqrt(h.pow(2).mean(-1, keepdim=True) + 1e-6)
+    attention = P.attention_block(normed, w, f"{p}.self_attn", cfg, positions, None)
+    torch.testing.assert_close(got, h + attention, atol=1e-5, rtol=1e-5)
+    assert not torch.allclose(got, h + constant, atol=1e-3)        # the attention does see its normed input
+
+
+def test_feed_forward_reads_the_stream_after_the_attention_was_added():
+    """/root/reference/somi_inference/models/qwen2.py:335-339: residual = h + attn; the second norm and the
+    feed-forward read that sum, not the layer's input.  With an attention term that is a known constant c the
+    layer is h + c + swiglu(rms_norm(h + c)), computed here inline with library routines.  A parallel block
+    (feed-forward from norm2(h)) or a feed-forward added to h alone fails it."""
+    cfg, w, c = _layer_with_constant_attention()
+    assert c.abs().max() > 1e-2
+    p = "model.layers.0"
+    norm2 = torch.linspace(0.6, 1.7, 8)
+    w[f"{p}.input_layernorm.weight"] = torch.linspace(1.4, 0.3, 8)
+    w[f"{p}.post_attention_layernorm.weight"] = norm2
+    h = torch.randn(6, 8)
+    mid = h + c
+    x = F.rms_norm(mid, (8,), norm2, 1e-6)
+    mlp = F.linear(F.silu(F.linear(x, w[f"{p}.mlp.gate_proj.weight"])) * F.linear(x, w[f"{p}.mlp.up_proj.weight"]),
+                   w[f"{p}.mlp.down_proj.weight"])
+    got = P.decoder_layer(h, w, 0, cfg, torch.arange(6))
+    torch.testing.assert_close(got, mid + mlp, atol=1e-5, rtol=1e-5)
+    # what the two plausible mistakes would give is far from it
+    x_parallel = F.rms_norm(h, (8,), norm2, 1e-6)
+    mlp_parallel = F.linear(F.silu(F.linear(x_parallel, w[f"{p}.mlp.gate_proj.weight"]))
+                            * F.linear(x_parallel, w[f"{p}.mlp.up_proj.weight"]), w[f"{p}.mlp.down_proj.weight"])
+    assert not torch.allclose(got, mid + mlp_parallel, atol=1e-3)
+
+
 def test_model_is_causal_and_tied_head_uses_embedding():
     cfg, w = _tiny_weights(layers=2)
     ids = [3, 1, 4, 1, 5, 9, 2, 6]
