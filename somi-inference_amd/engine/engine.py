@@ -179,8 +179,22 @@ class Engine:
 
     def abort(self, requests: list[Request]) -> None:
         """Take these requests out of the queues and give back their pages and state slots, whatever state a
-        failed step left them in; tokens that were drawn but not read are dropped."""
-        self._unread = None
+        failed step left them in.  Tokens of a launched step that the host has not read yet are read first, so
+        that a request which is not among ``requests`` (queued earlier through ``add_request`` and still
+        running) keeps its real token instead of a stand-in; if they cannot be read (the device failed), every
+        request that holds a stand-in is aborted too."""
+        requests = list(requests)
+        pending = self._unread
+        try:
+            self._read_unread()
+        except Exception:
+            self._unread = None
+            for portion in pending.portions:
+                if portion.request not in requests:
+                    requests.append(portion.request)
         for request in requests:
+            if request.status is not RequestStatus.FINISHED and request.output_tokens \
+                    and request.output_tokens[-1] == UNREAD:
+                request.output_tokens.pop()
             self.scheduler.abort(request)
         self.scheduler.drain_finished()

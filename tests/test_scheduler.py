@@ -345,6 +345,44 @@ def test_a_step_that_raises_aborts_the_calls_requests_and_the_next_call_runs():
     assert [(r.request_id, r.output_tokens) for r in done] == [(2, [7, 8])]
 
 
+def test_a_bystander_keeps_its_tokens_when_another_calls_step_raises_while_running_ahead():
+    """A request queued earlier through add_request decodes beside the request of a run() call.  The step that
+    raises was launched ahead of reading the step before, so both requests hold a stand-in for an unread token.
+    The call's request is aborted; the bystander gets its real token, is fed that token (not a stand-in) in its
+    next step and ends with exactly its scripted tokens."""
+    scripts = {0: [30, 31, 32, 33, 34, 35, 36, 37], 1: [40, 41, 42, 43, 44, 45]}
+
+    class FailingAhead(AheadRunner):
+        fail_at = 4
+
+        def step(self, entries, device_tokens=None):
+            if len(self.calls) == self.fail_at and device_tokens is not None:
+                self.fail_at = -1
+                raise RuntimeError("the step failed")
+            return super().step(entries, device_tokens)
+
+    cache = make_cache(num_blocks=16)
+    scheduler = Scheduler(cache, max_concurrent=4, max_num_batched_tokens=64)
+    runner, sampler = FailingAhead(cache), AheadSampler(scripts)
+    runner.log = sampler.log = []
+    engine = Engine(runner, scheduler, sampler, None)
+    bystander, mine = request(0, 5, 8), request(1, 3, 6)
+    engine.add_request(bystander)
+    with pytest.raises(RuntimeError, match="the step failed"):
+        engine.run(deque([(0, mine)]))
+    assert engine.steps_run_ahead >= 1, "the failing step was not one launched ahead"
+    assert mine.finish_reason == "aborted" and UNREAD not in mine.output_tokens
+    assert bystander.status is not RequestStatus.FINISHED and scheduler.running == [bystander]
+    assert UNREAD not in bystander.output_tokens
+    assert bystander.output_tokens == scripts[0][:len(bystander.output_tokens)] and bystander.output_tokens
+    done = engine.run()
+    assert [(r.request_id, r.output_tokens, r.finish_reason) for r in done] == [(0, scripts[0], "length")]
+    fed = [tokens for call in runner.calls for rid, tokens, _ in call if rid == 0]
+    assert all(t >= 0 for tokens in fed for t in tokens)
+    assert [tokens[0] for tokens in fed[1:]] == scripts[0][:7]
+    assert cache.free_pages() == [16] and not cache.live_requests()
+
+
 def test_portions_come_in_multiples_of_the_granule_except_the_one_that_ends_the_prompt():
     cache = make_cache(num_blocks=32)
     scheduler = Scheduler(cache, max_concurrent=4, max_num_batched_tokens=11, chunk=10, granule=4)
