@@ -235,9 +235,13 @@ attention_prefill_kernel(const bf16* __restrict__ q, int64_t q_stride, const bf1
 //   read serves at once fall into different pairs of the 32 banks; with 20 dwords a row the counters showed
 //   twice the conflicts).
 #define PREFILL_LDS_TOTAL (96 * 1024)   // LDS of a workgroup, tiles (static) and page list (dynamic) together, that a launch may ask for
-#ifndef PREFILL_WIDE_GROUPS
-#define PREFILL_WIDE_GROUPS 600    // from this many 128-query groups on, workgroups take 128 queries, else 64 (measured: 448 groups 72 against 82 us with 64 queries, 672 groups 136 against 119)
-#endif
+// The launch shapes go with the number of workgroups per compute unit, so their bounds are multiples of the device's
+// units (the figures in brackets: on the 256 units of an MI355X, where they were measured at 28 query heads).
+static int prefill_wide_groups(int units) { return units * 75 / 32; }        // [600] from this many 128-query groups on, workgroups take 128 queries, else 64 (448 groups 72 against 82 us with 64 queries, 672 groups 136 against 119)
+static int prefill_wide_groups_cached(int units) { return units; }           // [256] the same where at least half of the keys were cached before the step
+static int prefill_tile_wide_groups(int units) { return 2 * units; }         // [512] from this many 256-query groups on the tile kernel takes 256 queries a workgroup
+static int prefill_key_split_below(int units) { return 7 * units / 2; }      // [896] below this many 64-query workgroups two wavefronts share a query block's keys
+                                                                             // (448 workgroups 29 against 33 us, 512 tokens after 3,584 cached 83 against 108; 896 workgroups the same; 1,120 workgroups 94 against 89)
 // The launch shapes of the LDS kernel; a caller may ask for one (tests do, to reach each at small sizes).
 #define PREFILL_SHAPE_AUTO 0
 #define PREFILL_SHAPE_NARROW 1     // 64 queries a workgroup
@@ -245,18 +249,7 @@ attention_prefill_kernel(const bf16* __restrict__ q, int64_t q_stride, const bf1
 #define PREFILL_SHAPE_WIDE 3       // 128 queries
 #define PREFILL_SHAPE_TILE 4       // the 32 x 32 tile kernel: 128 queries a workgroup, two key splits
 #define PREFILL_SHAPE_TILE_WIDE 5  // the 32 x 32 tile kernel: 256 queries a workgroup
-#define PREFILL_TILE_WIDE_GROUPS 512   // from this many 256-query groups on the tile kernel takes 256 queries a workgroup
-#ifndef PREFILL_KEY_SPLIT_BELOW
-#define PREFILL_KEY_SPLIT_BELOW 896   // below this many 64-query workgroups two wavefronts share a query block's keys
-                                      // (measured at 7B head counts: 448 workgroups 29 against 33 us, 512 tokens after
-                                      // 3,584 cached 83 against 108; 896 workgroups the same; 1,120 workgroups 94 against 89)
-#endif
-#ifndef PREFILL_KEY_SPLIT_REACH
-#define PREFILL_KEY_SPLIT_REACH 1024  // and only where the longest workgroup walks at least this many keys (32 tiles)
-#endif
-#ifndef PREFILL_WIDE_GROUPS_CACHED
-#define PREFILL_WIDE_GROUPS_CACHED 256   // the same where at least half of the keys were cached before the step
-#endif
+#define PREFILL_KEY_SPLIT_REACH 1024  // keys are shared only where the longest workgroup walks at least this many (32 tiles)
 // KS = 2: twice the wavefronts; each query block is owned by KS of them, which take the 32-key tiles in turn
 // (tile index modulo KS, by absolute position) and join their sums, maxima and outputs through LDS at the
 // end.  The longest workgroup, which sets the time of a short prompt, has half as many steps to walk.
@@ -572,23 +565,36 @@ static int prefill_page_entries(int max_blocks, int page_size, int window) {
     return entries;
 }
 
+// The launch shape of the LDS kernel for a step.  128 queries per workgroup read every key and value tile half as
+// often as 64 do, but the longest workgroup sets the time: with few workgroups the smaller ones spread better over
+// the compute units.  Where most keys were cached before the step (max_context, the caller's hint of the longest
+// context a portion ends at, is several portions long) all workgroups are long and the wide ones win earlier.  Few
+// workgroups of 64 queries with many tiles each share a query block's keys between two wavefronts.
+static int prefill_lds_choice(int n_entries, int max_entry_len, int max_context, int nq, int window, bool split_fits,
+                              int units) {
+    const int64_t wide_groups = (int64_t)ceil_div(max_entry_len, 128) * n_entries * nq;
+    int reach = max_context;
+    if (window > 0 && reach > window + max_entry_len) reach = window + max_entry_len;
+    if (wide_groups >= prefill_wide_groups(units) ||
+        (wide_groups >= prefill_wide_groups_cached(units) && reach >= 2 * max_entry_len))
+        return PREFILL_SHAPE_WIDE;
+    const int64_t narrow_groups = (int64_t)ceil_div(max_entry_len, 64) * n_entries * nq;
+    if (narrow_groups < prefill_key_split_below(units) && reach >= PREFILL_KEY_SPLIT_REACH && split_fits)
+        return PREFILL_SHAPE_SPLIT;
+    return PREFILL_SHAPE_NARROW;
+}
+
 template <int DT>
 static int launch_prefill_lds(const void* q, int64_t q_stride, const void* kc, const void* vc, const int* block_table,
                               int max_blocks, const int* entry_start, const int* entry_first_pos, const int* entry_len, int n_entries,
                               int max_entry_len, int max_context, int shape, int nq, int nkv, int page_size,
                               int window, float scale, void* out, hipStream_t stream) {
-    // 128 queries per workgroup read every key and value tile half as often as 64 do, but the longest
-    // workgroup sets the time: with few workgroups the smaller ones spread better over the compute units.
-    // Where most keys were cached before the step (max_context, the caller's hint of the longest context a
-    // portion ends at, is several portions long) all workgroups are long and the wide ones win earlier.
-    const int64_t wide_groups = (int64_t)ceil_div(max_entry_len, 128) * n_entries * nq;
-    int reach = max_context;
-    if (window > 0 && reach > window + max_entry_len) reach = window + max_entry_len;
-    bool wide = wide_groups >= PREFILL_WIDE_GROUPS ||
-                (wide_groups >= PREFILL_WIDE_GROUPS_CACHED && reach >= 2 * max_entry_len);
-    if (shape != PREFILL_SHAPE_AUTO) wide = shape == PREFILL_SHAPE_WIDE;
-    const dim3 grid(nq, n_entries, ceil_div(max_entry_len, wide ? 128 : 64));
     const size_t page_list = (size_t)prefill_page_entries(max_blocks, page_size, window) * sizeof(int);
+    const bool split_fits = (int)page_list + prefill_lds_static(DT * 16, 2) <= PREFILL_LDS_TOTAL;
+    if (shape == PREFILL_SHAPE_AUTO)
+        shape = prefill_lds_choice(n_entries, max_entry_len, max_context, nq, window, split_fits, somi_units());
+    const bool wide = shape == PREFILL_SHAPE_WIDE;
+    const dim3 grid(nq, n_entries, ceil_div(max_entry_len, wide ? 128 : 64));
     if (wide) {
         if (page_list > 16 * 1024)                       // with the tiles beyond the default limit of LDS
             (void)hipFuncSetAttribute((const void*)attention_prefill_lds_kernel<DT, 2, 1>,
@@ -596,10 +602,7 @@ static int launch_prefill_lds(const void* q, int64_t q_stride, const void* kc, c
         hipLaunchKernelGGL((attention_prefill_lds_kernel<DT, 2, 1>), grid, dim3(256), page_list, stream, (const bf16*)q,
                            q_stride, (const bf16*)kc, (const bf16*)vc, block_table, max_blocks, entry_start,
                            entry_first_pos, entry_len, nq, nkv, page_size, window, scale * 1.44269504088896341f, (bf16*)out);
-    } else if ((shape == PREFILL_SHAPE_AUTO
-                    ? (int64_t)grid.x * grid.y * grid.z < PREFILL_KEY_SPLIT_BELOW && reach >= PREFILL_KEY_SPLIT_REACH
-                    : shape == PREFILL_SHAPE_SPLIT) &&
-               (int)page_list + prefill_lds_static(DT * 16, 2) <= PREFILL_LDS_TOTAL) {
+    } else if (shape == PREFILL_SHAPE_SPLIT && split_fits) {
         // few workgroups with many tiles each: the keys of a query block are split over two wavefronts
         if (page_list > 16 * 1024)
             (void)hipFuncSetAttribute((const void*)attention_prefill_lds_kernel<DT, 1, 2>,
@@ -667,7 +670,7 @@ extern "C" int somi_attention_prefill(const void* q, int64_t q_stride, const voi
                      D, page_size, max_blocks);
     if (tile_ok && (shape == PREFILL_SHAPE_AUTO || shape >= PREFILL_SHAPE_TILE)) {
         const int64_t groups = (int64_t)ceil_div(max_entry_len, 256) * n_entries * nq;
-        const bool wide = shape == PREFILL_SHAPE_AUTO ? groups >= PREFILL_TILE_WIDE_GROUPS : shape == PREFILL_SHAPE_TILE_WIDE;
+        const bool wide = shape == PREFILL_SHAPE_AUTO ? groups >= prefill_tile_wide_groups(somi_units()) : shape == PREFILL_SHAPE_TILE_WIDE;
         return somi_prefill_tile(q, q_stride, k_cache, v_cache, block_table, max_blocks, entry_start, entry_first_pos, entry_len,
                                  n_entries, max_entry_len, wide, nq, nkv, D, page_size, window, scale, out, stream);
     }
@@ -699,4 +702,17 @@ extern "C" int somi_attention_prefill(const void* q, int64_t q_stride, const voi
 #undef SOMI_PREFILL
 #undef SOMI_PREFILL_LDS
     return somi_fail("attention_prefill: unsupported head_dim %d", D);
+}
+
+// The launch shape (PREFILL_SHAPE_*) that somi_attention_prefill chooses with shape 0 on a device of `units` compute
+// units (0: the current device), given whether the tile kernel applies (head sizes 64 and 128, pages of 8 keys or
+// more) and whether the LDS kernel's two-wavefront form fits LDS: what a test of the choice asks without a GPU.
+extern "C" int somi_attention_prefill_choice(int n_entries, int max_entry_len, int max_context, int nq, int window,
+                                             int tile_applies, int split_fits, int units) {
+    if (units <= 0) units = somi_units();
+    if (tile_applies) {
+        const int64_t groups = (int64_t)ceil_div(max_entry_len, 256) * n_entries * nq;
+        return groups >= prefill_tile_wide_groups(units) ? PREFILL_SHAPE_TILE_WIDE : PREFILL_SHAPE_TILE;
+    }
+    return prefill_lds_choice(n_entries, max_entry_len, max_context, nq, window, split_fits != 0, units);
 }

@@ -29,7 +29,7 @@ HIPCC_FLAGS = [
     f"--offload-arch={OFFLOAD_ARCH}", "-O3", "-fPIC", "-std=c++17",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-result",
-] + os.environ.get("SOMI_HIPCC_EXTRA", "").split()
+]
 
 
 class KernelBuildError(RuntimeError):

@@ -35,6 +35,10 @@ template <typename T> __device__ __forceinline__ T from_float(float v);
 template <> __device__ __forceinline__ float from_float<float>(float v) { return v; }
 template <> __device__ __forceinline__ bf16 from_float<bf16>(float v) { return (bf16)v; }
 
+// Compute units of the current device, asked once per device (256 if the device cannot be asked): what the launch
+// shapes size their workgroup counts by.
+int somi_units();
+
 static inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 static inline int64_t ceil_div64(int64_t a, int64_t b) { return (a + b - 1) / b; }
 

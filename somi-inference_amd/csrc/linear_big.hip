@@ -623,17 +623,7 @@ big_split_reduce_plain_kernel(const BigArgs p) {
 }
 
 // ---------------------------------------------------------------------- host side
-static int big_compute_units() {
-    static int cached[64];
-    int device = 0;
-    if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) return 256;
-    if (cached[device] == 0) {
-        hipDeviceProp_t prop;
-        cached[device] = hipGetDeviceProperties(&prop, device) == hipSuccess && prop.multiProcessorCount > 0
-                             ? prop.multiProcessorCount : 256;
-    }
-    return cached[device];
-}
+static int big_compute_units() { return somi_units(); }
 
 // The wide tile moves fewer bytes per product and wins where it fills the device; the narrow one has twice the
 // workgroups.  Costs in units of a narrow tile's time: rounds of tiles x the tile's size (the narrow tile is

@@ -441,15 +441,8 @@ static int mid_launch(const void* x, const void* w, const float* bias, void* out
     return 0;
 }
 
-// A program that measures other shapes (chunk sizes, depths) can include this file with SOMI_MID_NO_ENTRY_POINTS
-// defined and instantiate the launchers above itself; the library builds what follows.
-#ifndef SOMI_MID_NO_ENTRY_POINTS
-#ifndef MID_CK
 #define MID_CK 64                                // K values per chunk and chunks in flight of the shapes that are built
-#endif
-#ifndef MID_DEPTH
 #define MID_DEPTH 2
-#endif
 
 template <int MT, typename TO, int FUSE>
 static int mid_strips(const void* x, const void* w, const float* bias, void* out, int M, int N, int K, int strips,
@@ -469,20 +462,18 @@ static int64_t mid_workspace_floats(int M, int N, int strips, int splits) {
 // compute unit a workgroup; K is split until there are about two workgroups per compute unit, in
 // pieces of at least 8 chunks, within the workspace.  Chosen by whole decode steps of 64 requests at 7B
 // layer sizes (7.7 ms with this rule: down in 8 splits, gate_up in 2; 8.0 ms with at most 5 or 3 splits,
-// 7.9 ms with twice as many); timing the kernel alone in a loop ranks the shapes differently.
-#ifndef MID_TARGET_WORKGROUPS
-#define MID_TARGET_WORKGROUPS 448             // K is split until about this many workgroups run
-#endif
-#ifndef MID_MIN_CHUNKS
+// 7.9 ms with twice as many); timing the kernel alone in a loop ranks the shapes differently.  The counts go
+// with the device's compute units (on the 256 of an MI355X: 448 workgroups aimed at, K split below 384 tiles, two
+// strips from 256 tiles of 128 columns on).
 #define MID_MIN_CHUNKS 8                      // chunks of K a split holds at least
-#endif
-static void mid_shape(int M, int N, int K, bool swiglu, int64_t workspace_floats, int* strips, int* splits) {
+static void mid_shape(int M, int N, int K, bool swiglu, int64_t workspace_floats, int units, int* strips, int* splits) {
     const int chunks = ceil_div(K, MID_CK);
-    int ns = (swiglu || ceil_div(N, 128) >= 256) ? 2 : 1;
+    const int target = 7 * units / 4;         // K is split until about this many workgroups run
+    int ns = (swiglu || ceil_div(N, 128) >= units) ? 2 : 1;
     int tiles = ceil_div(N, 64 * ns);
     int ks = 1;
-    if (tiles < 384) {
-        ks = min(ceil_div(MID_TARGET_WORKGROUPS, tiles), max(1, chunks / MID_MIN_CHUNKS));
+    if (tiles < 3 * units / 2) {
+        ks = min(ceil_div(target, tiles), max(1, chunks / MID_MIN_CHUNKS));
         const int per = ceil_div(chunks, ks);
         ks = ceil_div(chunks, per);                  // no empty split
     }
@@ -532,14 +523,14 @@ extern "C" int somi_linear_mid(const void* x, const void* w, const float* bias, 
     SOMI_REQUIRE(!swiglu || (N % 32 == 0 && bias == nullptr), "linear_mid: the gated form needs whole pairs of strips and no bias");
     if (M == 0) return 0;
     int strips, splits;
-    mid_shape(M, N, K, swiglu != 0, workspace ? workspace_floats : 0, &strips, &splits);
+    mid_shape(M, N, K, swiglu != 0, workspace ? workspace_floats : 0, somi_units(), &strips, &splits);
     return mid_dispatch<MID_PLAIN>(x, w, bias, out, out_dtype, M, N, K, strips, splits, swiglu != 0, workspace, MidFusion{}, stream);
 }
 
 // Column tiles (= rows of the statistics) that somi_linear_mid_residual launches for these sizes.
 extern "C" int somi_linear_mid_residual_tiles(int M, int N, int K) {
     int strips, splits;
-    mid_shape(M, N, K, false, 0, &strips, &splits);
+    mid_shape(M, N, K, false, 0, somi_units(), &strips, &splits);
     return ceil_div(N, 64 * strips);
 }
 
@@ -558,7 +549,7 @@ extern "C" int somi_linear_mid_residual(const void* x, const void* w, const floa
                  "linear_mid_residual: a stride of %d floats does not hold the sums of %d rows", stats_stride, M);
     if (M == 0) return 0;
     int strips, splits;
-    mid_shape(M, N, K, false, workspace ? workspace_floats : 0, &strips, &splits);
+    mid_shape(M, N, K, false, workspace ? workspace_floats : 0, somi_units(), &strips, &splits);
     MidFusion fusion{};
     fusion.h = h;
     fusion.norm_w = norm_w;
@@ -579,7 +570,7 @@ extern "C" int somi_linear_mid_scaled(const void* x, float eps, const float* sta
     SOMI_REQUIRE(!swiglu || (N % 32 == 0 && bias == nullptr), "linear_mid_scaled: the gated form needs whole pairs of strips and no bias");
     if (M == 0) return 0;
     int strips, splits;
-    mid_shape(M, N, K, swiglu != 0, workspace ? workspace_floats : 0, &strips, &splits);
+    mid_shape(M, N, K, swiglu != 0, workspace ? workspace_floats : 0, somi_units(), &strips, &splits);
     MidFusion fusion{};
     fusion.stats_in = stats;
     fusion.stats_blocks = stats_blocks;
@@ -601,4 +592,12 @@ extern "C" int somi_linear_mid_shaped(const void* x, const void* w, const float*
     if (M == 0) return 0;
     return mid_dispatch<MID_PLAIN>(x, w, bias, out, out_dtype, M, N, K, strips, splits, swiglu != 0, workspace, MidFusion{}, stream);
 }
-#endif
+
+// The launch shape (strips per wavefront, splits of K) that the entry points above choose for these sizes on a device
+// of `units` compute units (0: the current device): what a test of the choice asks without a GPU.
+extern "C" int somi_linear_mid_choice(int M, int N, int K, int swiglu, int64_t workspace_floats, int units, int* strips,
+                                      int* splits) {
+    SOMI_REQUIRE(M > 0 && N > 0 && K > 0 && units >= 0 && strips && splits, "linear_mid_choice: bad arguments");
+    mid_shape(M, N, K, swiglu != 0, workspace_floats, units > 0 ? units : somi_units(), strips, splits);
+    return 0;
+}

@@ -235,9 +235,6 @@ static int skinny_launch(const void* x, const void* w, const float* bias, void* 
     return 0;
 }
 
-// A program that measures other shapes (chunk sizes, depths) can include this file with SOMI_SKINNY_NO_ENTRY_POINTS
-// defined and instantiate the launchers above itself; the library builds what follows.
-#ifndef SOMI_SKINNY_NO_ENTRY_POINTS
 // The shapes that are built: 1, 2 or 4 strips with chunks of 64, two chunks in flight.
 template <int MT, typename TO>
 static int skinny_strips(const void* x, const void* w, const float* bias, void* out, int M, int N, int K, int waves,
@@ -321,4 +318,3 @@ extern "C" int somi_linear_skinny_shaped(const void* x, const void* w, const flo
     if (M == 0) return 0;
     return skinny_dispatch(x, w, bias, out, out_dtype, M, N, K, waves, strips, false, stream);
 }
-#endif

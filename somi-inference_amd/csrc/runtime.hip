@@ -36,4 +36,16 @@ extern "C" int somi_compute_units() {
     return prop.multiProcessorCount;
 }
 
+int somi_units() {
+    static int cached[64];
+    int device = 0;
+    if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) return 256;
+    if (cached[device] == 0) {
+        hipDeviceProp_t prop;
+        cached[device] = hipGetDeviceProperties(&prop, device) == hipSuccess && prop.multiProcessorCount > 0
+                             ? prop.multiProcessorCount : 256;
+    }
+    return cached[device];
+}
+
 extern "C" int somi_abi_version() { return 1; }

@@ -48,6 +48,18 @@ class PagedView:
 
 
 @dataclass
+class EntrySplit:
+    """The step's entries cut in two by their length, for a mixer that serves long portions and single tokens
+    (or portions of a few) with different kernels.  Every token of the step lies in exactly one of the two."""
+
+    threshold: int
+    long_entry_len: torch.Tensor    # [E] int32: an entry's length if it is longer than the threshold, else 0
+    short_tokens: torch.Tensor      # [Ns] int32: flat indices of the tokens of the entries of at most threshold tokens
+    num_long_tokens: int
+    num_short_tokens: int
+
+
+@dataclass
 class StepBatch:
     num_tokens: int
     num_entries: int
@@ -60,16 +72,21 @@ class StepBatch:
     context_lens: torch.Tensor      # [E] int32: tokens of each request after this step
     state_slots: torch.Tensor       # [E] int32
     logit_rows: torch.Tensor        # [R] int32 flat token indices whose logits are wanted
-    long_entry_len: torch.Tensor    # [E] int32: an entry's length if it is longer than SHORT_ENTRY tokens, else 0
-    short_tokens: torch.Tensor      # [Ns] int32: flat indices of the tokens of the entries of at most SHORT_ENTRY tokens
     paged: list[PagedView]
     entries: list[EntryInfo]        # host mirror
     max_entry_len: int
     max_context: int
     block_size: int
+    splits: dict[int, EntrySplit] = field(default_factory=dict)
 
-
-SHORT_ENTRY = 8      # entries of at most this many tokens are attended token by token (the decode kernel)
+    def split(self, threshold: int) -> EntrySplit:
+        """The entries cut at ``threshold`` tokens.  Only the thresholds that the model's mixers declared
+        (``Mixer.entry_split``) are laid out: the lists travel with the step's one copy to the device."""
+        try:
+            return self.splits[int(threshold)]
+        except KeyError:
+            raise KeyError(f"this step holds no split of its entries at {threshold} tokens (it has "
+                           f"{sorted(self.splits)}): a mixer declares the threshold it needs as entry_split") from None
 
 
 class _Padding:
@@ -80,9 +97,14 @@ class _Padding:
 PADDING = _Padding()      # request id of a padding entry
 
 
-def _layout(entries: list[StepEntry], cache: CacheManager, table_widths: list[int] | None, pad_to: int = 0):
+FIXED_SECTIONS = 8      # token ids, positions, token -> entry, entry offsets, first positions, contexts, slots, logit rows
+
+
+def _layout(entries: list[StepEntry], cache: CacheManager, table_widths: list[int] | None, pad_to: int = 0,
+            entry_splits: tuple[int, ...] = ()):
     """The step as host arrays: (sections, infos, widths).  ``table_widths`` fixes the block tables'
     widths (a captured graph needs the same layout at every replay); None = as narrow as possible.
+    ``entry_splits``: the lengths at which mixers want the entries cut into long and short ones.
 
     ``pad_to``: entries are added until there are this many.  A padding entry is one token (id 0, position 0)
     of no request: it stores nothing (slot -1), reads page 0 through a table row of zeros, uses the state
@@ -136,44 +158,57 @@ def _layout(entries: list[StepEntry], cache: CacheManager, table_widths: list[in
         np.asarray([i.first_position + i.length for i in infos], dtype=np.int32),
         np.asarray([i.state_slot for i in infos], dtype=np.int32),
         np.asarray(logit_rows, dtype=np.int32),
-        np.asarray([i.length if i.length > SHORT_ENTRY else 0 for i in infos], dtype=np.int32),
-        np.asarray([t for i in infos if i.length <= SHORT_ENTRY for t in range(i.start, i.start + i.length)], dtype=np.int32),
     ]
+    assert len(sections) == FIXED_SECTIONS
     for table, slots in zip(tables, slot_maps):
         sections += [slots, table.reshape(-1)]
+    for threshold in entry_splits:
+        sections += [
+            np.asarray([i.length if i.length > threshold else 0 for i in infos], dtype=np.int32),
+            np.asarray([t for i in infos if i.length <= threshold for t in range(i.start, i.start + i.length)],
+                       dtype=np.int32),
+        ]
     return sections, infos, widths
 
 
 def _views(on_device: torch.Tensor, sizes: list[int], infos: list[EntryInfo], widths: list[int],
-           page_sizes: list[int], block_size: int, max_context: int | None = None) -> StepBatch:
+           page_sizes: list[int], block_size: int, max_context: int | None = None,
+           entry_splits: tuple[int, ...] = ()) -> StepBatch:
     offsets = np.cumsum([0] + sizes)
 
     def part(i: int) -> torch.Tensor:
         return on_device[int(offsets[i]):int(offsets[i + 1])]
 
     e = len(infos)
-    paged = [PagedView(part(10 + 2 * g), part(11 + 2 * g).view(e, widths[g]), size) for g, size in enumerate(page_sizes)]
+    paged = [PagedView(part(FIXED_SECTIONS + 2 * g), part(FIXED_SECTIONS + 1 + 2 * g).view(e, widths[g]), size)
+             for g, size in enumerate(page_sizes)]
+    splits = {}
+    for index, threshold in enumerate(entry_splits):
+        at = FIXED_SECTIONS + 2 * len(page_sizes) + 2 * index
+        short = sum(i.length for i in infos if i.length <= threshold)
+        splits[int(threshold)] = EntrySplit(int(threshold), part(at), part(at + 1), sizes[0] - short, short)
     return StepBatch(
         num_tokens=sizes[0], num_entries=e, num_logit_rows=sizes[7],
         token_ids=part(0), positions=part(1), token_entry=part(2), entry_start=part(3),
         entry_first_position=part(4), context_lens=part(5), state_slots=part(6), logit_rows=part(7),
-        long_entry_len=part(8), short_tokens=part(9), paged=paged, entries=infos,
+        paged=paged, entries=infos, splits=splits,
         max_entry_len=max((i.length for i in infos), default=0),
         max_context=max_context if max_context is not None else max((i.first_position + i.length for i in infos), default=0),
         block_size=block_size,
     )
 
 
-def build_step(entries: list[StepEntry], cache: CacheManager, device: torch.device) -> StepBatch:
+def build_step(entries: list[StepEntry], cache: CacheManager, device: torch.device,
+               entry_splits: tuple[int, ...] = ()) -> StepBatch:
     """Lay out the step on the host and copy it to the device in one transfer.
 
     Pages for the new tokens must already be reserved: slot mappings and block
     tables are read from the cache manager as they stand.
     """
-    sections, infos, widths = _layout(entries, cache, None)
+    sections, infos, widths = _layout(entries, cache, None, entry_splits=tuple(entry_splits))
     packed = torch.from_numpy(np.concatenate(sections))
     return _views(packed.to(device), [s.size for s in sections], infos, widths,
-                  [group.page_size for group in cache.groups], cache.block_size)
+                  [group.page_size for group in cache.groups], cache.block_size, entry_splits=tuple(entry_splits))
 
 
 class StaticStep:
@@ -181,10 +216,11 @@ class StaticStep:
     whose device arrays stay in place, so that a captured HIP graph can be replayed on new contents."""
 
     def __init__(self, entries: list[StepEntry], cache: CacheManager, device: torch.device,
-                 table_widths: list[int], pad_to: int = 0) -> None:
+                 table_widths: list[int], pad_to: int = 0, entry_splits: tuple[int, ...] = ()) -> None:
         self.table_widths = list(table_widths)
         self.pad_to = int(pad_to)
-        sections, infos, widths = _layout(entries, cache, self.table_widths, self.pad_to)
+        self.entry_splits = tuple(entry_splits)
+        sections, infos, widths = _layout(entries, cache, self.table_widths, self.pad_to, self.entry_splits)
         self.sizes = [s.size for s in sections]
         # Staging in pinned memory, several buffers in turn: the copy to the device is asynchronous, so the
         # host can lay out the next step while the device still runs this one.  A buffer is written again
@@ -196,7 +232,8 @@ class StaticStep:
         # kernels that size their launch by the context use the widest the tables allow
         sizes = [group.page_size for group in cache.groups]
         self.batch = _views(self.device_buffer, self.sizes, infos, widths, sizes, cache.block_size,
-                            max_context=min((w * s for w, s in zip(self.table_widths, sizes)), default=cache.block_size))
+                            max_context=min((w * s for w, s in zip(self.table_widths, sizes)), default=cache.block_size),
+                            entry_splits=self.entry_splits)
         self._fill(sections, infos)
 
     STAGING = 4
@@ -213,7 +250,7 @@ class StaticStep:
         self.batch.entries = infos
 
     def update(self, entries: list[StepEntry], cache: CacheManager) -> StepBatch:
-        sections, infos, _ = _layout(entries, cache, self.table_widths, self.pad_to)
+        sections, infos, _ = _layout(entries, cache, self.table_widths, self.pad_to, self.entry_splits)
         if [s.size for s in sections] != self.sizes:
             raise ValueError("the entries do not fit the shape this step was laid out for")
         self._fill(sections, infos)

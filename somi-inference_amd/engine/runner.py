@@ -65,6 +65,7 @@ class ModelRunner:
         self.cache = cache
         self.device = model.runtime.device
         self.vocab_size = model.vocab_size
+        self.entry_splits = tuple(model.entry_splits())     # lengths at which mixers want a step's entries cut in two
         self.steps_run = 0
         # Steps of single decoded tokens are bound by kernel launches, so they are captured once per
         # shape as a HIP graph and replayed.  Only for models whose parts all launch on the stream
@@ -130,7 +131,7 @@ class ModelRunner:
             if self.decode_graphs and all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries):
                 logits = self._decode_with_graph(entries, device_tokens)
             else:
-                batch = build_step(entries, self.cache, self.device)
+                batch = build_step(entries, self.cache, self.device, self.entry_splits)
                 if device_tokens is not None:
                     batch.token_ids.copy_(device_tokens)
                 logits = self.model.forward(batch, self.cache.layer_caches)
@@ -149,7 +150,7 @@ class ModelRunner:
                  device_tokens: torch.Tensor | None = None) -> _DecodeGraph:
         """Capture the decode step of ``rows`` rows and these table widths, laid out for ``entries`` (none: all
         rows are padding, which is how graphs are captured ahead of any request)."""
-        static = StaticStep(entries, self.cache, self.device, widths, pad_to=rows)
+        static = StaticStep(entries, self.cache, self.device, widths, pad_to=rows, entry_splits=self.entry_splits)
         if device_tokens is not None:
             static.batch.token_ids[:len(entries)].copy_(device_tokens)
         # once outside a capture: lazy initialisation (library handles, first allocations) must

@@ -13,7 +13,8 @@ from . import ops
 # merge kernel goes: 128 requests 4.9 % faster than with a forced split).
 MIN_SPLIT = 64                  # keys per split at least (a multiple of the 16-key tile)
 MAX_SPLITS = 1024               # what the merge kernel holds
-DECODE_PORTION = 8              # portions of at most this many tokens take the decode kernel (engine.batch.SHORT_ENTRY)
+DECODE_PORTION = 8              # portions of at most this many tokens take the decode kernel; the attention part
+                                # declares it as its entry_split, so the step lists long entries and short tokens by it
 UNIT_HEAD_DIM = 128             # workgroups per compute unit: UNIT_HEAD_DIM / head size, at least MIN_PER_UNIT
 MIN_PER_UNIT = 2
 
@@ -62,14 +63,18 @@ def paged_attention(qkv: torch.Tensor, num_heads: int, k_cache: torch.Tensor, v_
         # portions of prompts: query tiles against key tiles.  Single tokens (and portions of a few) in the same
         # batch keep the kernel that splits a request's keys over workgroups: as a query tile with one live row
         # one workgroup would walk the whole context.
-        short = step.short_tokens.numel()
+        split = step.split(DECODE_PORTION)
+        short = split.num_short_tokens
+        if split.num_long_tokens + short != step.num_tokens or short != split.short_tokens.numel():
+            raise ValueError(f"the step's split at {DECODE_PORTION} tokens covers {split.num_long_tokens} + {short} "
+                             f"of its {step.num_tokens} tokens: rows of the output would stay unwritten")
         ops.attention_prefill(qkv, qkv.shape[1], k_cache, v_cache, block_table, step.entry_start,
                               step.entry_first_position, step.max_entry_len, num_heads, window, scale, out,
-                              max_context=step.max_context, entry_len=step.long_entry_len if short else None)
+                              max_context=step.max_context, entry_len=split.long_entry_len if short else None)
         if short:
             split_len, num_splits = decode_splits(short, groups, step.max_context, k_cache.shape[2], head_dim)
             ops.attention_decode(qkv, qkv.shape[1], k_cache, v_cache, block_table, step.token_entry, step.positions,
-                                 num_heads, window, scale, split_len, num_splits, out, token_list=step.short_tokens)
+                                 num_heads, window, scale, split_len, num_splits, out, token_list=split.short_tokens)
         return out
     split_len, num_splits = decode_splits(step.num_tokens, groups, step.max_context, k_cache.shape[2], head_dim)
     ops.attention_decode(qkv, qkv.shape[1], k_cache, v_cache, block_table, step.token_entry, step.positions,

@@ -81,6 +81,11 @@ class DecoderModel:
         import math
         return math.lcm(*[int(getattr(layer.mixer, "portion_granule", 1)) for layer in self.layers] or [1])
 
+    def entry_splits(self) -> list[int]:
+        """The entry lengths at which some mixer wants a step's entries cut into long and short ones."""
+        return sorted({int(layer.mixer.entry_split) for layer in self.layers
+                       if getattr(layer.mixer, "entry_split", None) is not None})
+
     # -------------------------------------------------------------------- cache
     def cache_needs(self) -> list[PagedSpec | FixedStateSpec | int | None]:
         """For each run of a layer: the cache its mixer needs, the index of the earlier

@@ -28,6 +28,7 @@ ROTATE_STORE_PASSES_ROWS = 128      # up to here the q/k/v product with rotation
 class GroupedQueryAttention(Mixer):
     graph_safe = True
     takes_normed_rows = True      # x only goes through the q/k/v projection, which norms rows while loading them
+    entry_split = attention_kernels.DECODE_PORTION    # longer portions take the tile kernel, the rest the decode kernel
 
     def __init__(self, prefix: str, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  position: PartSpec, qkv_bias: bool = True, out_bias: bool = False,

@@ -205,6 +205,8 @@ class Mixer(Part):
 
     takes_normed_rows = False      # True: x may arrive as parts.linear.NormedRows (rows still to be normed)
     portion_granule = 1            # a prompt portion that does not end its prompt holds a multiple of this many tokens
+    entry_split = None             # an int: ``step.split(entry_split)`` lists the entries longer than this many tokens
+                                   # and the tokens of the others, for mixers that serve the two with different kernels
 
     def forward(self, x: torch.Tensor, step: Any, cache: LayerCache | None) -> torch.Tensor:
         """x: [N, H] compute dtype -> [N, H] compute dtype, or a parts.linear.DeferredProduct of that shape

@@ -135,15 +135,19 @@ def read_model(model_dir: str, dtype=torch.float32) -> tuple[dict, dict]:
     return cfg, weights
 
 
-def model_logits(cfg: dict, w: dict, token_ids: list[int], first_position: int = 0) -> torch.Tensor:
+def model_logits(cfg: dict, w: dict, token_ids: list[int], first_position: int = 0,
+                 rows: list[int] | None = None) -> torch.Tensor:
     """models/qwen2.py:380-386 then models/qwen2_adapter.py:60-62: embed, layers, final norm, logits = h . E^T
-    (or lm_head when the checkpoint is untied).  Returns logits at every position, [T, V]."""
+    (or lm_head when the checkpoint is untied).  Returns logits at every position, [T, V], or at ``rows`` only
+    (the reference projects the last position alone, models/qwen2_adapter.py:95: the head works row by row)."""
     ids = torch.tensor(token_ids, dtype=torch.long)
     h = w["model.embed_tokens.weight"][ids]
     positions = torch.arange(first_position, first_position + len(token_ids))
     for index in range(cfg["num_hidden_layers"]):
         h = decoder_layer(h, w, index, cfg, positions)
     h = rms_norm(h, w["model.norm.weight"], cfg["rms_norm_eps"])
+    if rows is not None:
+        h = h[torch.tensor(rows, dtype=torch.long)]
     head = w["model.embed_tokens.weight"] if cfg.get("tie_word_embeddings", False) else w["lm_head.weight"]
     return h @ head.t()
 

@@ -190,7 +190,16 @@ def test_step_arrays_for_a_mixed_batch():
     assert step.paged[0].slot_mapping.tolist() == m.slots(0, "p", 0, 6) + m.slots(0, "d", 5, 1)
     assert step.max_entry_len == 6 and step.max_context == 6
     # no portion is longer than 8 tokens: every token is listed for the kernel that attends token by token
-    assert step.long_entry_len.tolist() == [0, 0] and step.short_tokens.tolist() == [0, 1, 2, 3, 4, 5, 6]
+    assert not step.splits
+    with pytest.raises(KeyError, match="entry_split"):
+        step.split(8)
+    # the lists a mixer asks for by declaring a threshold: entries longer than it, tokens of the others
+    cut = build_step(entries, m, torch.device("cpu"), entry_splits=(8, 4)).split(8)
+    assert cut.long_entry_len.tolist() == [0, 0] and cut.short_tokens.tolist() == [0, 1, 2, 3, 4, 5, 6]
+    assert (cut.num_long_tokens, cut.num_short_tokens) == (0, 7)
+    cut = build_step(entries, m, torch.device("cpu"), entry_splits=(8, 4)).split(4)
+    assert cut.long_entry_len.tolist() == [6, 0] and cut.short_tokens.tolist() == [6]
+    assert (cut.num_long_tokens, cut.num_short_tokens) == (6, 1)
     assert all(t.dtype == torch.int32 for t in (step.token_ids, step.positions, table, step.logit_rows))
 
 

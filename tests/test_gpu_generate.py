@@ -128,6 +128,72 @@ def test_temperature_sampling_does_not_depend_on_the_batch(dtype, model_folders)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_repetition_penalty_top_k_and_top_p_through_generate_follow_the_plain_rules(dtype, model_folders):
+    """Generation through the entry point with a repetition penalty (which reads each request's history, prompt
+    and outputs: /root/reference/somi_inference/core/continuous_batching.py:167, core/model_runner.py:36, and so
+    keeps the engine from running ahead), alone and with a temperature, top-k and top-p, in portions beside
+    decoding requests.  Every token of every request is held against the plain rules applied to the plain logits
+    of what the engine produced so far: the greedy token is the argmax of the penalised logits, a drawn token is
+    the one whose share of the plain distribution (penalty, temperature, top-k, top-p, softmax) covers the
+    request's uniform number."""
+    vocab = TINY["B"]["config"].vocab_size
+    prompts = [token_ids(vocab, n, 80 + n) for n in (4, 23, 40, 64, 100)]
+    cfg, weights = plain.read_model(model_folders["B"])
+    llm = LLM(model_folders["B"], dtype=dtype, block_size=8, num_blocks=96, max_concurrent=5,
+              max_num_batched_tokens=40, max_chunk=13, eos_token_id=-1)
+    exact = dtype == "float32"
+    penalty, new_tokens = 1.3, 16
+
+    greedy = llm.generate(prompts, max_new_tokens=new_tokens, temperature=0.0, repetition_penalty=penalty)
+    assert llm.engine.steps_run_ahead == 0 and llm.engine.num_steps > new_tokens
+    moved = 0
+    for index, (prompt, tokens) in enumerate(zip(prompts, greedy)):
+        assert len(tokens) == new_tokens
+        for n, token in enumerate(tokens):
+            history = prompt + tokens[:n]
+            logits = plain.model_logits(cfg, weights, history, rows=[len(history) - 1])[0]
+            ruled = plain.penalize_repetition(logits, history, penalty)
+            want = int(torch.argmax(ruled))
+            moved += int(want != int(torch.argmax(logits)))
+            if token != want:
+                assert not exact, f"prompt {index}, token {n}: {token} instead of {want}"
+                gap = float(ruled[want] - ruled[token])
+                assert 0.0 <= gap < 0.03, f"prompt {index}, token {n}: {token} instead of {want}, gap {gap}"
+    assert moved >= 5, "the penalty never changed the choice: the test says nothing about it"
+    unruled = llm.generate(prompts, max_new_tokens=new_tokens, temperature=0.0)
+    assert unruled != greedy
+
+    heavy = 0
+    for options in (dict(temperature=0.7, top_p=0.9), dict(temperature=0.9, top_k=12, top_p=0.8)):
+        seed = 31
+        drawn = llm.generate(prompts, max_new_tokens=new_tokens, repetition_penalty=penalty, seed=seed, **options)
+        assert drawn == llm.generate(prompts, max_new_tokens=new_tokens, repetition_penalty=penalty, seed=seed, **options)
+        for index, (prompt, tokens) in enumerate(zip(prompts, drawn)):
+            for n, token in enumerate(tokens):
+                history = prompt + tokens[:n]
+                logits = plain.model_logits(cfg, weights, history, rows=[len(history) - 1])[0]
+                share = plain.sampling_distribution(logits, history, options["temperature"], options.get("top_k", -1),
+                                                    options["top_p"], penalty).double()
+                cdf = torch.cumsum(share, dim=0)
+                u = uniform(seed + index, n)
+                low = float(cdf[token - 1]) if token > 0 else 0.0
+                # float32 holds the rules exactly.  bfloat16 logits differ by rounding: beside the 2 % of mass that
+                # may lie on the other side of an interval's edge, the entry at the edge of what top-k / top-p keep
+                # may fall on the other side of the cut, which rescales the cumulative sums by that entry's share
+                # (m / (1 - m) at the far end)
+                edge = float(share[share > 0].min())
+                slack = 1e-5 if exact else 0.02 + 1.5 * edge
+                assert low - slack <= u <= float(cdf[token]) + slack, \
+                    f"{options}, prompt {index}, draw {n}: token {token} covers [{low:.5f}, {float(cdf[token]):.5f}], drawn at {u:.5f}"
+                if exact:
+                    assert float(share[token]) > 0.0, f"{options}: token {token} lies outside what top-k / top-p keep"
+                heavy += int(int((share > 0).sum()) < vocab // 2)
+    assert heavy > 0, "top-k / top-p never cut anything away"
+    assert llm.kv_manager.free_pages() == [96]
+    llm.kv_manager.check_invariants()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_generation_of_the_windowed_configuration(dtype, model_folders):
     """Layers with a window of 20 keys beside layers that see everything: greedy tokens through the entry point
     (scheduler, captured decode steps, running ahead) against the plain implementation, with prompts shorter and

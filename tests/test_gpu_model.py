@@ -24,13 +24,14 @@ def peaky_folders(model_folders, tmp_path_factory):
 @pytest.fixture(scope="module")
 def oracle(model_folders, peaky_folders):
     """Plain logits of (folder kind, config name, token tuple), computed once."""
-    cache = {}
+    cache, models = {}, {}
 
     def get(kind: str, name: str, tokens: list[int]) -> torch.Tensor:
         key = (kind, name, tuple(tokens))
         if key not in cache:
-            folder = (model_folders if kind == "plain" else peaky_folders)[name]
-            cfg, weights = plain.read_model(folder)
+            if (kind, name) not in models:
+                models[(kind, name)] = plain.read_model((model_folders if kind == "plain" else peaky_folders)[name])
+            cfg, weights = models[(kind, name)]
             cache[key] = plain.model_logits(cfg, weights, tokens)
         return cache[key]
     return get
@@ -224,8 +225,9 @@ def test_step_contract_errors(model_folders):
 def test_decode_steps_of_many_requests_against_the_plain_implementation(name, dtype, peaky_folders, oracle):
     """70, 100, 150 and 260 requests decoding together (the products of 65 to 128 rows in passes and on the 128-row
     tile, beyond on 256-row tiles with K shared by workgroups, logits of many rows in one pass): four steps each,
-    through the captured graphs, and after the last one the logits of a handful of requests, short and long ones,
-    against the plain implementation."""
+    through the captured graphs, and after the last one the logits of every request, short and long ones,
+    against the plain implementation (a fault may sit in some rows of a tile only: at a pass's edge, in a padded
+    row of a graph's bucket)."""
     vocab, bs = TINY[name]["config"].vocab_size, TINY[name]["block_size"]
     pages = 270 * ((40 + 4 + bs - 1) // bs + 1)
     runner, _ = make_engine(peaky_folders[name], dtype, bs, pages, max_requests=270)
@@ -241,9 +243,8 @@ def test_decode_steps_of_many_requests_against_the_plain_implementation(name, dt
                 for seq, token in zip(tokens, logits.argmax(dim=-1).tolist()):
                     seq.append(int(token))
         logits = logits.cpu()
-        for i in (0, 1, batch // 3, 64, batch - 2, batch - 1):
-            assert_close(logits[i], oracle("peaky", name, tokens[i])[-1], dtype,
-                         f"{name} {dtype}: request {i} of {batch} after {len(tokens[i])} tokens")
+        want = torch.stack([oracle("peaky", name, tokens[i])[-1] for i in range(batch)])
+        assert_close(logits, want, dtype, f"{name} {dtype}: {batch} requests after 2 to 44 tokens", per_row=True)
         for rid in ids:
             runner.end(rid)
     runner.cache.check_invariants()

@@ -13,6 +13,7 @@ from somi_inference_amd.weights import RandomSource
 
 pytestmark = pytest.mark.gpu
 DEV = torch.device("cuda:0")
+SPLITS = (GroupedQueryAttention.entry_split,)      # what the runner takes from the model's mixers and hands to build_step
 DT = {"float32": torch.float32, "bfloat16": torch.bfloat16}
 TOL = {"float32": dict(atol=2e-5, rtol=1e-4), "bfloat16": dict(atol=3e-2, rtol=3e-2)}
 
@@ -100,7 +101,7 @@ def test_attention_part_whole_and_in_portions(dtype, nq, nkv, d, hidden, window)
         outs, at = [], 0
         for size in sizes:
             cache.reserve("r", size)
-            step = build_step([StepEntry("r", [0] * size, [])], cache, DEV)
+            step = build_step([StepEntry("r", [0] * size, [])], cache, DEV, SPLITS)
             outs.append(rows(attn.forward(x[at:at + size].contiguous(), step, cache.layer_caches[0])))
             cache.commit("r", size)
             at += size
@@ -130,7 +131,7 @@ def test_attention_part_reads_rows_still_to_be_normed(n_rows):
     for i, size in enumerate(sizes):
         cache.register(i)
         cache.reserve(i, size)
-    step = build_step([StepEntry(i, [0] * size, []) for i, size in enumerate(sizes)], cache, DEV)
+    step = build_step([StepEntry(i, [0] * size, []) for i, size in enumerate(sizes)], cache, DEV, SPLITS)
     got = rows(attn.forward(lazy, step, cache.layer_caches[0]))
     h1 = h0.cpu() + plain.swiglu(x0.float().cpu(), wf["m.gate_proj.weight"], wf["m.up_proj.weight"], wf["m.down_proj.weight"])
     x1 = plain.rms_norm(h1, wn["n.weight"], 1e-5)
@@ -166,11 +167,11 @@ def test_attention_part_far_key_among_hundreds_and_window_edge(dtype):
         want = plain.attention_block(x.float().cpu(), w, "a", cfg, torch.arange(length), window)
         cache.register("r")
         cache.reserve("r", length - 1)
-        attn.forward(x[:length - 1].contiguous(), build_step([StepEntry("r", [0] * (length - 1), [])], cache, DEV),
+        attn.forward(x[:length - 1].contiguous(), build_step([StepEntry("r", [0] * (length - 1), [])], cache, DEV, SPLITS),
                      cache.layer_caches[0])
         cache.commit("r", length - 1)
         cache.reserve("r", 1)
-        got = rows(attn.forward(x[length - 1:].contiguous(), build_step([StepEntry("r", [0], [])], cache, DEV),
+        got = rows(attn.forward(x[length - 1:].contiguous(), build_step([StepEntry("r", [0], [])], cache, DEV, SPLITS),
                                 cache.layer_caches[0]))
         if dtype == "float32":
             torch.testing.assert_close(got.cpu(), want[-1:], atol=1e-4, rtol=1e-3)
@@ -224,7 +225,7 @@ def test_block_with_zero_projections_is_the_identity():
     cache.reserve("r", 5)
     h = torch.randn(5, 32, device=DEV)
     stream = ResidualStream(h.clone())
-    block.forward(stream, build_step([StepEntry("r", [0] * 5, [])], cache, DEV), cache.layer_caches[0])
+    block.forward(stream, build_step([StepEntry("r", [0] * 5, [])], cache, DEV, SPLITS), cache.layer_caches[0])
     assert torch.equal(stream.settle(), h)
 
 

@@ -73,3 +73,47 @@ def test_token_view_reads_prompt_and_output_as_one_sequence_without_copying():
     with pytest.raises(IndexError):
         view[6]
     assert request != Request("r", [5, 6, 7], 4) and request == request      # a request is itself
+
+
+def test_launch_shapes_inside_the_library_go_with_the_devices_compute_units():
+    """The few-rows split-K product and the prefill attention size their launches by workgroups per compute unit.
+    The library answers for a device of any size without touching a GPU: on 256 units the figures that were
+    measured there, on a device of half or 304 units the same rules scaled."""
+    import ctypes
+    lib = ops.library()
+    strips, splits = ctypes.c_int(), ctypes.c_int()
+
+    def mid(m, n, k, swiglu, units, workspace=1 << 40):
+        assert lib.somi_linear_mid_choice(m, n, k, int(swiglu), ctypes.c_int64(workspace), units,
+                                          ctypes.byref(strips), ctypes.byref(splits)) == 0
+        return strips.value, splits.value
+
+    # 7B down projection, 64 rows, 256 units: 56 column tiles of 64, 296 chunks: 448 / 56 = 8 splits of 37 chunks
+    assert mid(64, 3584, 18944, False, 256) == (1, 8)
+    # gate_up (37,888 columns): two strips, 296 tiles < 384: 2 splits; on 128 units 296 tiles are enough: no split
+    assert mid(64, 37888, 3584, True, 256) == (2, 2)
+    assert mid(64, 37888, 3584, True, 128) == (2, 1)
+    # the same down projection on half the device is split half as often; without a workspace not at all
+    assert mid(64, 3584, 18944, False, 128) == (1, 4)
+    assert mid(64, 3584, 18944, False, 256, workspace=0) == (1, 1)
+    # the logits' 152,064 columns: two strips once 128-column tiles outnumber the units (1,188 tiles of 128)
+    assert mid(32, 152064, 3584, False, 256)[0] == 2 and mid(32, 152064, 3584, False, 2048)[0] == 1
+
+    NARROW, SPLIT, WIDE, TILE, TILE_WIDE = 1, 2, 3, 4, 5
+    shape = lambda entries, longest, context, nq, units, tile=0, fits=1, window=0: \
+        lib.somi_attention_prefill_choice(entries, longest, context, nq, window, tile, fits, units)
+    # 2,048 tokens, 28 heads, 256 units: 448 groups of 128 queries < 600: 64 queries a workgroup; 896 such
+    # workgroups are not below 896, so nothing is shared; on 304 units 896 < 1,064: two wavefronts share the keys
+    assert shape(1, 2048, 2048, 28, 256) == NARROW
+    assert shape(1, 2048, 2048, 28, 304) == SPLIT
+    assert shape(1, 2048, 2048, 28, 304, fits=0) == NARROW
+    # 3,072 tokens: 672 groups >= 600: 128 queries; on 304 units the bound is 712, and 1,344 workgroups of 64
+    # queries are too many to share keys
+    assert shape(1, 3072, 3072, 28, 256) == WIDE and shape(1, 3072, 3072, 28, 304) == NARROW
+    # 512 tokens after 3,584 cached: 112 groups, below one a unit: shared keys; with 12 such portions 1,344: wide
+    assert shape(1, 512, 4096, 28, 256) == SPLIT and shape(12, 512, 4096, 28, 256) == WIDE
+    # a short context (no workgroup walks 1,024 keys) keeps the plain shape
+    assert shape(1, 512, 512, 28, 256) == NARROW
+    # the tile kernel: 256 queries a workgroup from two groups a unit on
+    assert shape(1, 2048, 2048, 28, 256, tile=1) == TILE and shape(1, 8192, 8192, 28, 256, tile=1) == TILE_WIDE
+    assert shape(1, 8192, 8192, 28, 512, tile=1) == TILE

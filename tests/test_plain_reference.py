@@ -265,6 +265,12 @@ def test_model_is_causal_and_tied_head_uses_embedding():
     assert not torch.allclose(P.model_logits(cfg2, w2, ids), full)
 
 
+def test_logits_at_chosen_rows_are_the_rows_of_all_logits():
+    cfg, w = _tiny_weights(layers=2)
+    ids = [3, 1, 4, 1, 5, 9, 2, 6]
+    torch.testing.assert_close(P.model_logits(cfg, w, ids, rows=[7, 2]), P.model_logits(cfg, w, ids)[[7, 2]])
+
+
 def test_model_logits_do_not_depend_on_a_shift_of_positions():
     # only distances count: the same tokens at positions p.. and p+s.. give the same logits
     cfg, w = _tiny_weights(layers=2)
