@@ -656,6 +656,7 @@ extern "C" int somi_attention_prefill(const void* q, int64_t q_stride, const voi
     SOMI_REQUIRE(D % 16 == 0 && D >= 16 && D <= 256, "attention_prefill: head_dim %d must be a multiple of 16 up to 256", D);
     SOMI_REQUIRE(page_size > 0 && page_size % 4 == 0, "attention_prefill: page size %d must be a multiple of 4", page_size);
     SOMI_REQUIRE(window >= 0, "attention_prefill: window must be >= 0");
+    SOMI_REQUIRE(scale >= 0.f, "attention_prefill: the scale of the scores must not be negative, got %g", (double)scale);
     SOMI_REQUIRE(shape >= PREFILL_SHAPE_AUTO && shape <= PREFILL_SHAPE_TILE_WIDE, "attention_prefill: unknown launch shape %d", shape);
     SOMI_REQUIRE(n_entries <= 65535 && nq <= 65535, "attention_prefill: too many entries or heads");
     SOMI_REQUIRE(max_entry_len <= 65535 * 128, "attention_prefill: a portion of %d tokens is too long", max_entry_len);

@@ -20,8 +20,9 @@
 //     scores are then two runs of 8 consecutive keys, which is the B-operand layout of the second product, so the
 //     weights go from the first product to the second in registers, and a value fragment is one 16-byte read of
 //     the page's transposed values;
-//   * the scale and the change to base 2 go into the query fragments once; the running reference point enters
-//     the score product as its addend, so a score leaves the matrix core ready for exp2; the reference point
+//   * of the scale (times log2 e for base 2) the power of two goes into the query fragments once, exactly; the
+//     rest, a factor in [1, 2), multiplies the float32 scores on their way into exp2, so no score is computed from
+//     a rounded query; the running reference point enters the score product as its addend; the reference point
 //     follows the maximum lazily (only when a score passes it by more than 2^8), so outputs are rarely rescaled;
 //     the row sums come from one more matrix product with a fragment of ones;
 //   * measured on this part, LDS reads and matrix instructions of a compute unit do not overlap well: a step's
@@ -67,7 +68,7 @@ __global__ void __launch_bounds__(QBLK * KS * 64, 2)
 prefill_tile_kernel(const bf16* __restrict__ q, int64_t q_stride, const bf16* __restrict__ kc, const bf16* __restrict__ vc,
                     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ entry_start,
                     const int* __restrict__ entry_first_pos, const int* __restrict__ entry_len, int nq, int nkv,
-                    int page_size, int window, float scale_log2, bf16* __restrict__ out) {
+                    int page_size, int window, float scale_pow2, float scale_rest, bf16* __restrict__ out) {
     constexpr int THREADS = QBLK * KS * 64;
     constexpr int CH = D / 8;                    // 16-byte pieces of a key row
     constexpr int KROW = D * 2;                  // bytes
@@ -178,12 +179,16 @@ prefill_tile_kernel(const bf16* __restrict__ q, int64_t q_stride, const bf16* __
         const bf16* qrow = q + (int64_t)(start + qi) * q_stride + (int64_t)h * D;
 #pragma unroll
         for (int k = 0; k < KSTEPS; ++k) {
-            // the scale (and the change to base 2) goes into the query once: scores leave the product ready for exp2
+            // Of the scale (times log2 e, the change to base 2) only its power of two goes into the query, which
+            // bfloat16 takes without rounding; the rest, a factor in [1, 2), multiplies the float32 scores.  So the
+            // scores are those of the unscaled product, as in the kernels that scale after it.
             const bf16x8 raw = *reinterpret_cast<const bf16x8*>(qrow + k * 16 + hf * 8);
 #pragma unroll
-            for (int x = 0; x < 8; ++x) qf[k][x] = (bf16)((float)raw[x] * scale_log2);
+            for (int x = 0; x < 8; ++x) qf[k][x] = (bf16)((float)raw[x] * scale_pow2);
         }
     }
+    // Scores, m_run and neg_m are in units of the product of the power-of-two-scaled query: exp2 takes them times
+    // scale_rest.
     // m_run: what the weights are relative to (-inf: nothing seen yet); neg_m: its negative in every register, the
     // addend of the score product, so that scores arrive with the maximum already subtracted
     float m_run = -INFINITY;
@@ -257,10 +262,10 @@ prefill_tile_kernel(const bf16* __restrict__ q, int64_t q_stride, const bf16* __
             // weights may then exceed 1 (up to 2^TILE_LAZY), which float32 sums and bfloat16 weights hold as well, and
             // the sums and outputs are rescaled rarely.  A query's decision depends on its own scores only.
             const bool fresh = m_run == -INFINITY;
-            const bool move = fresh ? mx > -INFINITY : mx > TILE_LAZY;
+            const bool move = fresh ? mx > -INFINITY : mx * scale_rest > TILE_LAZY;
             if (__builtin_amdgcn_ballot_w64(move) != 0) {
                 const float delta = move ? mx : 0.f;      // how far the reference point moves up
-                const float corr = fresh ? 0.f : __builtin_amdgcn_exp2f(-delta);
+                const float corr = fresh ? 0.f : __builtin_amdgcn_exp2f(-delta * scale_rest);
                 m_run = move ? (fresh ? mx : m_run + mx) : m_run;
 #pragma unroll
                 for (int b = 0; b < DBLK; ++b)
@@ -276,7 +281,7 @@ prefill_tile_kernel(const bf16* __restrict__ q, int64_t q_stride, const bf16* __
             }
             float pr[16];
 #pragma unroll
-            for (int r = 0; r < 16; ++r) pr[r] = __builtin_amdgcn_exp2f(sc[r]);
+            for (int r = 0; r < 16; ++r) pr[r] = __builtin_amdgcn_exp2f(sc[r] * scale_rest);
             bf16x8 pf[2];
 #pragma unroll
             for (int t = 0; t < 2; ++t)
@@ -340,7 +345,8 @@ prefill_tile_kernel(const bf16* __restrict__ q, int64_t q_stride, const bf16* __
         const float m_other = hand[DBLK * 16 * 64], l_other = hand[(DBLK * 16 + 1) * 64];
         const float m_new = tile_max2(m_run, m_other);
         const float m_use = m_new == -INFINITY ? 0.f : m_new;
-        const float mine = __builtin_amdgcn_exp2f(m_run - m_use), theirs = __builtin_amdgcn_exp2f(m_other - m_use);
+        const float mine = __builtin_amdgcn_exp2f((m_run - m_use) * scale_rest);
+        const float theirs = __builtin_amdgcn_exp2f((m_other - m_use) * scale_rest);
         l_run = l_run * mine + l_other * theirs;
 #pragma unroll
         for (int b = 0; b < DBLK; ++b)
@@ -377,9 +383,13 @@ static int launch_tile(const void* q, int64_t q_stride, const void* kc, const vo
         lds_allowed[device] = lds;
     }
     const dim3 grid(nq, n_entries, ceil_div(max_entry_len, QBLK * 32));
+    // scale * log2(e) = 2^e * rest with rest in [1, 2)
+    int exponent = 0;
+    const float rest = 2.f * frexpf(scale * 1.44269504088896341f, &exponent);
+    const float pow2 = ldexpf(1.f, exponent - 1);
     hipLaunchKernelGGL((prefill_tile_kernel<D, QBLK, KS>), grid, dim3(QBLK * KS * 64), lds, stream, (const bf16*)q, q_stride,
                        (const bf16*)kc, (const bf16*)vc, block_table, max_blocks, entry_start, entry_first_pos, entry_len,
-                       nq, nkv, page_size, window, scale * 1.44269504088896341f, (bf16*)out);
+                       nq, nkv, page_size, window, pow2, rest, (bf16*)out);
     SOMI_LAUNCH_CHECK("attention_prefill_tile");
     return 0;
 }

@@ -19,6 +19,9 @@
 // Calls no hipMalloc, hipFree or other allocating routine.  Every call on a GPU uses that GPU's one array, which
 // keeps the last call's contents (each call writes every element it later reads, so nothing has to be cleared):
 // calls that overlap on one GPU (two streams, two threads) race; calls on one stream, or ordered by events, do not.
+// The first call on a GPU asks the runtime for the array's address on that GPU (hipGetSymbolAddress, which may load
+// the library's code for that GPU): make it outside stream capture.  Later calls on that GPU only launch the two
+// kernels on `stream` and may be captured into a graph.
 // Returns 0, or non-zero after storing a message for somi_last_error().
 extern "C" int somi_sample_no_alloc(const float* logits, int rows, int vocab, const float* temperature,
                                     const float* uniform, int* out, hipStream_t stream);

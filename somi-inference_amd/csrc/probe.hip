@@ -10,19 +10,24 @@ typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
 
-// Reads `pieces` 16-byte pieces once, every workgroup a contiguous share in steps of its 256 lanes, four loads in
-// flight a lane; the exclusive-or of everything read goes to out[blockIdx.x] so that no load can be dropped.
-__global__ void __launch_bounds__(256)
+// Reads `pieces` 16-byte pieces once, every workgroup a contiguous share in steps of its NT lanes, DEPTH loads in
+// flight a lane (NT: 256 or 512 lanes a workgroup; NONTEMPORAL: loads that tell the caches not to keep the line); the
+// exclusive-or of everything read goes to out[blockIdx.x] so that no load can be dropped.
+template <int NT, int DEPTH, bool NONTEMPORAL>
+__global__ void __launch_bounds__(NT)
 probe_stream_read_kernel(const u32x4* __restrict__ src, int64_t pieces, unsigned int* __restrict__ out) {
     const int64_t per_block = (pieces + gridDim.x - 1) / gridDim.x;
     const int64_t begin = per_block * blockIdx.x, end = begin + per_block < pieces ? begin + per_block : pieces;
     u32x4 acc = {0u, 0u, 0u, 0u};
     int64_t i = begin + threadIdx.x;
-    for (; i + 3 * 256 < end; i += 4 * 256) {
-        const u32x4 a = src[i], b = src[i + 256], c = src[i + 512], d = src[i + 768];
-        acc ^= a ^ b ^ c ^ d;
+    for (; i + (DEPTH - 1) * NT < end; i += DEPTH * NT) {
+        u32x4 v[DEPTH];
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d) v[d] = NONTEMPORAL ? __builtin_nontemporal_load(src + i + d * NT) : src[i + d * NT];
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d) acc ^= v[d];
     }
-    for (; i < end; i += 256) acc ^= src[i];
+    for (; i < end; i += NT) acc ^= src[i];
     unsigned int v = acc[0] ^ acc[1] ^ acc[2] ^ acc[3];
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) v ^= __shfl_xor(v, off, 64);
@@ -51,22 +56,51 @@ probe_mfma_kernel(int iters, float* __restrict__ out) {
     if (sum == -1.f) out[0] = sum;          // never true: the products stay
 }
 
-// Streams `bytes` (a multiple of 16, 16-byte aligned) from src once.  out: [blocks] words the caller zeroed,
-// blocks = somi_probe_stream_blocks().
-extern "C" int somi_probe_stream_blocks() {
-    int device = 0;
-    hipDeviceProp_t prop;
-    if (hipGetDevice(&device) != hipSuccess || hipGetDeviceProperties(&prop, device) != hipSuccess) return 2048;
-    return prop.multiProcessorCount * 8;
+// The launch shapes of the streaming read, so that the figure reported as the machine's own is the best of them and
+// not what one arbitrary kernel happens to reach.
+struct ProbeShape { const char* name; int threads, depth, nontemporal, blocks_per_unit; };
+static const ProbeShape probe_shapes[] = {
+    {"256 lanes x 4 loads, 8 workgroups a unit", 256, 4, 0, 8},
+    {"256 lanes x 8 loads, 8 workgroups a unit", 256, 8, 0, 8},
+    {"256 lanes x 16 loads, 4 workgroups a unit", 256, 16, 0, 4},
+    {"512 lanes x 8 loads, 4 workgroups a unit", 512, 8, 0, 4},
+    {"512 lanes x 8 loads, 2 workgroups a unit", 512, 8, 0, 2},
+    {"256 lanes x 8 loads, non-temporal, 8 workgroups a unit", 256, 8, 1, 8},
+    {"512 lanes x 16 loads, non-temporal, 4 workgroups a unit", 512, 16, 1, 4},
+};
+#define PROBE_SHAPES ((int)(sizeof(probe_shapes) / sizeof(probe_shapes[0])))
+
+extern "C" int somi_probe_stream_shapes() { return PROBE_SHAPES; }
+extern "C" const char* somi_probe_stream_shape_name(int shape) {
+    return shape >= 0 && shape < PROBE_SHAPES ? probe_shapes[shape].name : "";
 }
 
-extern "C" int somi_probe_stream_read(const void* src, int64_t bytes, unsigned int* out, hipStream_t stream) {
+// Workgroups of the streaming read in launch shape `shape`: what `out` must hold.
+extern "C" int somi_probe_stream_blocks(int shape) {
+    if (shape < 0 || shape >= PROBE_SHAPES) return 0;
+    return somi_units() * probe_shapes[shape].blocks_per_unit;
+}
+
+// Streams `bytes` (a multiple of 16, 16-byte aligned) from src once in launch shape `shape`.  out:
+// [somi_probe_stream_blocks(shape)] words the caller zeroed.
+extern "C" int somi_probe_stream_read(const void* src, int64_t bytes, int shape, unsigned int* out, hipStream_t stream) {
     SOMI_REQUIRE(src != nullptr && out != nullptr && bytes > 0 && bytes % 16 == 0 && (uintptr_t)src % 16 == 0,
                  "probe_stream_read: a 16-byte aligned buffer of a multiple of 16 bytes is needed");
-    hipLaunchKernelGGL(probe_stream_read_kernel, dim3(somi_probe_stream_blocks()), dim3(256), 0, stream,
-                       (const u32x4*)src, bytes / 16, out);
-    SOMI_LAUNCH_CHECK("probe_stream_read");
-    return 0;
+    SOMI_REQUIRE(shape >= 0 && shape < PROBE_SHAPES, "probe_stream_read: launch shape %d (0 to %d)", shape, PROBE_SHAPES - 1);
+    const ProbeShape& ps = probe_shapes[shape];
+    const dim3 grid(somi_probe_stream_blocks(shape)), block(ps.threads);
+    const u32x4* from = (const u32x4*)src;
+    const int64_t pieces = bytes / 16;
+#define SOMI_PROBE(NT, DEPTH, NTL)                                                                              \
+    if (ps.threads == NT && ps.depth == DEPTH && ps.nontemporal == NTL) {                                        \
+        hipLaunchKernelGGL((probe_stream_read_kernel<NT, DEPTH, NTL != 0>), grid, block, 0, stream, from, pieces, out); \
+        SOMI_LAUNCH_CHECK("probe_stream_read");                                                                  \
+        return 0;                                                                                                \
+    }
+    SOMI_PROBE(256, 4, 0) SOMI_PROBE(256, 8, 0) SOMI_PROBE(256, 16, 0) SOMI_PROBE(512, 8, 0)
+    SOMI_PROBE(256, 8, 1) SOMI_PROBE(512, 16, 1)
+#undef SOMI_PROBE
+    return somi_fail("probe_stream_read: launch shape %d has no kernel", shape);
 }
 
 // Runs the products on every compute unit (two wavefronts per SIMD); returns the number of flops through *flops.

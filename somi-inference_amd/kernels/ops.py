@@ -641,14 +641,23 @@ def sample_filter(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.
                                         _stream()))
 
 
-def probe_stream_read(buffer: torch.Tensor) -> None:
-    """Streams ``buffer`` (any dtype, contiguous, a multiple of 16 bytes) once through the compute units: the
-    time of this call is what reading that many bytes costs on this machine."""
+def probe_stream_shapes() -> list[str]:
+    """Names of the launch shapes of the streaming read (lanes a workgroup, loads in flight a lane, workgroups a
+    compute unit, cache hints): a measurement runs each and reports the best."""
+    lib = library()
+    lib.somi_probe_stream_shape_name.restype = ctypes.c_char_p
+    return [lib.somi_probe_stream_shape_name(i).decode() for i in range(lib.somi_probe_stream_shapes())]
+
+
+def probe_stream_read(buffer: torch.Tensor, shape: str | int = 0) -> None:
+    """Streams ``buffer`` (any dtype, contiguous, a multiple of 16 bytes) once through the compute units in the named
+    launch shape: the time of this call is what reading that many bytes costs on this machine."""
     _need(buffer, "probe buffer")
     size = buffer.numel() * buffer.element_size()
     lib = library()
-    sink = torch.zeros((lib.somi_probe_stream_blocks(),), dtype=torch.int32, device=buffer.device)
-    _check(lib.somi_probe_stream_read(_ptr(buffer), ctypes.c_int64(size), _ptr(sink), _stream()))
+    index = probe_stream_shapes().index(shape) if isinstance(shape, str) else int(shape)
+    sink = torch.zeros((max(1, lib.somi_probe_stream_blocks(index)),), dtype=torch.int32, device=buffer.device)
+    _check(lib.somi_probe_stream_read(_ptr(buffer), ctypes.c_int64(size), index, _ptr(sink), _stream()))
 
 
 def probe_mfma(iters: int, device: torch.device | str = "cuda:0") -> float:

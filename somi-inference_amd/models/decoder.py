@@ -10,6 +10,7 @@ from __future__ import annotations
 import torch
 
 from ..kernels import ops
+from ..kernels.stages import stage
 from ..parts.base import FixedStateSpec, LayerCache, PagedSpec, Runtime
 from ..parts.registry import build_part
 from ..parts.residual import ResidualStream
@@ -103,14 +104,39 @@ class DecoderModel:
         """Run the step's tokens; float32 logits ``[len(step.logit_rows), vocab]``."""
         if not self.loaded:
             raise RuntimeError("model weights are not loaded")
-        h = self.embedding.forward(step.token_ids)
-        if self.embedding_position is not None:
-            self.embedding_position.encode_embeddings(h, step)
+        with stage("embedding"):
+            h = self.embedding.forward(step.token_ids)
+            if self.embedding_position is not None:
+                self.embedding_position.encode_embeddings(h, step)
         stream = ResidualStream(h)
         for run, index in enumerate(self.order):
             self.layers[index].forward(stream, step, caches[run])
         h = stream.settle()
         if step.num_logit_rows == 0:
             return torch.empty((0, self.vocab_size), dtype=torch.float32, device=h.device)
-        rows = ops.gather_rows(h, step.logit_rows)
-        return self.head.forward(self.final_norm.forward(rows))
+        with stage("final norm"):
+            rows = self.final_norm.forward(ops.gather_rows(h, step.logit_rows))
+        with stage("head"):
+            return self.head.forward(rows)
+
+    # ------------------------------------------------------------- what a step costs
+    def step_flops(self, tokens: int, attended: int, logit_rows: int) -> float:
+        """Floating-point operations of the matrix products of a step of ``tokens`` tokens that see ``attended``
+        (token, key) pairs in all and want ``logit_rows`` logits: every run of every layer, and the head."""
+        return (sum(self.layers[index].flops(tokens, attended) for index in self.order)
+                + self.head.flops(logit_rows))
+
+    def step_weight_bytes(self) -> int:
+        """Bytes of the weights that a step reads whole, from what the parts declare: every tensor but the
+        embedding's, of which a step gathers one row a token (unless the head is tied to it and multiplies by it)."""
+        from ..weights.loader import device_dtype
+        gathered = set() if getattr(self.head, "tied", False) else {spec.name for spec in self.embedding.weight_specs()}
+        total = 0
+        for spec in self.weight_specs():
+            if spec.name in gathered:
+                continue
+            count = 1
+            for size in spec.shape:
+                count *= size
+            total += count * torch.empty((), dtype=device_dtype(spec.role, self.runtime.dtype)).element_size()
+        return total

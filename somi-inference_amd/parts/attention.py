@@ -17,6 +17,7 @@ import torch
 
 from ..kernels import attention as attention_kernels
 from ..kernels import ops
+from ..kernels.stages import stage
 from ..weights.spec import MATRIX, VECTOR, WeightSpec
 from .base import Fetch, LayerCache, Mixer, PagedKVSpec, PartSpec, Runtime
 from .linear import NormedRows, Projection
@@ -82,11 +83,17 @@ class GroupedQueryAttention(Mixer):
         names = [p for p, _ in self._projections()]
         self.qkv = Projection.stacked(
             [fetch(self.name(f"{p}.weight")) for p in names],
-            [fetch(self.name(f"{p}.bias")) for p in names] if self.qkv_bias else None)
+            [fetch(self.name(f"{p}.bias")) for p in names] if self.qkv_bias else None, label="q/k/v")
         out = self.names["o"]
         self.out = Projection(fetch(self.name(f"{out}.weight")),
-                              fetch(self.name(f"{out}.bias")) if self.out_bias else None)
+                              fetch(self.name(f"{out}.bias")) if self.out_bias else None, label="o")
         self.position.load(fetch, runtime)
+
+    def flops(self, tokens: int, attended: int) -> float:
+        """The projections, and q.k and p.v (two operations a product, head_dim channels, every query head) over the
+        (token, key) pairs the step's tokens see."""
+        return (self.qkv.flops(tokens) + self.out.flops(tokens)
+                + 4.0 * self.num_heads * self.head_dim * attended)
 
     # -------------------------------------------------------------------- cache
     def cache_spec(self) -> PagedKVSpec | None:
@@ -101,20 +108,23 @@ class GroupedQueryAttention(Mixer):
         view = step.paged[cache.group]
         nkv_new = 0 if self.shares_cache else self.num_kv_heads
         rotation = self.position.rotation_table()
-        qkv = self._project_rotate_store(x, step, view, cache, rotation)     # a few rows: one kernel
+        with stage(self.qkv.label):
+            qkv = self._project_rotate_store(x, step, view, cache, rotation)     # a few rows: one kernel
         if qkv is None:
             qkv = self.qkv(x)                               # [N, (nq + 2 nkv) * D]
-            if rotation is None:
-                self.position.encode_qk(qkv, step, self.num_heads, nkv_new, self.head_dim)
-                inv_freq, rotary_dim = None, 0
-            else:
-                inv_freq, rotary_dim = rotation
-            ops.rope_kv_store(qkv, step.positions, view.slot_mapping if nkv_new else None, inv_freq, rotary_dim,
-                              self.num_heads, nkv_new, self.head_dim,
-                              cache.k if nkv_new else None, cache.v if nkv_new else None)
-        attended = attention_kernels.paged_attention(
-            qkv, self.num_heads, cache.k, cache.v, view.block_table, step,
-            window=self.window or 0, scale=self.scale)
+            with stage("position encoding, k/v into pages"):
+                if rotation is None:
+                    self.position.encode_qk(qkv, step, self.num_heads, nkv_new, self.head_dim)
+                    inv_freq, rotary_dim = None, 0
+                else:
+                    inv_freq, rotary_dim = rotation
+                ops.rope_kv_store(qkv, step.positions, view.slot_mapping if nkv_new else None, inv_freq, rotary_dim,
+                                  self.num_heads, nkv_new, self.head_dim,
+                                  cache.k if nkv_new else None, cache.v if nkv_new else None)
+        with stage("attention"):
+            attended = attention_kernels.paged_attention(
+                qkv, self.num_heads, cache.k, cache.v, view.block_table, step,
+                window=self.window or 0, scale=self.scale)
         return self.out.deferred(attended)        # the residual stream may add it in the kernel that computes it
 
     def _project_rotate_store(self, x, step, view, cache: LayerCache, rotation) -> torch.Tensor | None:

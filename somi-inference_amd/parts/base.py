@@ -171,6 +171,12 @@ class Part:
     def load(self, fetch: Fetch, runtime: Runtime) -> None:
         self.runtime = runtime
 
+    def flops(self, tokens: int, attended: int) -> float:
+        """Floating-point operations of the part's matrix products in a step of ``tokens`` tokens that see
+        ``attended`` (token, key) pairs in all (a windowed mixer sees fewer: an upper bound then).  What a
+        measurement divides by the step's time; element-wise work is not counted."""
+        return 0.0
+
 
 class Norm(Part):
     def forward(self, h: torch.Tensor) -> torch.Tensor:
@@ -240,6 +246,9 @@ class Block(Part):
         self.runtime = runtime
         for part in self.parts():
             part.load(fetch, runtime)
+
+    def flops(self, tokens: int, attended: int) -> float:
+        return sum(part.flops(tokens, attended) for part in self.parts())
 
     def forward(self, stream: Any, step: Any, cache: LayerCache | None) -> None:
         raise NotImplementedError

@@ -58,5 +58,9 @@ class LMHead(Part):
     def tie(self, embedding: TokenEmbedding) -> None:
         self.weight = embedding.weight
 
+    def flops(self, tokens: int, attended: int = 0) -> float:
+        """Of the logits of ``tokens`` rows."""
+        return 2.0 * tokens * self.vocab_size * self.hidden_size
+
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         return linear_kernels.linear(x, self.weight, None, torch.float32)

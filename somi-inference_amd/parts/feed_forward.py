@@ -6,6 +6,7 @@ import torch
 
 from ..kernels import linear as linear_kernels
 from ..kernels import ops
+from ..kernels.stages import stage
 from ..weights.spec import MATRIX, WeightSpec
 from .base import FeedForward, Fetch, Runtime
 from .linear import NormedRows, Projection
@@ -56,20 +57,29 @@ class SwiGLU(FeedForward):
         if self.interleaved:
             b, h = self.INTERLEAVE, self.hidden_size
             merged = torch.stack([gate.view(-1, b, h), up.view(-1, b, h)], dim=1).reshape(-1, h).contiguous()
-            self.gate_up = Projection(merged)
+            self.gate_up = Projection(merged, label="gate_up")
         else:
-            self.gate_up = Projection.stacked([gate, up])
-        self.down = Projection(fetch(self.name(f"{self.names['down']}.weight")))
+            self.gate_up = Projection.stacked([gate, up], label="gate_up")
+        self.down = Projection(fetch(self.name(f"{self.names['down']}.weight")), label="down")
+
+    def flops(self, tokens: int, attended: int) -> float:
+        return self.gate_up.flops(tokens) + self.down.flops(tokens)
 
     def forward(self, x, step=None):
         if isinstance(x, NormedRows):
             if self.interleaved and self.gate_up.fusable(x.h.shape[0]):
                 # norm, gate_up and SiLU . up in one kernel
-                return self.down.deferred(linear_kernels.linear_scaled(x.weighted, x.norm.eps, x.stats,
-                                                                       self.gate_up.weight, swiglu=True))
+                with stage(self.gate_up.label):
+                    gated = linear_kernels.linear_scaled(x.weighted, x.norm.eps, x.stats, self.gate_up.weight, swiglu=True)
+                return self.down.deferred(gated)
             x = x.materialize()
         if not self.interleaved:
-            return self.down.deferred(ops.silu_mul(self.gate_up(x)))
+            projected = self.gate_up(x)
+            with stage("activation"):
+                return self.down.deferred(ops.silu_mul(projected))
         if x.data_ptr() % 16 == 0:
-            return self.down.deferred(linear_kernels.linear_swiglu(x, self.gate_up.weight))
-        return self.down.deferred(ops.silu_mul(self.gate_up(x), block=self.INTERLEAVE))
+            with stage(self.gate_up.label):
+                return self.down.deferred(linear_kernels.linear_swiglu(x, self.gate_up.weight))
+        projected = self.gate_up(x)
+        with stage("activation"):
+            return self.down.deferred(ops.silu_mul(projected, block=self.INTERLEAVE))

@@ -10,6 +10,7 @@ import torch
 
 from ..kernels import linear as linear_kernels
 from ..kernels import ops
+from ..kernels.stages import stage
 
 
 class NormedRows:
@@ -41,7 +42,8 @@ class DeferredProduct:
     def add_to(self, h: torch.Tensor, next_norm=None) -> "NormedRows | None":
         """h += the product, in place.  With the norm that follows, returns its rows, still to be normed."""
         weight = next_norm.weight if next_norm is not None else None
-        stats, weighted = linear_kernels.linear_residual(self.x, self.projection.weight, self.projection.bias, h, weight)
+        with stage(self.projection.label):
+            stats, weighted = linear_kernels.linear_residual(self.x, self.projection.weight, self.projection.bias, h, weight)
         return NormedRows(h, weighted, stats, next_norm) if next_norm is not None else None
 
 
@@ -49,25 +51,31 @@ class Projection:
     """``[out, in]`` weight (compute dtype) and optional float32 bias, fused from one or more
     checkpoint tensors that share their input (q/k/v, gate/up) by stacking their rows."""
 
-    def __init__(self, weight: torch.Tensor, bias: torch.Tensor | None = None) -> None:
+    def __init__(self, weight: torch.Tensor, bias: torch.Tensor | None = None, label: str = "projection") -> None:
         self.weight = weight
         self.bias = bias
+        self.label = label                 # the name of its stage where stages are timed
         self.out_features, self.in_features = weight.shape
 
+    def flops(self, rows: int) -> float:
+        return 2.0 * rows * self.out_features * self.in_features
+
     @classmethod
-    def stacked(cls, weights: list[torch.Tensor], biases: list[torch.Tensor] | None = None) -> "Projection":
+    def stacked(cls, weights: list[torch.Tensor], biases: list[torch.Tensor] | None = None,
+                label: str = "projection") -> "Projection":
         weight = weights[0] if len(weights) == 1 else torch.cat(weights, dim=0).contiguous()
         bias = None
         if biases:
             bias = biases[0] if len(biases) == 1 else torch.cat(biases, dim=0).contiguous()
-        return cls(weight, bias)
+        return cls(weight, bias, label)
 
     def __call__(self, x: "torch.Tensor | NormedRows", out_dtype: torch.dtype | None = None) -> torch.Tensor:
-        if isinstance(x, NormedRows):
-            if out_dtype in (None, torch.bfloat16) and self.fusable(x.h.shape[0]):
-                return linear_kernels.linear_scaled(x.weighted, x.norm.eps, x.stats, self.weight, self.bias)
-            x = x.materialize()
-        return linear_kernels.linear(x, self.weight, self.bias, out_dtype)
+        with stage(self.label):
+            if isinstance(x, NormedRows):
+                if out_dtype in (None, torch.bfloat16) and self.fusable(x.h.shape[0]):
+                    return linear_kernels.linear_scaled(x.weighted, x.norm.eps, x.stats, self.weight, self.bias)
+                x = x.materialize()
+            return linear_kernels.linear(x, self.weight, self.bias, out_dtype)
 
     def fusable(self, rows: int) -> bool:
         """The kernels that fuse this product with the norm before it or the residual add after it take it."""

@@ -11,6 +11,7 @@ from __future__ import annotations
 import torch
 
 from ..kernels import ops
+from ..kernels.stages import stage
 from .base import Norm
 from .linear import DeferredProduct, NormedRows
 
@@ -38,16 +39,18 @@ class ResidualStream:
             if lazy and getattr(norm, "fusable", False):
                 return pending.add_to(self.h, norm)
             pending.add_to(self.h)
-        if self._pending is not None:
-            delta, self._pending = self._pending, None
-            return norm.add_forward(self.h, delta)
-        return norm.forward(self.h)
+        with stage("residual add, norm"):
+            if self._pending is not None:
+                delta, self._pending = self._pending, None
+                return norm.add_forward(self.h, delta)
+            return norm.forward(self.h)
 
     def settle(self) -> torch.Tensor:
         """Apply a queued add and return the float32 rows."""
         if isinstance(self._pending, DeferredProduct):
             self._pending.add_to(self.h)
         elif self._pending is not None:
-            ops.residual_add(self.h, self._pending)
+            with stage("residual add, norm"):
+                ops.residual_add(self.h, self._pending)
         self._pending = None
         return self.h

@@ -15,6 +15,7 @@ from __future__ import annotations
 import torch
 
 from ..kernels import ops
+from ..kernels.stages import stage
 from .params import SamplingParams
 from .rng import uniform
 
@@ -108,6 +109,10 @@ class Sampler:
         if rows == 0:
             raise ValueError("nothing to sample")
 
+        with stage("sampling"):
+            return self._draw(logits, plist, histories, seeds, counters, rows)
+
+    def _draw(self, logits, plist, histories, seeds, counters, rows) -> PendingTokens:
         needs_copy = any(p.repetition_penalty != 1.0 and h for p, h in zip(plist, histories)) or any(
             p.temperature > 0.0 and (p.top_k != -1 or p.top_p != 1.0) for p in plist)
         work = logits.clone() if needs_copy else logits

@@ -863,6 +863,44 @@ def test_attention_prefill_tile_kernel_over_long_contexts(nq, nkv, d, page, wind
     torch.testing.assert_close(out.float(), want.float(), atol=2e-2, rtol=2e-2)
 
 
+@pytest.mark.parametrize("d", [64, 128])
+@pytest.mark.parametrize("shape", [1, 3, 4, 5, "decode"], ids=["narrow", "wide", "tile", "tile-wide", "decode"])
+def test_attention_scores_that_are_large_products_of_a_few_channels(d, shape):
+    """Queries and keys whose products sit in three channels of size nine: scores spread over +-100, so the softmax
+    sees every bit of them.  The scale belongs on the float32 scores (/root/reference/somi_inference/models/qwen2.py:
+    179, core/flash_attention_triton.py:113, 159): a kernel that rounds scale * q to bfloat16 before the product is
+    off by 6e-2 here, one that scales the float32 product by 1e-2 (the output's own rounding), against the dense
+    float32 softmax of the same bfloat16 inputs."""
+    n, nq, nkv, page = 300, 4, 1, 16
+    gen = torch.Generator().manual_seed(1)
+    q = torch.randn(n, nq, d, generator=gen) * 0.3
+    k = torch.randn(n, nkv, d, generator=gen) * 0.3
+    big = [3, d // 2 + 6, d - 27]
+    q[:, :, big] = torch.randn(n, nq, 3, generator=gen) * 9.0
+    k[:, :, big] = torch.randn(n, nkv, 3, generator=gen) * 9.0
+    v = torch.randn(n, nkv, d, generator=gen)
+    q, k, v = q.bfloat16(), k.bfloat16(), v.bfloat16()
+    scale = d ** -0.5
+    want = dense_attention_reference(q.float(), k.float(), v.float(), list(range(n)), 0, 0, scale)
+    assert float((torch.einsum("ihd,jhd->hij", q.float(), k.float().expand(n, nq, d)) * scale).abs().max()) > 60.0
+    pages = (n + page - 1) // page
+    table = torch.randperm(pages, generator=gen).tolist()
+    kc = torch.zeros(pages, nkv, page, d, dtype=torch.bfloat16, device=DEV)
+    vc = torch.zeros(pages, nkv, d, page, dtype=torch.bfloat16, device=DEV)
+    pos = torch.arange(n, device=DEV)
+    where = torch.tensor(table, device=DEV)[pos // page]
+    kc[where, :, pos % page] = k.to(DEV)
+    vc[where, :, :, pos % page] = v.to(DEV)
+    flat = q.reshape(n, nq * d).contiguous().to(DEV)
+    out = torch.full((n, nq * d), float("nan"), dtype=torch.bfloat16, device=DEV)
+    if shape == "decode":
+        ops.attention_decode(flat, nq * d, kc, vc, i32([table]), i32([0] * n), i32(list(range(n))), nq, 0, scale, 64, 5, out)
+    else:
+        ops.attention_prefill(flat, nq * d, kc, vc, i32([table]), i32([0, n]), i32([0]), n, nq, 0, scale, out, shape=shape)
+    error = (out.float().view(n, nq, d).cpu() - want).abs()
+    assert float(error.max()) < 2e-2, f"max error {float(error.max()):.3e}"
+
+
 @pytest.mark.parametrize("width, first", [(10_000, 150_000), (13_000, 200_000), (25_000, 390_000)])
 def test_attention_prefill_under_very_wide_block_tables(width, first):
     """Contexts of hundreds of thousands of tokens: block tables of 10,000 pages (the tile kernel with a long list
