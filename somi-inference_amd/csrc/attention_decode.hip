@@ -34,6 +34,17 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 
 __device__ __forceinline__ bf16x8 ld8(const bf16* p) { return *reinterpret_cast<const bf16x8*>(p); }
 __device__ __forceinline__ short4_t ld4(const bf16* p) { return *reinterpret_cast<const short4_t*>(p); }
+// The same for keys and values: a decode step reads each of them once, so the loads tell the caches not to keep the
+// lines (a streaming read measures 6.6 TB/s that way against 5.9 on an MI355X).
+typedef __attribute__((ext_vector_type(4))) unsigned int decode_u32x4;
+__device__ __forceinline__ bf16x8 ld8_once(const bf16* p) {
+    union { decode_u32x4 raw; bf16x8 values; } u;
+    u.raw = __builtin_nontemporal_load(reinterpret_cast<const decode_u32x4*>(p));
+    return u.values;
+}
+__device__ __forceinline__ short4_t ld4_once(const bf16* p) {
+    return __builtin_nontemporal_load(reinterpret_cast<const short4_t*>(p));
+}
 // Four elements in the lower half of an eight-wide operand, zeros above.
 __device__ __forceinline__ bf16x8 half_step(const bf16* p) {
     union { bf16x8 wide; short4_t half[2]; } u;
@@ -317,7 +328,7 @@ attention_decode_lds_kernel(const bf16* __restrict__ q, int64_t q_stride, const 
                 if (K_CHUNKS % 256 == 0 || c < K_CHUNKS) {
                     const int row = c / (D / 8), col = c % (D / 8);
                     const int pos = j0 + row;
-                    kreg[i] = ld8(k_head + page_of(pos) * page_stride + (page_offset(pos) * D + col * 8));
+                    kreg[i] = ld8_once(k_head + page_of(pos) * page_stride + (page_offset(pos) * D + col * 8));
                 }
             }
             const int kg = tid & 7;
@@ -327,7 +338,7 @@ attention_decode_lds_kernel(const bf16* __restrict__ q, int64_t q_stride, const 
 #pragma unroll
             for (int i = 0; i < V_PER_THREAD; ++i) {
                 const int d = (tid >> 3) + 32 * i;
-                if (D % 32 == 0 || d < D) vreg[i] = ld4(vbase + (int64_t)d * page_size);
+                if (D % 32 == 0 || d < D) vreg[i] = ld4_once(vbase + (int64_t)d * page_size);
             }
             if (vpos == vlo || vpos == vhi) {          // the groups that hold the first and the last visible key
 #pragma unroll

@@ -99,7 +99,9 @@ template <int N> __device__ __forceinline__ void big_wait_vmcnt() { asm volatile
 // tile are asked for before the finished tile is stored, so the stores and the first loads overlap.
 // BM: rows of a tile, 256 (two wavefronts along m) or 128 (one: for 65 to 128 rows, where a 256-row tile would
 // spend half of its products on rows that are not there).
-template <int BM, int BN, int S, int NW, int EPI, bool KTAIL>
+// WONCE: the weight is read once (one row tile: every weight tile has a single reader), so its loads tell the caches
+// not to keep the lines, as the few-rows products' weight streams do.
+template <int BM, int BN, int S, int NW, int EPI, bool KTAIL, bool WONCE>
 __global__ void __launch_bounds__(NW * 64, 1)
 linear_big_kernel(const BigArgs p) {
     extern __shared__ __attribute__((aligned(1024))) char lds[];
@@ -181,7 +183,8 @@ linear_big_kernel(const BigArgs p) {
             if ((kt_first + kt * splits) * BK + (is_b ? piece_b[i] : piece_a[i]) * 8 >= K) src = (const char*)big_zero_piece;
         }
         char* dst = lds + at + (wave * (is_b ? LB : LA) + i) * 1024;
-        __builtin_amdgcn_global_load_lds((const BIG_GLOBAL void*)src, (BIG_LDS void*)dst, 16, 0, 0);
+        if (WONCE && is_b) __builtin_amdgcn_global_load_lds((const BIG_GLOBAL void*)src, (BIG_LDS void*)dst, 16, 0, SOMI_LOAD_ONCE);
+        else __builtin_amdgcn_global_load_lds((const BIG_GLOBAL void*)src, (BIG_LDS void*)dst, 16, 0, 0);
     };
     auto issue_piece = [&](int q, int slot, int i) { issue(q & 1, q >> 1, slot * HB, i); };                 // wide ring
     auto issue_stage = [&](int kt, int buf, int i) {                                                       // narrow ring
@@ -640,15 +643,15 @@ static bool big_use_wide(int m, int n) {
 #define BIG_TILE_LOW 1
 static bool big_use_low(int m, int tile) { return tile == BIG_TILE_LOW || (tile == 0 && m <= 128); }
 
-template <int BM, int BN, int S, int NW, int EPI, bool KTAIL>
-static int big_launch_one(const BigArgs& args, hipStream_t stream) {
+template <int BM, int BN, int S, int NW, int EPI, bool KTAIL, bool WONCE>
+static int big_launch_once(const BigArgs& args, hipStream_t stream) {
     const int lds_bytes = S == 5 ? 5 * 256 * BIG_ROW_BYTES : S * (BM + BN) * BIG_ROW_BYTES;
     static bool raised[64];
     int device = 0;
     hipError_t err = hipGetDevice(&device);
     if (err != hipSuccess || device < 0 || device >= 64) return somi_fail("linear_big: hipGetDevice failed");
     if (!raised[device]) {
-        err = hipFuncSetAttribute((const void*)linear_big_kernel<BM, BN, S, NW, EPI, KTAIL>,
+        err = hipFuncSetAttribute((const void*)linear_big_kernel<BM, BN, S, NW, EPI, KTAIL, WONCE>,
                                   hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
         if (err != hipSuccess) return somi_fail("linear_big: %d bytes of LDS refused: %s", lds_bytes, hipGetErrorString(err));
         raised[device] = true;
@@ -661,7 +664,7 @@ static int big_launch_one(const BigArgs& args, hipStream_t stream) {
         const int cus_per_die = big_compute_units() / 8 > 0 ? big_compute_units() / 8 : 1;
         per_die = per < cus_per_die ? per : cus_per_die;
     }
-    hipLaunchKernelGGL((linear_big_kernel<BM, BN, S, NW, EPI, KTAIL>), dim3(per_die * 8), dim3(NW * 64), lds_bytes, stream, args);
+    hipLaunchKernelGGL((linear_big_kernel<BM, BN, S, NW, EPI, KTAIL, WONCE>), dim3(per_die * 8), dim3(NW * 64), lds_bytes, stream, args);
     SOMI_LAUNCH_CHECK("linear_big");
     if (EPI == BIG_RESIDUAL && args.partial != nullptr) {
         if (args.reduce_plain)
@@ -670,6 +673,14 @@ static int big_launch_one(const BigArgs& args, hipStream_t stream) {
             hipLaunchKernelGGL(big_split_reduce_kernel, dim3(args.stats_rows, ceil_div(args.M, 16)), dim3(256), 0, stream, args);
         SOMI_LAUNCH_CHECK("linear_big: reduce");
     }
+    return 0;
+}
+
+// A weight that one row tile reads is read once: its loads carry the hint (the 128-row tile is only ever used so).
+template <int BM, int BN, int S, int NW, int EPI, bool KTAIL>
+static int big_launch_one(const BigArgs& args, hipStream_t stream) {
+    if (BM == 128 || args.tiles_m == 1) return big_launch_once<BM, BN, S, NW, EPI, KTAIL, true>(args, stream);
+    if constexpr (BM != 128) return big_launch_once<BM, BN, S, NW, EPI, KTAIL, false>(args, stream);
     return 0;
 }
 

@@ -107,8 +107,9 @@ linear_fused_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, cons
         const bool inside = !TAIL || k0 + lchunk * 8 < K;
 #pragma unroll
         for (int i = 0; i < NL; ++i)
-            st[i] = __builtin_amdgcn_raw_buffer_load_b128(
-                i < NS * 2 ? wres : xres, inside ? goff[i] + (unsigned)k0 * 2u : SOMI_OUT_OF_RANGE, 0, 0);
+            st[i] = i < NS * 2
+                        ? __builtin_amdgcn_raw_buffer_load_b128(wres, inside ? goff[i] + (unsigned)k0 * 2u : SOMI_OUT_OF_RANGE, 0, SOMI_LOAD_ONCE)
+                        : __builtin_amdgcn_raw_buffer_load_b128(xres, inside ? goff[i] + (unsigned)k0 * 2u : SOMI_OUT_OF_RANGE, 0, 0);
     };
     auto stash = [&](const u32x4 (&st)[NL]) {
 #pragma unroll

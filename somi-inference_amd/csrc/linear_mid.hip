@@ -300,7 +300,7 @@ linear_mid_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, const 
 #pragma unroll
         for (int i = 0; i < WLD; ++i)
             st.wv[i] = __builtin_amdgcn_raw_buffer_load_b128(
-                wres, inside ? wgoff[i] + (unsigned)k0 * 2u : SOMI_OUT_OF_RANGE, 0, 0);
+                wres, inside ? wgoff[i] + (unsigned)k0 * 2u : SOMI_OUT_OF_RANGE, 0, SOMI_LOAD_ONCE);
 #pragma unroll
         for (int j = 0; j < XL; ++j)
             st.xv[j] = __builtin_amdgcn_raw_buffer_load_b128(

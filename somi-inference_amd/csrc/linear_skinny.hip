@@ -84,7 +84,8 @@ linear_skinny_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, con
 #pragma unroll
         for (int i = 0; i < NL; ++i) {
             const unsigned off = inside ? goff[i] + (unsigned)k0 * 2u : SOMI_OUT_OF_RANGE;
-            st[i] = __builtin_amdgcn_raw_buffer_load_b128(i < NS * WL ? wres : xres, off, 0, 0);
+            st[i] = i < NS * WL ? __builtin_amdgcn_raw_buffer_load_b128(wres, off, 0, SOMI_LOAD_ONCE)
+                                : __builtin_amdgcn_raw_buffer_load_b128(xres, off, 0, 0);
         }
     };
     auto stash = [&](const u32x4 (&st)[NL]) {

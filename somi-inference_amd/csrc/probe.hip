@@ -34,6 +34,33 @@ probe_stream_read_kernel(const u32x4* __restrict__ src, int64_t pieces, unsigned
     if ((threadIdx.x & 63) == 0) atomicXor(out + blockIdx.x, v);
 }
 
+// The same through buffer loads (the weight streams of the few-rows products are buffer loads) with the cache policy
+// bits AUX of the instruction: 0 none, 1 sc0, 2 nt (non-temporal), 16 sc1, and their sums.
+template <int AUX>
+__global__ void __launch_bounds__(256)
+probe_stream_buffer_kernel(const u32x4* __restrict__ src, int64_t pieces, unsigned int* __restrict__ out) {
+    constexpr int NT = 256, DEPTH = 8;
+    const int64_t per_block = (pieces + gridDim.x - 1) / gridDim.x;
+    const int64_t begin = per_block * blockIdx.x, end = begin + per_block < pieces ? begin + per_block : pieces;
+    // a workgroup's share is below 2 GiB: one buffer descriptor covers it
+    const __amdgpu_buffer_rsrc_t res = __builtin_amdgcn_make_buffer_rsrc((void*)(src + begin), 0, (int)((end - begin) * 16), 0x00020000u);
+    u32x4 acc = {0u, 0u, 0u, 0u};
+    const int64_t count = end - begin;
+    int64_t i = threadIdx.x;
+    for (; i + (DEPTH - 1) * NT < count; i += DEPTH * NT) {
+        u32x4 v[DEPTH];
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d) v[d] = __builtin_amdgcn_raw_buffer_load_b128(res, (unsigned)((i + d * NT) * 16), 0, AUX);
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d) acc ^= v[d];
+    }
+    for (; i < count; i += NT) acc ^= __builtin_amdgcn_raw_buffer_load_b128(res, (unsigned)(i * 16), 0, AUX);
+    unsigned int v = acc[0] ^ acc[1] ^ acc[2] ^ acc[3];
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v ^= __shfl_xor(v, off, 64);
+    if ((threadIdx.x & 63) == 0) atomicXor(out + blockIdx.x, v);
+}
+
 // Every wavefront multiplies `iters` times four independent 32 x 32 x 16 bfloat16 products (32,768 flops each).
 __global__ void __launch_bounds__(512)
 probe_mfma_kernel(int iters, float* __restrict__ out) {
@@ -67,6 +94,14 @@ static const ProbeShape probe_shapes[] = {
     {"512 lanes x 8 loads, 2 workgroups a unit", 512, 8, 0, 2},
     {"256 lanes x 8 loads, non-temporal, 8 workgroups a unit", 256, 8, 1, 8},
     {"512 lanes x 16 loads, non-temporal, 4 workgroups a unit", 512, 16, 1, 4},
+    // buffer loads of 256 lanes x 8, 8 workgroups a unit; `nontemporal` holds 100 + the cache policy bits
+    {"buffer loads, no policy bits", 256, 8, 100, 8},
+    {"buffer loads, sc0", 256, 8, 101, 8},
+    {"buffer loads, nt", 256, 8, 102, 8},
+    {"buffer loads, sc0 nt", 256, 8, 103, 8},
+    {"buffer loads, sc1", 256, 8, 116, 8},
+    {"buffer loads, sc1 nt", 256, 8, 118, 8},
+    {"buffer loads, sc0 sc1 nt", 256, 8, 119, 8},
 };
 #define PROBE_SHAPES ((int)(sizeof(probe_shapes) / sizeof(probe_shapes[0])))
 
@@ -100,6 +135,16 @@ extern "C" int somi_probe_stream_read(const void* src, int64_t bytes, int shape,
     SOMI_PROBE(256, 4, 0) SOMI_PROBE(256, 8, 0) SOMI_PROBE(256, 16, 0) SOMI_PROBE(512, 8, 0)
     SOMI_PROBE(256, 8, 1) SOMI_PROBE(512, 16, 1)
 #undef SOMI_PROBE
+#define SOMI_PROBE_BUFFER(AUX)                                                                                   \
+    if (ps.nontemporal == 100 + AUX) {                                                                           \
+        SOMI_REQUIRE(bytes / grid.x < ((int64_t)1 << 31), "probe_stream_read: too many bytes a workgroup for a buffer descriptor"); \
+        hipLaunchKernelGGL((probe_stream_buffer_kernel<AUX>), grid, block, 0, stream, from, pieces, out);        \
+        SOMI_LAUNCH_CHECK("probe_stream_read");                                                                  \
+        return 0;                                                                                                \
+    }
+    SOMI_PROBE_BUFFER(0) SOMI_PROBE_BUFFER(1) SOMI_PROBE_BUFFER(2) SOMI_PROBE_BUFFER(3) SOMI_PROBE_BUFFER(16)
+    SOMI_PROBE_BUFFER(18) SOMI_PROBE_BUFFER(19)
+#undef SOMI_PROBE_BUFFER
     return somi_fail("probe_stream_read: launch shape %d has no kernel", shape);
 }
 
