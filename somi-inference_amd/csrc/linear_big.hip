@@ -83,7 +83,21 @@ struct BigArgs {
                                       // (the splits of a tile run side by side and so read neighbouring lines of a row)
     int stats_rows;                   // rows of stats_out (one per 64 columns of the tiles)
     int reduce_plain;                 // the splits' sums end as the plain form does: out = s * sum + bias in bfloat16
+    // Streamed: the (tile, stage) units of the whole product, tiles in launch order, stages within a tile, are dealt
+    // out to `stream_wgs` workgroups in equal contiguous ranges, so any number of tiles keeps every compute unit busy
+    // to the end.  A range may begin or end inside a tile: such a segment leaves its sums in one of the workgroup's
+    // two slots ([stream_wgs][2][BM x BN] float32: 0 for a segment that begins the range, 1 for one that ends it)
+    // and big_stream_finish_kernel adds a tile's segments in stage order and does what the epilogue would have done.
+    int stream_wgs;                   // 0: not streamed
+    float* slots;
 };
+
+// silu(gate) * up = gate * up / (1 + e^-gate) with the hardware's base-2 exponential and reciprocal (each within
+// one unit in the last place of float32; the result is rounded to bfloat16): nine instructions a value where expf and
+// a float32 division take twenty-five, which a 2,048-row gate_up product feels (its end is 38.8 million values).
+__device__ __forceinline__ float big_silu_mul(float gate, float up) {
+    return gate * up * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(-1.44269504088896341f * gate));
+}
 
 template <int N> __device__ __forceinline__ void big_wait_vmcnt() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
 
@@ -125,8 +139,10 @@ linear_big_kernel(const BigArgs p) {
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave / WAVES_N, wn = wave % WAVES_N;
     const int M = p.M, N = p.N, K = p.K;
-    const int splits = HALF ? 1 : p.splits;                      // workgroups that share a tile's K
-    int KT = (K + BK - 1) / BK;                                   // stages this workgroup walks: kt_first, kt_first + splits, ...
+    const bool streamed = p.stream_wgs > 0;
+    const int splits = HALF || streamed ? 1 : p.splits;          // workgroups that share a tile's K
+    const int KTF = (K + BK - 1) / BK;                            // stages of a whole tile
+    int KT = KTF;                                                 // stages this workgroup walks: kt_first, kt_first + splits, ...
     int kt_first = 0;
     const int64_t stage_bytes = (int64_t)ROW_BYTES * splits;      // from one of its stages to the next
     const int lrow = lane >> 3, lpos = lane & 7;
@@ -139,7 +155,16 @@ linear_big_kernel(const BigArgs p) {
     const int die_first = (blockIdx.x & 7) * per, die_end = die_first + per < total ? die_first + per : total;
     const int stride = HALF ? (int)(gridDim.x >> 3) : per;
     int logical = die_first + (blockIdx.x >> 3);
-    if (logical >= die_end) return;
+    // streamed: the workgroups of a die hold neighbouring ranges of units (neighbouring tiles: what they share of
+    // the operands meets in the die's L2); position pos owns the units [pos U / W, (pos + 1) U / W)
+    const int pos = (blockIdx.x & 7) * (int)(gridDim.x >> 3) + (int)(blockIdx.x >> 3);
+    int64_t unit = 0, unit_end = 0, unit_first = 0;
+    if (streamed) {
+        const int64_t units = (int64_t)p.tiles_m * p.tiles_n * KTF;
+        unit_first = unit = units * pos / p.stream_wgs;
+        unit_end = units * (pos + 1) / p.stream_wgs;
+        if (unit >= unit_end) return;
+    } else if (logical >= die_end) return;
 
     // ------------------------------------------------------------------ loads: global -> LDS
     // An instruction covers 8 rows of 128 bytes; lane l writes LDS position l % 8 of row l / 8 and reads the
@@ -151,15 +176,23 @@ linear_big_kernel(const BigArgs p) {
     for (int i = 0; i < LA; ++i) piece_a[i] = lpos ^ ((((wave * LA + i) * 8 + lrow) >> 1) & 7);
 #pragma unroll
     for (int i = 0; i < LB; ++i) piece_b[i] = lpos ^ ((((wave * LB + i) * 8 + lrow) >> 1) & 7);
-    auto aim = [&](int item) {                 // point the loads at a tile (and, with K split, at this split's stages)
-        const int tile = item / splits;
+    // point the loads at a tile (and, with K split, at this split's stages; streamed: at the stages of the segment
+    // that begins at unit `item`)
+    auto aim = [&](int64_t item) {
+        const int tile = streamed ? (int)(item / KTF) : (int)item / splits;
         const int tn = tile / p.tiles_m, tm = tile % p.tiles_m;
         const int mlim = M - tm * BM, nlim = N - tn * BN;
         xa = (const char*)(p.x + (int64_t)tm * BM * p.ldx);
         wb = (const char*)(p.w + (int64_t)tn * BN * p.ldw);
-        if (!HALF && splits > 1) {
-            kt_first = item % splits;
-            KT = ((K + BK - 1) / BK - kt_first + splits - 1) / splits;
+        if (streamed) {
+            kt_first = (int)(item % KTF);
+            const int64_t left = unit_end - item;
+            KT = left < KTF - kt_first ? (int)left : KTF - kt_first;
+            xa += (int64_t)kt_first * ROW_BYTES;
+            wb += (int64_t)kt_first * ROW_BYTES;
+        } else if (!HALF && splits > 1) {
+            kt_first = (int)item % splits;
+            KT = (KTF - kt_first + splits - 1) / splits;
             xa += (int64_t)kt_first * ROW_BYTES;
             wb += (int64_t)kt_first * ROW_BYTES;
         }
@@ -214,7 +247,7 @@ linear_big_kernel(const BigArgs p) {
     };
 
     // the first tile's first pieces
-    aim(logical);
+    aim(streamed ? unit : (int64_t)logical);
     if (HALF) {
 #pragma unroll
         for (int q = 0; q < 5; ++q)
@@ -228,11 +261,15 @@ linear_big_kernel(const BigArgs p) {
     }
 
     while (true) {
-        const int tile = logical / splits;
+        const int tile = streamed ? (int)(unit / KTF) : logical / splits;
         const int tn = tile / p.tiles_m, tm = tile % p.tiles_m;
         const int m0 = tm * BM, n0 = tn * BN;
         const int next = logical + stride;
-        const bool has_next = HALF && next < die_end;
+        // streamed: the segment [unit, unit + KT) of this tile; one that is not the tile's whole K goes to a slot
+        const int64_t next_unit = unit + KT;
+        const bool whole = !streamed || KT == KTF;
+        float* const slot = streamed ? p.slots + ((int64_t)pos * 2 + (unit == unit_first ? 0 : 1)) * (BM * BN) : nullptr;
+        const bool has_next = streamed ? next_unit < unit_end : HALF && next < die_end;
 
         f32x16 acc[WTM][WTN];
 #pragma unroll
@@ -361,9 +398,9 @@ linear_big_kernel(const BigArgs p) {
                     }
             }
         }
-        if (has_next) {
+        if (HALF && has_next) {
             // the next tile's pieces A0 B0 A1 go out now, into the slots the stores below do not use
-            aim(next);
+            aim(streamed ? next_unit : (int64_t)next);
 #pragma unroll
             for (int q = 0; q < 3; ++q)
 #pragma unroll
@@ -376,7 +413,31 @@ linear_big_kernel(const BigArgs p) {
         // into whole rows and stores 16 bytes a lane.
         char* stg = lds + STG + wave * STG_WAVE;
 
-        if (EPI == BIG_PLAIN || EPI == BIG_SWIGLU) {
+        if (!whole) {
+            // a segment of the tile's K: the sums as they are, whole rows of the tile-local slot
+            constexpr int SROW = 32 * 4 + 16;
+#pragma unroll
+            for (int i = 0; i < WTM; ++i) {
+#pragma unroll
+                for (int j = 0; j < WTN; ++j) {
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                        const f32x16& t = acc[i][j];
+                        f32x4 v = {t[4 * g], t[4 * g + 1], t[4 * g + 2], t[4 * g + 3]};
+                        *(f32x4*)(stg + ml * SROW + (8 * g + 4 * nh) * 4) = v;
+                    }
+                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+                    for (int pass = 0; pass < 4; ++pass) {
+                        const int row = pass * 8 + (lane >> 3), piece = lane & 7;
+                        const f32x4 v = *(const f32x4*)(stg + row * SROW + piece * 16);
+                        const int rt = wm * 128 + i * 32 + row, ct = wn * (BN / WAVES_N) + j * 32 + piece * 4;
+                        *(f32x4*)(slot + rt * BN + ct) = v;
+                    }
+                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                }
+            }
+        } else if (EPI == BIG_PLAIN || EPI == BIG_SWIGLU) {
             constexpr int CW = EPI == BIG_SWIGLU ? WTN * 16 : WTN * 32;      // output columns of the wavefront per row
             constexpr int SROW = CW * 2 + 8;                                   // staged row: 8 bytes of padding spread the banks
             constexpr int LPR = CW * 2 / 16;                                   // lanes per row when reading back
@@ -397,7 +458,7 @@ linear_big_kernel(const BigArgs p) {
 #pragma unroll
                             for (int c = 0; c < 4; ++c) {
                                 const float gate = s * t[4 * g + c], up = s * t[4 * g + c + 8];
-                                v[c] = (bf16)(gate / (1.f + expf(-gate)) * up);
+                                v[c] = (bf16)big_silu_mul(gate, up);
                             }
                             *(bf16x4*)(stg + ml * SROW + (j * 16 + 8 * g + 4 * nh) * 2) = v;
                         }
@@ -507,13 +568,24 @@ linear_big_kernel(const BigArgs p) {
         }
 
         if (!has_next) break;
-        // the staging is read: slots 3 and 4 take the next tile's B1 and A2
+        // the staging is read
         __syncthreads();
+        if constexpr (HALF) {
+            // slots 3 and 4 take the next tile's B1 and A2
 #pragma unroll
-        for (int q = 3; q < 5; ++q)
+            for (int q = 3; q < 5; ++q)
 #pragma unroll
-            for (int i = 0; i < LA; ++i) issue_piece(q, q, i);
+                for (int i = 0; i < LA; ++i) issue_piece(q, q, i);
+        } else {
+            // (streamed) the next segment from its first stages on
+            aim(next_unit);
+#pragma unroll
+            for (int st = 0; st < S - 1; ++st)
+#pragma unroll
+                for (int i = 0; i < L; ++i) issue_stage(st, st, i);
+        }
         logical = next;
+        unit = next_unit;
     }
 }
 
@@ -625,14 +697,146 @@ big_split_reduce_plain_kernel(const BigArgs p) {
     }
 }
 
+// The end of a streamed product for the tiles whose K more than one workgroup walked.  The boundary between the
+// ranges of workgroup b - 1 and workgroup b (blockIdx.x = b - 1) that lies inside a tile, and is the first to do so,
+// stands for that tile: a workgroup takes 16 of the tile's rows (blockIdx.y), adds the tile's segments in stage
+// order (the slots of the workgroups b - 1, b, ... while their ranges begin inside the tile) and ends as the form's
+// epilogue does: plain (row scale, bias, bfloat16), gated, or into the stream / float32 with the next norm's rows and
+// the sums of squares (one row of the statistics per 64 columns, as the epilogue lays them out).
+template <int BM, int BN>
+__global__ void __launch_bounds__(256)
+big_stream_finish_kernel(const BigArgs p, int epi) {
+    const int W = p.stream_wgs, M = p.M, N = p.N;
+    const int KTF = (p.K + BIG_BK - 1) / BIG_BK;
+    const int64_t units = (int64_t)p.tiles_m * p.tiles_n * KTF;
+    const int b = blockIdx.x + 1;
+    const int64_t at = units * b / W;
+    if (at % KTF == 0) return;                                    // the ranges meet between two tiles
+    const int tile = (int)(at / KTF);
+    const int64_t tile_first = (int64_t)tile * KTF, tile_end = tile_first + KTF;
+    if (units * (b - 1) / W > tile_first) return;                 // an earlier boundary stands for this tile
+    const int tn = tile / p.tiles_m, tm = tile % p.tiles_m;
+    const int row = threadIdx.x >> 4, cg = threadIdx.x & 15;
+    const int rt = blockIdx.y * 16 + row, gm = tm * BM + rt;
+    constexpr int QUADS = BN / 64;                                // quads of columns a thread takes: 64 columns apart
+    f32x4 sum[QUADS];
+#pragma unroll
+    for (int q = 0; q < QUADS; ++q) sum[q] = f32x4{0.f, 0.f, 0.f, 0.f};
+    // In the gated form a thread needs the gate and the up value of a channel: quad q of thread cg is then the
+    // quad (q * 16 + cg) of the row's BN / 8 (gate quad, up quad) pairs instead of the columns 64 q + 4 cg.
+    auto column = [&](int q) { return epi == BIG_SWIGLU ? ((q * 16 + cg) >> 2) * 32 + ((q * 16 + cg) & 3) * 4 : q * 64 + cg * 4; };
+    f32x4 up[QUADS];
+#pragma unroll
+    for (int q = 0; q < QUADS; ++q) up[q] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int w = b - 1; w < W; ++w) {
+        const int64_t first = units * w / W, end = units * (w + 1) / W;
+        if (first >= tile_end) break;
+        if (first >= end) continue;                               // a workgroup without units left nothing
+        const float* slot = p.slots + ((int64_t)w * 2 + (first < tile_first ? 1 : 0)) * (BM * BN) + rt * BN;
+#pragma unroll
+        for (int q = 0; q < QUADS; ++q) {
+            if (epi == BIG_SWIGLU && q >= QUADS / 2) break;
+            const int c = column(q);
+            sum[q] += *(const f32x4*)(slot + c);
+            if (epi == BIG_SWIGLU) up[q] += *(const f32x4*)(slot + c + 16);
+        }
+    }
+    if (epi == BIG_PLAIN || epi == BIG_SWIGLU) {
+        if (gm >= M) return;
+        const float scale = p.row_scale != nullptr ? p.row_scale[gm] : 1.f;
+        const int out_n = epi == BIG_SWIGLU ? N / 2 : N;
+        const bool aligned = (out_n & 3) == 0 && ((uintptr_t)p.out & 7) == 0;
+#pragma unroll
+        for (int q = 0; q < QUADS; ++q) {
+            if (epi == BIG_SWIGLU && q >= QUADS / 2) break;
+            const int c = column(q);
+            const int gn = tn * BN + c;                           // first of the four columns of the product
+            if (gn >= N) continue;
+            bf16x4 v;
+            int gc;                                               // first output column
+            if (epi == BIG_SWIGLU) {
+                gc = (tn * BN + (c >> 5) * 32) / 2 + (c & 15);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const float gate = scale * sum[q][e], u = scale * up[q][e];
+                    v[e] = (bf16)big_silu_mul(gate, u);
+                }
+            } else {
+                gc = gn;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] = (bf16)(scale * sum[q][e] + (p.bias != nullptr && gn + e < N ? p.bias[gn + e] : 0.f));
+            }
+            bf16* dst = p.out + (int64_t)gm * out_n + gc;
+            if (aligned && gc + 4 <= out_n) *(bf16x4*)dst = v;
+            else
+                for (int e = 0; e < 4; ++e)
+                    if (gc + e < out_n) dst[e] = v[e];
+        }
+        return;
+    }
+    // into the stream (or float32 results as they are)
+    const bool aligned = (N & 3) == 0 && ((uintptr_t)p.h & 15) == 0 && (p.weighted == nullptr || ((uintptr_t)p.weighted & 7) == 0);
+#pragma unroll
+    for (int q = 0; q < QUADS; ++q) {
+        const int gn = tn * BN + q * 64 + cg * 4;
+        float sq = 0.f;
+        if (gm < M && gn < N) {
+            float* hp = p.h + (int64_t)gm * N + gn;
+            if (aligned && gn + 4 <= N) {
+                f32x4 hv = p.overwrite ? f32x4{0.f, 0.f, 0.f, 0.f} : *(const f32x4*)hp;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    hv[e] += sum[q][e] + (p.bias != nullptr ? p.bias[gn + e] : 0.f);
+                    sq += hv[e] * hv[e];
+                }
+                *(f32x4*)hp = hv;
+                if (p.weighted != nullptr) {
+                    bf16x4 wv;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) wv[e] = (bf16)(p.norm_w[gn + e] * hv[e]);
+                    *(bf16x4*)(p.weighted + (int64_t)gm * N + gn) = wv;
+                }
+            } else {
+                for (int e = 0; e < 4; ++e)
+                    if (gn + e < N) {
+                        const float hv = (p.overwrite ? 0.f : hp[e]) + sum[q][e] + (p.bias != nullptr ? p.bias[gn + e] : 0.f);
+                        hp[e] = hv;
+                        sq += hv * hv;
+                        if (p.weighted != nullptr) p.weighted[(int64_t)gm * N + gn + e] = (bf16)(p.norm_w[gn + e] * hv);
+                    }
+            }
+        }
+        if (p.stats_out != nullptr) {
+            // the 16 lanes of a row add their squares in a fixed order; every lane takes part
+#pragma unroll
+            for (int off = 8; off > 0; off >>= 1) sq += __shfl_xor(sq, off, 64);
+            if (cg == 0 && gm < M) p.stats_out[(int64_t)(tn * QUADS + q) * p.stats_width + gm] = sq;
+        }
+    }
+}
+
 // ---------------------------------------------------------------------- host side
 static int big_compute_units() { return somi_units(); }
+
+// Streaming (BigArgs.stream_wgs) is there for the asking (tile code + BIG_TILE_STREAM) and is never chosen: measured at
+// 7B layer sizes on an MI355X it loses to whole tiles, or to tiles that share their K in turns, at every number of
+// rows.  With equal contiguous ranges of units the workgroups of a die no longer walk the row tiles of a column tile
+// in step, so a weight tile is no longer read from memory once and from the L2 seven times (2,048 rows: q/k/v 110 us
+// against 83, down 343 against 243, gate_up 629 against 494, the slots' traffic included); with one row tile, where
+// nothing is shared, a stage of a workgroup takes as long as its loads' latency, and twice the workgroups wait
+// twice as long (gate_up at 256 rows: 110 us against 104).
+#define BIG_STREAM_MIN_STAGES 1          // stages a workgroup gets at least where streaming is asked for
+static bool big_streams(int tiles, int k, int cus) {
+    (void)tiles; (void)k; (void)cus;
+    return false;
+}
 
 // The wide tile moves fewer bytes per product and wins where it fills the device; the narrow one has twice the
 // workgroups.  Costs in units of a narrow tile's time: rounds of tiles x the tile's size (the narrow tile is
 // about 8 % less efficient per product).
-static bool big_use_wide(int m, int n) {
-    const int cus = big_compute_units();
+static bool big_use_wide(int m, int n, int k, int cus = 0) {
+    (void)k;
+    if (cus <= 0) cus = big_compute_units();
     const int tm = ceil_div(m, BIG_BM);
     const double wide = (double)ceil_div(tm * ceil_div(n, 256), cus) * 2.0;
     const double narrow = (double)ceil_div(tm * ceil_div(n, 128), cus) * 1.08;
@@ -642,6 +846,15 @@ static bool big_use_wide(int m, int n) {
 // The 128-row tile: asked for (tile code BIG_TILE_LOW), or chosen for up to 128 rows.
 #define BIG_TILE_LOW 1
 static bool big_use_low(int m, int tile) { return tile == BIG_TILE_LOW || (tile == 0 && m <= 128); }
+// A tile code may carry a word on streaming: + BIG_TILE_STREAM asks for it, + BIG_TILE_NO_STREAM forbids it
+// (measurements and tests of each tile shape either way); without, the launcher chooses.
+#define BIG_TILE_STREAM 1000
+#define BIG_TILE_NO_STREAM 2000
+static int big_tile_shape(int tile) { return tile % BIG_TILE_STREAM; }
+static bool big_tile_code_ok(int tile) {
+    const int shape = big_tile_shape(tile);
+    return tile >= 0 && tile < 3 * BIG_TILE_STREAM && (shape == 0 || shape == BIG_TILE_LOW || shape == 128 || shape == 256);
+}
 
 template <int BM, int BN, int S, int NW, int EPI, bool KTAIL, bool WONCE>
 static int big_launch_once(const BigArgs& args, hipStream_t stream) {
@@ -664,8 +877,13 @@ static int big_launch_once(const BigArgs& args, hipStream_t stream) {
         const int cus_per_die = big_compute_units() / 8 > 0 ? big_compute_units() / 8 : 1;
         per_die = per < cus_per_die ? per : cus_per_die;
     }
-    hipLaunchKernelGGL((linear_big_kernel<BM, BN, S, NW, EPI, KTAIL, WONCE>), dim3(per_die * 8), dim3(NW * 64), lds_bytes, stream, args);
+    const int grid = args.stream_wgs > 0 ? args.stream_wgs : per_die * 8;
+    hipLaunchKernelGGL((linear_big_kernel<BM, BN, S, NW, EPI, KTAIL, WONCE>), dim3(grid), dim3(NW * 64), lds_bytes, stream, args);
     SOMI_LAUNCH_CHECK("linear_big");
+    if (args.stream_wgs > 1) {
+        hipLaunchKernelGGL((big_stream_finish_kernel<BM, BN>), dim3(args.stream_wgs - 1, BM / 16), dim3(256), 0, stream, args, EPI);
+        SOMI_LAUNCH_CHECK("linear_big: finish");
+    }
     if (EPI == BIG_RESIDUAL && args.partial != nullptr) {
         if (args.reduce_plain)
             hipLaunchKernelGGL(big_split_reduce_plain_kernel, dim3(ceil_div(args.N, 64), ceil_div(args.M, 16)), dim3(256), 0, stream, args);
@@ -676,12 +894,14 @@ static int big_launch_once(const BigArgs& args, hipStream_t stream) {
     return 0;
 }
 
-// A weight that one row tile reads is read once: its loads carry the hint (the 128-row tile is only ever used so).
+// A weight that one row tile reads is read once: the 128-row tile's loads of it carry the hint (decode steps of 96
+// and 128 requests 4 and 2 % shorter).  The 256-row tiles are left without: where they have one row tile it changes
+// nothing inside decode steps (256 requests: 17.5 ms either way), and a weight that is still in the memory-side
+// cache from the call before is read slower with it (7B q/k/v at 256 rows in a loop: 85 us against 74).
 template <int BM, int BN, int S, int NW, int EPI, bool KTAIL>
 static int big_launch_one(const BigArgs& args, hipStream_t stream) {
-    if (BM == 128 || args.tiles_m == 1) return big_launch_once<BM, BN, S, NW, EPI, KTAIL, true>(args, stream);
-    if constexpr (BM != 128) return big_launch_once<BM, BN, S, NW, EPI, KTAIL, false>(args, stream);
-    return 0;
+    if constexpr (BM == 128) return big_launch_once<BM, BN, S, NW, EPI, KTAIL, true>(args, stream);
+    else return big_launch_once<BM, BN, S, NW, EPI, KTAIL, false>(args, stream);
 }
 
 // How many workgroups share a tile's K in the residual form (tiles of three whole stages): as many as give about
@@ -704,26 +924,41 @@ static int big_splits(int tiles, int m, int n, int k, int64_t workspace_floats) 
 template <int EPI>
 static int big_launch(BigArgs& args, int tile, hipStream_t stream, float* workspace = nullptr, int64_t workspace_floats = 0) {
     const bool ktail = args.K % BIG_BK != 0;
+    const int shape = big_tile_shape(tile), word = tile - shape;
+    const int cus = big_compute_units();
     args.splits = 1;
     args.partial = nullptr;
+    args.stream_wgs = 0;
+    args.slots = nullptr;
     auto split_k = [&]() {                     // the tiles are set: share their K where they are few
-        if (EPI != BIG_RESIDUAL || workspace == nullptr) return;
+        if (EPI != BIG_RESIDUAL || workspace == nullptr || word == BIG_TILE_STREAM) return;
         args.splits = big_splits(args.tiles_m * args.tiles_n, args.M, args.N, args.K, workspace_floats);
         if (args.splits > 1) args.partial = workspace;
     };
-    if (big_use_low(args.M, tile)) {
+    auto stream_units = [&](int bm, int bn) {  // or deal out (tile, stage) units where the tiles' rounds leave units idle
+        if (workspace == nullptr || args.splits > 1 || word == BIG_TILE_NO_STREAM) return;
+        const int tiles = args.tiles_m * args.tiles_n, wgs = cus / 8 * 8;
+        if (wgs < 8 || (int64_t)wgs * 2 * bm * bn > workspace_floats) return;
+        if (word == BIG_TILE_STREAM ? (int64_t)tiles * ceil_div(args.K, BIG_BK) >= wgs : big_streams(tiles, args.K, cus)) {
+            args.stream_wgs = wgs;
+            args.slots = workspace;
+        }
+    };
+    if (big_use_low(args.M, shape)) {
         // up to 128 rows: one row tile of 128, four wavefronts side by side over 256 columns
         args.tiles_m = ceil_div(args.M, 128);
         args.tiles_n = ceil_div(args.N, 256);
         args.stats_rows = args.tiles_n * 4;
         split_k();
+        stream_units(128, 256);
         return ktail ? big_launch_one<128, 256, 3, 4, EPI, true>(args, stream) : big_launch_one<128, 256, 3, 4, EPI, false>(args, stream);
     }
-    const bool wide = tile == 0 ? big_use_wide(args.M, args.N) : tile == 256;
+    const bool wide = shape == 0 ? big_use_wide(args.M, args.N, args.K) : shape == 256;
     args.tiles_m = ceil_div(args.M, BIG_BM);
     args.tiles_n = ceil_div(args.N, wide ? 256 : 128);
     args.stats_rows = wide ? args.tiles_n * 4 : args.tiles_n * 2;
     if (!wide) split_k();
+    if (wide || word == BIG_TILE_STREAM) stream_units(BIG_BM, wide ? 256 : 128);
     if (wide) return ktail ? big_launch_one<256, 256, 5, 8, EPI, true>(args, stream) : big_launch_one<256, 256, 5, 8, EPI, false>(args, stream);
     return ktail ? big_launch_one<256, 128, 3, 4, EPI, true>(args, stream) : big_launch_one<256, 128, 3, 4, EPI, false>(args, stream);
 }
@@ -775,17 +1010,43 @@ extern "C" int somi_row_scale(const float* stats, int blocks, int width, int m, 
 // Workgroup columns that write row statistics in the residual form: the first size of stats_out.
 // tile: 0 lets the launcher choose (the 128-row tile up to 128 rows, else 256-row tiles of the width that fills the
 // device better); 128 or 256 asks for that width of the 256-row tile, 1 for the 128-row tile (128 x 256).
-extern "C" int somi_linear_big_stats_blocks(int m, int n, int tile) {
+extern "C" int somi_linear_big_stats_blocks(int m, int n, int k, int tile) {
+    tile = big_tile_shape(tile);
     if (big_use_low(m, tile)) return ceil_div(n, 256) * 4;
-    const bool wide = tile == 0 ? big_use_wide(m, n) : tile == 256;
+    const bool wide = tile == 0 ? big_use_wide(m, n, k) : tile == 256;
     return wide ? ceil_div(n, 256) * 4 : ceil_div(n, 128) * 2;
 }
 
 // Workgroups that share a tile's K in somi_linear_big_residual with this much workspace (1: K is not split).
 extern "C" int somi_linear_big_splits(int m, int n, int k, int tile, int64_t workspace_floats) {
+    if (tile - big_tile_shape(tile) == BIG_TILE_STREAM) return 1;
+    tile = big_tile_shape(tile);
     if (big_use_low(m, tile)) return big_splits(ceil_div(m, 128) * ceil_div(n, 256), m, n, k, workspace_floats);
-    const bool wide = tile == 0 ? big_use_wide(m, n) : tile == 256;
+    const bool wide = tile == 0 ? big_use_wide(m, n, k) : tile == 256;
     return wide ? 1 : big_splits(ceil_div(m, BIG_BM) * ceil_div(n, 128), m, n, k, workspace_floats);
+}
+
+// Workgroups that the product's (tile, stage) units are dealt out to with this much workspace, as the entry points
+// choose (0: the tiles are handed out whole), for a device of `units` compute units (0: the current device).
+extern "C" int somi_linear_big_streams(int m, int n, int k, int tile, int64_t workspace_floats, int units) {
+    const int cus = units > 0 ? units : big_compute_units();
+    const int shape = big_tile_shape(tile), word = tile - shape;
+    if (word == BIG_TILE_NO_STREAM) return 0;
+    int bm = 256, bn = 128, tiles;
+    bool may = false;
+    if (big_use_low(m, shape)) {
+        bm = 128; bn = 256; tiles = ceil_div(m, 128) * ceil_div(n, 256);
+        may = big_splits(tiles, m, n, k, workspace_floats) <= 1 || word == BIG_TILE_STREAM;
+    } else {
+        const bool wide = shape == 0 ? big_use_wide(m, n, k, cus) : shape == 256;
+        bn = wide ? 256 : 128;
+        tiles = ceil_div(m, BIG_BM) * ceil_div(n, bn);
+        may = wide || word == BIG_TILE_STREAM;
+    }
+    const int wgs = cus / 8 * 8;
+    if (!may || wgs < 8 || (int64_t)wgs * 2 * bm * bn > workspace_floats) return 0;
+    const bool yes = word == BIG_TILE_STREAM ? (int64_t)tiles * ceil_div(k, BIG_BK) >= wgs : big_streams(tiles, k, cus);
+    return yes ? wgs : 0;
 }
 
 // out = s * (x . w^T) + bias -> bfloat16 [M, N]; with swiglu w is [N, K] with gate and up rows interleaved in blocks
@@ -797,7 +1058,7 @@ extern "C" int somi_linear_big(const void* x, int64_t ldx, const void* w, int64_
     if (big_check("linear_big", x, ldx, w, ldw, m, n, k) != 0) return 1;
     SOMI_REQUIRE(out != nullptr, "linear_big: no output");
     SOMI_REQUIRE(!swiglu || (n % 32 == 0 && bias == nullptr), "linear_big: the gated form needs N a multiple of 32 and no bias");
-    SOMI_REQUIRE(tile == 0 || tile == BIG_TILE_LOW || tile == 128 || tile == 256, "linear_big: tile code %d (0, 1, 128 or 256)", tile);
+    SOMI_REQUIRE(big_tile_code_ok(tile), "linear_big: tile code %d (0, 1, 128 or 256, + 1000 or 2000)", tile);
     BigArgs args = {};
     args.x = (const bf16*)x; args.ldx = ldx; args.w = (const bf16*)w; args.ldw = ldw; args.bias = bias;
     args.M = m; args.N = n; args.K = k; args.out = (bf16*)out;
@@ -809,7 +1070,8 @@ extern "C" int somi_linear_big(const void* x, int64_t ldx, const void* w, int64_
         args.reduce_plain = 1;
         return big_launch<BIG_RESIDUAL>(args, tile, stream, workspace, workspace_floats);
     }
-    return swiglu ? big_launch<BIG_SWIGLU>(args, tile, stream) : big_launch<BIG_PLAIN>(args, tile, stream);
+    return swiglu ? big_launch<BIG_SWIGLU>(args, tile, stream, workspace, workspace_floats)
+                  : big_launch<BIG_PLAIN>(args, tile, stream, workspace, workspace_floats);
 }
 
 // h += x . w^T + bias, float32 in place [M, N].  norm_w / weighted (or null): weighted = bfloat16(norm_w * h);
@@ -825,7 +1087,7 @@ extern "C" int somi_linear_big_residual(const void* x, int64_t ldx, const void* 
     SOMI_REQUIRE(h != nullptr, "linear_big_residual: no residual stream");
     SOMI_REQUIRE((weighted == nullptr) == (norm_w == nullptr), "linear_big_residual: the norm's weight and its rows come together");
     SOMI_REQUIRE(stats_out == nullptr || stats_width >= m, "linear_big_residual: row statistics of width %d do not cover %d rows", stats_width, m);
-    SOMI_REQUIRE(tile == 0 || tile == BIG_TILE_LOW || tile == 128 || tile == 256, "linear_big_residual: tile code %d (0, 1, 128 or 256)", tile);
+    SOMI_REQUIRE(big_tile_code_ok(tile), "linear_big_residual: tile code %d (0, 1, 128 or 256, + 1000 or 2000)", tile);
     BigArgs args = {};
     args.x = (const bf16*)x; args.ldx = ldx; args.w = (const bf16*)w; args.ldw = ldw; args.bias = bias;
     args.M = m; args.N = n; args.K = k; args.h = h; args.norm_w = norm_w; args.weighted = (bf16*)weighted;
@@ -838,12 +1100,15 @@ extern "C" int somi_linear_big_residual(const void* x, int64_t ldx, const void* 
 // out = x . w^T + bias -> float32 [M, N] (logits of many rows, which must not pass through bfloat16): the residual
 // form's end writing its sums instead of adding them, without the norm's by-products.
 extern "C" int somi_linear_big_f32(const void* x, int64_t ldx, const void* w, int64_t ldw, const float* bias, float* out,
-                                   int m, int n, int k, int tile, hipStream_t stream) {
+                                   int m, int n, int k, int tile, float* workspace, int64_t workspace_floats,
+                                   hipStream_t stream) {
     if (big_check("linear_big_f32", x, ldx, w, ldw, m, n, k) != 0) return 1;
     SOMI_REQUIRE(out != nullptr, "linear_big_f32: no output");
-    SOMI_REQUIRE(tile == 0 || tile == BIG_TILE_LOW || tile == 128 || tile == 256, "linear_big_f32: tile code %d (0, 1, 128 or 256)", tile);
+    SOMI_REQUIRE(big_tile_code_ok(tile), "linear_big_f32: tile code %d (0, 1, 128 or 256, + 1000 or 2000)", tile);
     BigArgs args = {};
     args.x = (const bf16*)x; args.ldx = ldx; args.w = (const bf16*)w; args.ldw = ldw; args.bias = bias;
     args.M = m; args.N = n; args.K = k; args.h = out; args.overwrite = 1;
-    return big_launch<BIG_RESIDUAL>(args, tile, stream);
+    SOMI_REQUIRE(workspace == nullptr || (((uintptr_t)workspace & 15) == 0 && workspace_floats >= 0),
+                 "linear_big_f32: the workspace must be aligned to 16 bytes");
+    return big_launch<BIG_RESIDUAL>(args, tile, stream, workspace, workspace_floats);
 }

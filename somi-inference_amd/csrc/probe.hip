@@ -61,6 +61,41 @@ probe_stream_buffer_kernel(const u32x4* __restrict__ src, int64_t pieces, unsign
     if ((threadIdx.x & 63) == 0) atomicXor(out + blockIdx.x, v);
 }
 
+// The read pattern of a tiled matrix product's weight operand: the buffer is a matrix of rows of `row_bytes`; a
+// workgroup owns 256 consecutive rows and walks them in steps of 128 bytes a row (2,048 loads of 16 bytes a step, two
+// steps in flight).  SHARE workgroups own the same rows and take the steps in turns (SHARE = 1: each its own rows).
+template <int SHARE>
+__global__ void __launch_bounds__(256)
+probe_tile_rows_kernel(const char* __restrict__ src, int row_groups, int row_bytes, unsigned int* __restrict__ out) {
+    const int group = blockIdx.x / SHARE, turn = blockIdx.x % SHARE;
+    if (group >= row_groups) return;
+    const int steps = row_bytes / 128;
+    const char* base = src + ((int64_t)group * 256 + (threadIdx.x >> 3)) * row_bytes + (threadIdx.x & 7) * 16;
+    u32x4 acc = {0u, 0u, 0u, 0u};
+    u32x4 a[8], b[8];
+    auto fetch = [&](u32x4 (&to)[8], int step) {
+#pragma unroll
+        for (int pass = 0; pass < 8; ++pass)
+            to[pass] = *(const u32x4*)(base + (int64_t)pass * 32 * row_bytes + (int64_t)step * 128);
+    };
+    int step = turn;
+    if (step < steps) fetch(a, step);
+    for (; step < steps; step += 2 * SHARE) {
+        if (step + SHARE < steps) fetch(b, step + SHARE);
+#pragma unroll
+        for (int pass = 0; pass < 8; ++pass) acc ^= a[pass];
+        if (step + 2 * SHARE < steps) fetch(a, step + 2 * SHARE);
+        if (step + SHARE < steps) {
+#pragma unroll
+            for (int pass = 0; pass < 8; ++pass) acc ^= b[pass];
+        }
+    }
+    unsigned int v = acc[0] ^ acc[1] ^ acc[2] ^ acc[3];
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v ^= __shfl_xor(v, off, 64);
+    if ((threadIdx.x & 63) == 0) atomicXor(out + (blockIdx.x & 1023), v);
+}
+
 // Every wavefront multiplies `iters` times four independent 32 x 32 x 16 bfloat16 products (32,768 flops each).
 __global__ void __launch_bounds__(512)
 probe_mfma_kernel(int iters, float* __restrict__ out) {
@@ -102,6 +137,10 @@ static const ProbeShape probe_shapes[] = {
     {"buffer loads, sc1", 256, 8, 116, 8},
     {"buffer loads, sc1 nt", 256, 8, 118, 8},
     {"buffer loads, sc0 sc1 nt", 256, 8, 119, 8},
+    // the weight operand of a tiled product: 256 rows of 7,168 bytes a workgroup, 128 bytes of each row a step
+    // (`nontemporal` holds 200 + the workgroups that share a group of rows and take its steps in turns)
+    {"tile rows: 256 rows x 128 bytes a step", 256, 2, 201, 0},
+    {"tile rows, steps shared by 8 workgroups in turns", 256, 2, 208, 0},
 };
 #define PROBE_SHAPES ((int)(sizeof(probe_shapes) / sizeof(probe_shapes[0])))
 
@@ -113,6 +152,7 @@ extern "C" const char* somi_probe_stream_shape_name(int shape) {
 // Workgroups of the streaming read in launch shape `shape`: what `out` must hold.
 extern "C" int somi_probe_stream_blocks(int shape) {
     if (shape < 0 || shape >= PROBE_SHAPES) return 0;
+    if (probe_shapes[shape].nontemporal >= 200) return 1024;
     return somi_units() * probe_shapes[shape].blocks_per_unit;
 }
 
@@ -135,6 +175,16 @@ extern "C" int somi_probe_stream_read(const void* src, int64_t bytes, int shape,
     SOMI_PROBE(256, 4, 0) SOMI_PROBE(256, 8, 0) SOMI_PROBE(256, 16, 0) SOMI_PROBE(512, 8, 0)
     SOMI_PROBE(256, 8, 1) SOMI_PROBE(512, 16, 1)
 #undef SOMI_PROBE
+    if (ps.nontemporal >= 200) {
+        // rows of 7,168 bytes (a K of 3,584 bfloat16): as many whole groups of 256 rows as the buffer holds
+        const int row_bytes = 7168, share = ps.nontemporal - 200;
+        const int groups = (int)(bytes / ((int64_t)row_bytes * 256));
+        SOMI_REQUIRE(groups > 0, "probe_stream_read: the buffer holds no group of 256 rows");
+        if (share == 1) hipLaunchKernelGGL((probe_tile_rows_kernel<1>), dim3(groups), block, 0, stream, (const char*)src, groups, row_bytes, out);
+        else hipLaunchKernelGGL((probe_tile_rows_kernel<8>), dim3(groups * 8), block, 0, stream, (const char*)src, groups, row_bytes, out);
+        SOMI_LAUNCH_CHECK("probe_stream_read");
+        return 0;
+    }
 #define SOMI_PROBE_BUFFER(AUX)                                                                                   \
     if (ps.nontemporal == 100 + AUX) {                                                                           \
         SOMI_REQUIRE(bytes / grid.x < ((int64_t)1 << 31), "probe_stream_read: too many bytes a workgroup for a buffer descriptor"); \

@@ -9,7 +9,6 @@ from . import ops
 SKINNY_MAX_ROWS = 64   # what the skinny MFMA kernel takes
 MID_PASSES_ROWS = 128  # up to here a product with long K and few columns runs the split-K kernel in passes of 64 rows
 SKINNY_ROWS = 64       # up to here the few-rows kernels run; beyond, the many-rows kernel (ops.linear_big)
-RESIDUAL_PASSES_ROWS = 128   # up to here a product into the residual stream with few columns runs in passes of 64 rows
 
 
 LONG_K = 8192            # a K that the split-K kernel cuts into eight pieces of sixteen chunks
@@ -38,19 +37,6 @@ def prefers_mid_passes(m: int, n: int, k: int) -> bool:
     return SKINNY_ROWS < m <= MID_PASSES_ROWS and k >= LONG_K and n <= FEW_COLUMNS_PER_UNIT * ops.compute_units()
 
 
-RESIDUAL_PASSES_MAX_K = LONG_K   # below this K
-
-
-def residual_in_passes(m: int, n: int, k: int) -> bool:
-    """A product into the residual stream with few columns, a short K and little more than 64 rows (o of 65 to 128
-    requests) runs as passes of the few-rows kernel: the tiles of the many-rows kernel are too few to fill the
-    device there, and with so short a K sharing it among workgroups does not pay (7B sizes, 128 rows, inside decode
-    steps: two passes 2 x 12 us, the many-rows kernel with K split 35 + 12).  A long K (down) is what that split is
-    for: steps of 80 / 96 / 128 requests are 3.4 / 2.5 / 2.4 % shorter with it than with passes."""
-    return (ops.FUSED_MAX_ROWS < m <= RESIDUAL_PASSES_ROWS and n <= FEW_COLUMNS_PER_UNIT * ops.compute_units()
-            and k < RESIDUAL_PASSES_MAX_K)
-
-
 def linear_swiglu(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
     """silu(x @ gate.T) * (x @ up.T) for bfloat16 rows; weight: [2 I, K], gate and up rows interleaved in blocks
     of 16."""
@@ -65,24 +51,10 @@ def linear_swiglu(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
 def linear_residual(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, h: torch.Tensor,
                     next_norm_weight: torch.Tensor | None = None) -> tuple[torch.Tensor, torch.Tensor | None]:
     """h += x @ weight.T (+ bias) in place, by the kernel that :func:`linear` would take for the sizes; see
-    :func:`ops.linear_residual`."""
+    :func:`ops.linear_residual`.  More than 64 rows take the many-rows kernel, which shares a tile's K among workgroups
+    where its tiles are few (o and down of 65 to some hundred rows; passes of the few-rows kernel over 64 rows each
+    measured the same inside decode steps of 128 requests, 10.70 against 10.72 ms)."""
     m, n = x.shape[0], weight.shape[0]
-    if residual_in_passes(m, n, x.shape[1]):
-        # one kernel for every pass, the short last one too: the passes' statistics have one row per workgroup and
-        # lie side by side in one table
-        k = x.shape[1]
-        mid = _mid_is_faster(ops.FUSED_MAX_ROWS, n, k)
-        stats = torch.empty((ops.residual_stats_blocks(ops.FUSED_MAX_ROWS, n, k, mid), ops.stats_width(m)),
-                            dtype=torch.float32, device=x.device)
-        weighted = None
-        if next_norm_weight is not None:
-            weighted = torch.empty((m, n), dtype=torch.bfloat16, device=x.device)
-        for at in range(0, m, ops.FUSED_MAX_ROWS):
-            upto = min(at + ops.FUSED_MAX_ROWS, m)
-            ops.linear_residual(x[at:upto], weight, bias, h[at:upto], next_norm_weight, mid=mid,
-                                stats_out=stats[:, at:at + ops.stats_width(upto - at)],
-                                weighted_out=weighted[at:upto] if weighted is not None else None)
-        return stats, weighted
     if m > ops.FUSED_MAX_ROWS:
         return ops.linear_big_residual(x, weight, bias, h, next_norm_weight)
     mid = _mid_is_faster(m, n, x.shape[1])

@@ -319,7 +319,9 @@ def linear_skinny_swiglu(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
     return out
 
 
-MID_WORKSPACE_FLOATS = 8 << 20        # 32 MB per device: partial sums of a split K (the kernel splits less if it is short)
+# 136 MB per device: partial sums of a split K (a kernel splits less if it is short) and, in the streamed many-rows
+# product, two slots of a 256 x 256 tile's sums for each of 256 workgroups
+MID_WORKSPACE_FLOATS = 34 << 20
 _mid_workspaces: dict[torch.device, torch.Tensor] = {}
 
 
@@ -389,7 +391,7 @@ def linear_big(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None 
     if out is None:
         out = torch.empty((m, cols), dtype=torch.bfloat16, device=x.device)
     _need(out, "linear_big out", torch.bfloat16, (m, cols))
-    workspace = _mid_workspace(x.device) if split_k and not swiglu else None
+    workspace = _mid_workspace(x.device) if split_k else None
     _check(library().somi_linear_big(_ptr(x), ctypes.c_int64(x.stride(0)), _ptr(weight), ctypes.c_int64(weight.stride(0)),
                                      _ptr(bias), _ptr(out), m, n, k, _ptr(row_scale), 1 if swiglu else 0, int(tile),
                                      _ptr(workspace), ctypes.c_int64(workspace.numel() if workspace is not None else 0),
@@ -408,7 +410,7 @@ def linear_big_residual(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tenso
     m, n, k = _big_operands(x, weight, bias, "linear_big_residual")
     _need(h, "residual stream", torch.float32, (m, n))
     lib = library()
-    blocks = lib.somi_linear_big_stats_blocks(m, n, int(tile))
+    blocks = lib.somi_linear_big_stats_blocks(m, n, k, int(tile))
     stats = torch.empty((blocks, _stats_width(m)), dtype=torch.float32, device=x.device)
     weighted = None
     if next_norm_weight is not None:
@@ -430,14 +432,25 @@ def linear_big_f32(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | N
     if out is None:
         out = torch.empty((m, n), dtype=torch.float32, device=x.device)
     _need(out, "linear_big_f32 out", torch.float32, (m, n))
+    workspace = _mid_workspace(x.device)
     _check(library().somi_linear_big_f32(_ptr(x), ctypes.c_int64(x.stride(0)), _ptr(weight), ctypes.c_int64(weight.stride(0)),
-                                         _ptr(bias), _ptr(out), m, n, k, int(tile), _stream()))
+                                         _ptr(bias), _ptr(out), m, n, k, int(tile), _ptr(workspace),
+                                         ctypes.c_int64(workspace.numel()), _stream()))
     return out
+
+
+BIG_TILE_STREAM, BIG_TILE_NO_STREAM = 1000, 2000      # added to a tile code: ask for the streamed form, or forbid it
 
 
 def linear_big_splits(m: int, n: int, k: int, tile: int = 0) -> int:
     """Workgroups that share a tile's K in :func:`linear_big_residual` for these sizes (1: K is not split)."""
     return library().somi_linear_big_splits(m, n, k, int(tile), ctypes.c_int64(MID_WORKSPACE_FLOATS))
+
+
+def linear_big_streams(m: int, n: int, k: int, tile: int = 0, units: int = 0) -> int:
+    """Workgroups that the (tile, stage) units of the many-rows product are dealt out to for these sizes (0: tiles
+    are handed out whole), on a device of ``units`` compute units (0: the current device)."""
+    return library().somi_linear_big_streams(m, n, k, int(tile), ctypes.c_int64(MID_WORKSPACE_FLOATS), int(units))
 
 
 def residual_stats_blocks(m: int, n: int, k: int, mid: bool) -> int:

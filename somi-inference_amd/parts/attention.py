@@ -23,8 +23,6 @@ from .base import Fetch, LayerCache, Mixer, PagedKVSpec, PartSpec, Runtime
 from .linear import NormedRows, Projection
 from .registry import build_part
 
-ROTATE_STORE_PASSES_ROWS = 128      # up to here the q/k/v product with rotation and store runs in passes of its 64 rows
-
 
 class GroupedQueryAttention(Mixer):
     graph_safe = True
@@ -135,7 +133,7 @@ class GroupedQueryAttention(Mixer):
         inv_freq, rotary_dim = rotation
         rows = x.shape[0]
         if (rotary_dim != self.head_dim or self.head_dim % 32 or cache.k.dtype != torch.bfloat16
-                or rows > ROTATE_STORE_PASSES_ROWS or not self.qkv.fusable(min(rows, ops.FUSED_MAX_ROWS))):
+                or rows > ops.FUSED_MAX_ROWS or not self.qkv.fusable(rows)):
             return None
         if isinstance(x, NormedRows):
             weighted, eps, stats = x.weighted, x.norm.eps, x.stats
@@ -143,18 +141,6 @@ class GroupedQueryAttention(Mixer):
             weighted, eps, stats = x, 0.0, None
         else:
             return None
-        if rows <= ops.FUSED_MAX_ROWS:
-            return ops.linear_rope_store(weighted, eps, stats, self.qkv.weight, self.qkv.bias, step.positions,
-                                         view.slot_mapping, inv_freq, self.num_heads, self.num_kv_heads, self.head_dim,
-                                         cache.k, cache.v)
-        # a little more than the kernel's 64 rows: in passes (7B sizes, 128 rows: 2 x 19 us against 69 for the row
-        # scales, the many-rows product, whose 128 x 256 tiles are 18 workgroups there, and the rotation and store)
-        q = torch.empty((rows, self.num_heads * self.head_dim), dtype=torch.bfloat16, device=weighted.device)
-        for at in range(0, rows, ops.FUSED_MAX_ROWS):
-            upto = min(at + ops.FUSED_MAX_ROWS, rows)
-            ops.linear_rope_store(weighted[at:upto], eps,
-                                  stats[:, at:at + ops.stats_width(upto - at)] if stats is not None else None,
-                                  self.qkv.weight, self.qkv.bias, step.positions[at:upto], view.slot_mapping[at:upto],
-                                  inv_freq, self.num_heads, self.num_kv_heads, self.head_dim, cache.k, cache.v,
-                                  out=q[at:upto])
-        return q
+        return ops.linear_rope_store(weighted, eps, stats, self.qkv.weight, self.qkv.bias, step.positions,
+                                     view.slot_mapping, inv_freq, self.num_heads, self.num_kv_heads, self.head_dim,
+                                     cache.k, cache.v)

@@ -821,6 +821,88 @@ def test_many_rows_product_into_the_stream_with_k_split_over_workgroups(m, n, k,
     torch.testing.assert_close(no_bias, h0 + F.linear(x.float(), w.float()), **tol)
 
 
+STREAM = ops.BIG_TILE_STREAM
+STREAMED_TILES = [STREAM + 1, STREAM + 128, STREAM + 256]
+STREAMED_IDS = ["128-row", "256x128", "256x256"]
+# (tile, stage) units dealt out to 256 workgroups: between one and a few stages each, so that a tile's K is walked by
+# up to a dozen workgroups (300 x 1100), by two or three (700 x 520), with tails in M, N and K (K = 200 ends in a stage)
+STREAMED_SHAPES = [(300, 1100, 2056), (100, 2072, 2056), (700, 520, 4104), (2048, 264, 1032), (1500, 3000, 200)]
+
+
+@pytest.mark.parametrize("tile", STREAMED_TILES, ids=STREAMED_IDS)
+@pytest.mark.parametrize("m,n,k", STREAMED_SHAPES)
+def test_many_rows_product_with_its_units_dealt_out_plain_and_float32(m, n, k, tile):
+    """The streamed form of the many-rows product: workgroups walk equal ranges of (tile, stage) units, the segments
+    that do not cover a tile's K leave their sums in slots, and a second kernel ends the tiles that were shared.
+    Plain (bias, row scales, bfloat16) and float32 results against F.linear and against the same tile unstreamed."""
+    if ops.linear_big_streams(m, n, k, tile=tile) == 0:
+        pytest.skip("too few units for this tile")
+    x, w, bias = rnd(m, k, dtype="bfloat16", seed=1), rnd(n, k, dtype="bfloat16", seed=2, scale=0.3), rnd(n, seed=3)
+    want = F.linear(x.float(), w.float(), bias)
+    tol = dict(atol=0.02 * float(want.abs().max()), rtol=2e-2)
+    got = ops.linear_big(x, w, bias, tile=tile)
+    torch.testing.assert_close(got.float(), want, **tol)
+    whole = ops.linear_big(x, w, bias, tile=tile - STREAM + ops.BIG_TILE_NO_STREAM, split_k=False)
+    torch.testing.assert_close(got.float(), whole.float(), atol=float(want.abs().max()) * 2 ** -7, rtol=2 ** -7)
+    assert torch.equal(ops.linear_big(x, w, bias, tile=tile), got)              # the slots are used again: the same bits
+    eps, width = 1e-5, 16 * ((m + 15) // 16)
+    stats = torch.zeros(2, width, device=DEV)
+    stats[:, :m] = torch.rand(2, m, device=DEV) * k * 4
+    s = torch.rsqrt(stats[:, :m].sum(0) / k + eps)[:, None]
+    scaled = ops.linear_big(x, w, None, eps=eps, stats=stats, tile=tile)
+    want_scaled = s * (x.float() @ w.float().t())
+    torch.testing.assert_close(scaled.float(), want_scaled, atol=0.02 * float(want_scaled.abs().max()), rtol=2e-2)
+    out = torch.full((m, n), 7.0, device=DEV)
+    f32 = ops.linear_big_f32(x, w, bias, tile=tile, out=out)
+    torch.testing.assert_close(f32, want, atol=2e-5 * float(want.abs().max()) * math.sqrt(k), rtol=1e-5)
+
+
+@pytest.mark.parametrize("tile", STREAMED_TILES, ids=STREAMED_IDS)
+@pytest.mark.parametrize("m,inter,k", [(700, 272, 4104), (1500, 1488, 200), (100, 1040, 2056), (2048, 144, 1032)])
+def test_many_rows_product_with_its_units_dealt_out_and_the_gate_in_its_end(m, inter, k, tile):
+    if ops.linear_big_streams(m, 2 * inter, k, tile=tile) == 0:
+        pytest.skip("too few units for this tile")
+    x = rnd(m, k, dtype="bfloat16", seed=6)
+    gate, up = rnd(inter, k, dtype="bfloat16", seed=7, scale=0.2), rnd(inter, k, dtype="bfloat16", seed=8, scale=0.2)
+    eps, width = 1e-6, 16 * ((m + 15) // 16)
+    stats = torch.zeros(2, width, device=DEV)
+    stats[:, :m] = torch.rand(2, m, device=DEV) * k * 4
+    s = torch.rsqrt(stats[:, :m].sum(0) / k + eps)[:, None]
+    want = F.silu(s * (x.float() @ gate.float().t())) * (s * (x.float() @ up.float().t()))
+    got = ops.linear_big(x, _interleave16(gate, up), swiglu=True, eps=eps, stats=stats, tile=tile)
+    assert got.shape == (m, inter)
+    torch.testing.assert_close(got.float(), want, atol=0.02 * float(want.abs().max()) + 1e-3, rtol=2e-2)
+    whole = ops.linear_big(x, _interleave16(gate, up), swiglu=True, eps=eps, stats=stats,
+                           tile=tile - STREAM + ops.BIG_TILE_NO_STREAM)
+    torch.testing.assert_close(got.float(), whole.float(), atol=float(want.abs().max()) * 2 ** -7 + 1e-3, rtol=2 ** -7)
+
+
+@pytest.mark.parametrize("tile", STREAMED_TILES, ids=STREAMED_IDS)
+@pytest.mark.parametrize("m,n,k", STREAMED_SHAPES)
+def test_many_rows_product_with_its_units_dealt_out_into_the_residual_stream(m, n, k, tile):
+    if ops.linear_big_streams(m, n, k, tile=tile) == 0:
+        pytest.skip("too few units for this tile")
+    x, w, bias = rnd(m, k, dtype="bfloat16", seed=9), rnd(n, k, dtype="bfloat16", seed=10, scale=0.2), rnd(n, seed=11)
+    h0 = rnd(m, n, seed=12)
+    norm_w = rnd(n, seed=13).abs() + 0.5
+    want_h = h0 + F.linear(x.float(), w.float(), bias)
+    tol = dict(atol=2e-4 * float(want_h.abs().max()) + 1e-4, rtol=1e-4)
+    h = h0.clone()
+    stats, weighted = ops.linear_big_residual(x, w, bias, h, norm_w, tile=tile)
+    torch.testing.assert_close(h, want_h, **tol)
+    assert torch.equal(weighted, (norm_w * h).to(torch.bfloat16))
+    torch.testing.assert_close(stats[:, :m].sum(0), h.pow(2).sum(1), rtol=1e-4, atol=1e-3)
+    whole = h0.clone()
+    whole_stats, _ = ops.linear_big_residual(x, w, bias, whole, norm_w, tile=tile - STREAM + ops.BIG_TILE_NO_STREAM,
+                                             split_k=False)
+    assert whole_stats.shape == stats.shape
+    torch.testing.assert_close(h, whole, **tol)
+    torch.testing.assert_close(stats[:, :m], whole_stats[:, :m], rtol=1e-3, atol=1e-3)
+    again = h0.clone()
+    ops.linear_big_residual(x, w, bias, again, norm_w, tile=tile)
+    assert torch.equal(again, h)
+
+
 @pytest.mark.parametrize("nq, nkv, d, page, window", [(8, 2, 128, 16, 0), (14, 2, 64, 8, 700), (4, 4, 128, 64, 1500)])
 @pytest.mark.parametrize("shape", [0, 4, 5], ids=["auto", "tile", "tile-wide"])
 def test_attention_prefill_tile_kernel_over_long_contexts(nq, nkv, d, page, window, shape):

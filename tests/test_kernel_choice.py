@@ -46,11 +46,6 @@ def test_a_split_is_no_longer_than_the_page_list_in_lds_holds(device_of_256_unit
 
 
 def test_rows_of_a_product_into_the_stream_choose_their_kernel(device_of_256_units):
-    # o of 65 to 128 requests (short K, few columns) runs in passes of the few-rows kernel; down (long K) does not
-    assert products.residual_in_passes(96, 3584, 3584) and products.residual_in_passes(128, 3584, 3584)
-    assert not products.residual_in_passes(96, 3584, 18944)
-    assert not products.residual_in_passes(64, 3584, 3584) and not products.residual_in_passes(129, 3584, 3584)
-    assert not products.residual_in_passes(96, 152064, 3584)
     # a kept product with a long K and few columns: passes of the split-K kernel up to 128 rows
     assert products.prefers_mid_passes(100, 3584, 18944) and not products.prefers_mid_passes(129, 3584, 18944)
     assert not products.prefers_mid_passes(100, 37888, 3584)
@@ -117,3 +112,16 @@ def test_launch_shapes_inside_the_library_go_with_the_devices_compute_units():
     # the tile kernel: 256 queries a workgroup from two groups a unit on
     assert shape(1, 2048, 2048, 28, 256, tile=1) == TILE and shape(1, 8192, 8192, 28, 256, tile=1) == TILE_WIDE
     assert shape(1, 8192, 8192, 28, 512, tile=1) == TILE
+
+
+def test_the_many_rows_product_deals_out_units_only_where_it_is_asked_to():
+    """Dealing out (tile, stage) units is there for the asking and never chosen (it measured slower than whole tiles
+    at every number of rows); asked for, it takes a workgroup a compute unit, within what the workspace holds."""
+    streams = lambda m, n, k, tile=0, units=256: ops.linear_big_streams(m, n, k, tile, units)
+    for m in (128, 256, 512, 2048):
+        assert streams(m, 4608, 3584) == 0 and streams(m, 37888, 3584) == 0 and streams(m, 3584, 18944) == 0
+    asked = ops.BIG_TILE_STREAM + 256
+    assert streams(2048, 4608, 3584, asked) == 256 and streams(2048, 4608, 3584, asked, units=272) == 272
+    assert streams(2048, 4608, 3584, asked, units=500) == 0       # more workgroups than the workspace has slots for
+    assert streams(64, 256, 64, asked) == 0                        # fewer units than workgroups
+    assert streams(2048, 4608, 3584, ops.BIG_TILE_NO_STREAM + 256) == 0
