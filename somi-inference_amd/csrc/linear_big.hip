@@ -83,6 +83,7 @@ struct BigArgs {
                                       // (the splits of a tile run side by side and so read neighbouring lines of a row)
     int stats_rows;                   // rows of stats_out (one per 64 columns of the tiles)
     int reduce_plain;                 // the splits' sums end as the plain form does: out = s * sum + bias in bfloat16
+                                      // (2: and are then rotated and stored, see big_split_reduce_rope_kernel)
     // Streamed: the (tile, stage) units of the whole product, tiles in launch order, stages within a tile, are dealt
     // out to `stream_wgs` workgroups in equal contiguous ranges, so any number of tiles keeps every compute unit busy
     // to the end.  A range may begin or end inside a tile: such a segment leaves its sums in one of the workgroup's
@@ -90,6 +91,13 @@ struct BigArgs {
     // and big_stream_finish_kernel adds a tile's segments in stage order and does what the epilogue would have done.
     int stream_wgs;                   // 0: not streamed
     float* slots;
+    // the q/k/v product whose splits' sums end rotated and stored (big_split_reduce_rope_kernel)
+    const int* positions;             // [M]
+    const int* cache_slots;           // [M]: page * page_size + offset of the token's k and v, or -1 for no store
+    const float* inv_freq;            // [D / 2]
+    bf16* k_cache;                    // [pages, nkv, page_size, D]
+    bf16* v_cache;                    // [pages, nkv, D, page_size]
+    int nq, nkv, D, page_size;
 };
 
 // silu(gate) * up = gate * up / (1 + e^-gate) with the hardware's base-2 exponential and reciprocal (each within
@@ -815,6 +823,70 @@ big_stream_finish_kernel(const BigArgs p, int epi) {
     }
 }
 
+// The end of the q/k/v product where K was split: the splits' sums, added in split order, scaled per row, plus the
+// bias, rounded to bfloat16, then what the rotary encoding and the cache store do in a kernel of their own elsewhere
+// (rope_kv.hip, and the end of the few-rows q/k/v product in linear_fused.hip, whose rounding this follows: the sum is
+// rounded before it is rotated, so k in the cache does not depend on which kernel wrote it): q and k heads are rotated
+// by the token's position (x' = x cos + rotate_half(x) sin, channels j and j + D/2 together), q goes to out
+// [M, nq D], k and v to their pages (v transposed inside a page).  A workgroup takes one head of 16 rows; a thread
+// the channels j .. j + 3 and j + D/2 .. of a row.
+// Reference: somi_inference/models/qwen2.py:95-113, 286-293; core/paged_attention.py:246-292.
+__global__ void __launch_bounds__(256)
+big_split_reduce_rope_kernel(const BigArgs p) {
+    const int row = threadIdx.x >> 4, lane = threadIdx.x & 15;
+    const int gm = blockIdx.y * 16 + row, head = blockIdx.x;
+    const int M = p.M, N = p.N, D = p.D, half = D / 2, nq = p.nq, nkv = p.nkv;
+    if (gm >= M) return;
+    const float scale = p.row_scale != nullptr ? p.row_scale[gm] : 1.f;
+    const int64_t plane = (int64_t)M * N;
+    const float pos = (float)p.positions[gm];
+    const int slot = p.cache_slots[gm];
+    for (int j = lane * 4; j < half; j += 64) {
+        const int gn = head * D + j;
+        const float* pp = p.partial + (int64_t)gm * N + gn;
+        f32x4 lo = {0.f, 0.f, 0.f, 0.f}, hi = lo;
+        for (int sp = 0; sp < p.splits; ++sp) {
+            lo += *(const f32x4*)(pp + sp * plane);
+            hi += *(const f32x4*)(pp + sp * plane + half);
+        }
+        bf16x4 first, second;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const float x1 = (float)(bf16)(scale * lo[e] + (p.bias != nullptr ? p.bias[gn + e] : 0.f));
+            const float x2 = (float)(bf16)(scale * hi[e] + (p.bias != nullptr ? p.bias[gn + half + e] : 0.f));
+            if (head < nq + nkv) {
+                const float angle = pos * p.inv_freq[j + e];
+                const float c = cosf(angle), sn = sinf(angle);
+                first[e] = (bf16)(x1 * c - x2 * sn);
+                second[e] = (bf16)(x2 * c + x1 * sn);
+            } else {
+                first[e] = (bf16)x1;
+                second[e] = (bf16)x2;
+            }
+        }
+        if (head < nq) {
+            bf16* to = p.out + (int64_t)gm * nq * D + head * D + j;
+            *(bf16x4*)to = first;
+            *(bf16x4*)(to + half) = second;
+            continue;
+        }
+        if (slot < 0) continue;
+        const int64_t page = slot / p.page_size, off = slot % p.page_size;
+        if (head < nq + nkv) {
+            bf16* to = p.k_cache + ((page * nkv + (head - nq)) * p.page_size + off) * D + j;
+            *(bf16x4*)to = first;
+            *(bf16x4*)(to + half) = second;
+        } else {
+            bf16* to = p.v_cache + ((page * nkv + (head - nq - nkv)) * D + j) * p.page_size + off;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                to[(int64_t)e * p.page_size] = first[e];
+                to[(int64_t)(half + e) * p.page_size] = second[e];
+            }
+        }
+    }
+}
+
 // ---------------------------------------------------------------------- host side
 static int big_compute_units() { return somi_units(); }
 
@@ -885,7 +957,9 @@ static int big_launch_once(const BigArgs& args, hipStream_t stream) {
         SOMI_LAUNCH_CHECK("linear_big: finish");
     }
     if (EPI == BIG_RESIDUAL && args.partial != nullptr) {
-        if (args.reduce_plain)
+        if (args.reduce_plain == 2)
+            hipLaunchKernelGGL(big_split_reduce_rope_kernel, dim3(args.nq + 2 * args.nkv, ceil_div(args.M, 16)), dim3(256), 0, stream, args);
+        else if (args.reduce_plain)
             hipLaunchKernelGGL(big_split_reduce_plain_kernel, dim3(ceil_div(args.N, 64), ceil_div(args.M, 16)), dim3(256), 0, stream, args);
         else
             hipLaunchKernelGGL(big_split_reduce_kernel, dim3(args.stats_rows, ceil_div(args.M, 16)), dim3(256), 0, stream, args);
@@ -1110,5 +1184,39 @@ extern "C" int somi_linear_big_f32(const void* x, int64_t ldx, const void* w, in
     args.M = m; args.N = n; args.K = k; args.h = out; args.overwrite = 1;
     SOMI_REQUIRE(workspace == nullptr || (((uintptr_t)workspace & 15) == 0 && workspace_floats >= 0),
                  "linear_big_f32: the workspace must be aligned to 16 bytes");
+    return big_launch<BIG_RESIDUAL>(args, tile, stream, workspace, workspace_floats);
+}
+
+// The q/k/v product of many rows with the rotary encoding of q and k and the store of k and v into their cache pages
+// in its end, for the sizes at which the plain form shares a tile's K among workgroups (somi_linear_big_splits > 1
+// with this workspace; refused otherwise: the caller then runs somi_linear_big and the rotation as two calls).
+// w: [(nq + 2 nkv) D, K], the rows of the q heads, then the k heads, then the v heads; row_scale (or null): [M];
+// q: [M, nq D] bfloat16, out, rotated; positions, slots: [M] (slot = page * page_size + offset, or -1: nothing is
+// stored for the row); inv_freq: [D / 2] (the whole head is rotated); k_cache [pages, nkv, page_size, D], v_cache
+// [pages, nkv, D, page_size].  D a multiple of 8.
+extern "C" int somi_linear_big_rope_store(const void* x, int64_t ldx, const void* w, int64_t ldw, const float* bias, void* q,
+                                          int m, int k, const float* row_scale, const int* positions, const int* slots,
+                                          const float* inv_freq, void* k_cache, void* v_cache, int nq, int nkv, int D,
+                                          int page_size, int tile, float* workspace, int64_t workspace_floats,
+                                          hipStream_t stream) {
+    SOMI_REQUIRE(nq > 0 && nkv > 0 && D > 0 && D % 8 == 0, "linear_big_rope_store: head_dim (%d) must be a multiple of 8", D);
+    const int64_t columns = (int64_t)(nq + 2 * nkv) * D;
+    SOMI_REQUIRE(columns < ((int64_t)1 << 30), "linear_big_rope_store: too many columns");
+    const int n = (int)columns;
+    if (big_check("linear_big_rope_store", x, ldx, w, ldw, m, n, k) != 0) return 1;
+    SOMI_REQUIRE(q && positions && slots && inv_freq && k_cache && v_cache && page_size > 0,
+                 "linear_big_rope_store: q, positions, slots, inv_freq and the caches are needed");
+    SOMI_REQUIRE((uintptr_t)q % 8 == 0 && (uintptr_t)k_cache % 8 == 0, "linear_big_rope_store: q and the k cache must be 8-byte aligned");
+    SOMI_REQUIRE(big_tile_code_ok(tile), "linear_big_rope_store: tile code %d (0, 1, 128 or 256, + 1000 or 2000)", tile);
+    SOMI_REQUIRE(workspace != nullptr && ((uintptr_t)workspace & 15) == 0, "linear_big_rope_store: a workspace aligned to 16 bytes is needed");
+    SOMI_REQUIRE(somi_linear_big_splits(m, n, k, tile, workspace_floats) > 1,
+                 "linear_big_rope_store: at m=%d n=%d k=%d the product does not share K among workgroups", m, n, k);
+    BigArgs args = {};
+    args.x = (const bf16*)x; args.ldx = ldx; args.w = (const bf16*)w; args.ldw = ldw; args.bias = bias;
+    args.M = m; args.N = n; args.K = k; args.out = (bf16*)q; args.row_scale = row_scale;
+    args.positions = positions; args.cache_slots = slots; args.inv_freq = inv_freq;
+    args.k_cache = (bf16*)k_cache; args.v_cache = (bf16*)v_cache;
+    args.nq = nq; args.nkv = nkv; args.D = D; args.page_size = page_size;
+    args.reduce_plain = 2;
     return big_launch<BIG_RESIDUAL>(args, tile, stream, workspace, workspace_floats);
 }

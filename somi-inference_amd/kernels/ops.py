@@ -439,6 +439,42 @@ def linear_big_f32(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | N
     return out
 
 
+def linear_big_rope_store(x: torch.Tensor, eps: float, stats: torch.Tensor | None, weight: torch.Tensor,
+                          bias: torch.Tensor | None, positions: torch.Tensor, slots: torch.Tensor,
+                          inv_freq: torch.Tensor, nq: int, nkv: int, head_dim: int, k_cache: torch.Tensor,
+                          v_cache: torch.Tensor, tile: int = 0) -> torch.Tensor:
+    """The q/k/v product of many bfloat16 rows where it shares a tile's K among workgroups
+    (:func:`linear_big_splits` > 1), with the rows' scales (from ``stats``, as :func:`linear_big` takes them), the
+    rotary encoding of q and k and the store of k and v into their cache pages in the kernel that adds the splits'
+    sums -> q [M, nq * D], rotated.  Arguments as :func:`linear_rope_store`."""
+    n = (nq + 2 * nkv) * head_dim
+    m, n_w, k = _big_operands(x, weight, bias, "linear_big_rope_store")
+    if n_w != n:
+        raise KernelError(f"linear_big_rope_store: the weight has {n_w} rows, {nq} + 2 x {nkv} heads of {head_dim} are {n}")
+    row_scale = None
+    if stats is not None:
+        _need(stats, "row statistics", torch.float32)
+        if stats.dim() != 2 or stats.shape[1] < m:
+            raise KernelError(f"linear_big_rope_store: row statistics must be [blocks, >= {m}], got {tuple(stats.shape)}")
+        row_scale = torch.empty((m,), dtype=torch.float32, device=x.device)
+        _check(library().somi_row_scale(_ptr(stats), stats.shape[0], stats.shape[1], m, k, ctypes.c_float(eps),
+                                        _ptr(row_scale), _stream()))
+    _need(positions, "positions", torch.int32, (m,))
+    _need(slots, "slot mapping", torch.int32, (m,))
+    _need(inv_freq, "inv_freq", torch.float32, (head_dim // 2,))
+    _need(k_cache, "k cache", torch.bfloat16)
+    if k_cache.dim() != 4 or k_cache.shape[1] != nkv or k_cache.shape[3] != head_dim:
+        raise KernelError(f"linear_big_rope_store: cache shape {tuple(k_cache.shape)} != [pages, {nkv}, page, {head_dim}]")
+    _need(v_cache, "v cache", torch.bfloat16, _v_shape(k_cache))
+    q = torch.empty((m, nq * head_dim), dtype=torch.bfloat16, device=x.device)
+    workspace = _mid_workspace(x.device)
+    _check(library().somi_linear_big_rope_store(
+        _ptr(x), ctypes.c_int64(x.stride(0)), _ptr(weight), ctypes.c_int64(weight.stride(0)), _ptr(bias), _ptr(q), m, k,
+        _ptr(row_scale), _ptr(positions), _ptr(slots), _ptr(inv_freq), _ptr(k_cache), _ptr(v_cache), nq, nkv, head_dim,
+        k_cache.shape[2], int(tile), _ptr(workspace), ctypes.c_int64(workspace.numel()), _stream()))
+    return q
+
+
 BIG_TILE_STREAM, BIG_TILE_NO_STREAM = 1000, 2000      # added to a tile code: ask for the streamed form, or forbid it
 
 

@@ -126,14 +126,15 @@ class GroupedQueryAttention(Mixer):
         return self.out.deferred(attended)        # the residual stream may add it in the kernel that computes it
 
     def _project_rotate_store(self, x, step, view, cache: LayerCache, rotation) -> torch.Tensor | None:
-        """q of the step's tokens, rotated, with k and v in their pages, by the q/k/v product itself; None where
-        that kernel does not apply (many rows, float32, a head that is not rotated as a whole, no k/v of its own)."""
+        """q of the step's tokens, rotated, with k and v in their pages, by the q/k/v product itself (up to 64 rows) or
+        by the kernel that adds the sums of its K splits (some hundred rows); None where neither applies (many rows,
+        float32, a head that is not rotated as a whole, no k/v of its own)."""
         if rotation is None or self.shares_cache:
             return None
         inv_freq, rotary_dim = rotation
         rows = x.shape[0]
         if (rotary_dim != self.head_dim or self.head_dim % 32 or cache.k.dtype != torch.bfloat16
-                or rows > ops.FUSED_MAX_ROWS or not self.qkv.fusable(rows)):
+                or not self.qkv.fusable(rows)):
             return None
         if isinstance(x, NormedRows):
             weighted, eps, stats = x.weighted, x.norm.eps, x.stats
@@ -141,6 +142,14 @@ class GroupedQueryAttention(Mixer):
             weighted, eps, stats = x, 0.0, None
         else:
             return None
+        if rows > ops.FUSED_MAX_ROWS:
+            # some hundred rows: the many-rows product shares a tile's K among workgroups, and the kernel that adds
+            # their sums rotates and stores (more rows have tiles enough: the product, then the rotation)
+            if ops.linear_big_splits(rows, self.qkv.out_features, self.qkv.in_features) <= 1:
+                return None
+            return ops.linear_big_rope_store(weighted, eps, stats, self.qkv.weight, self.qkv.bias, step.positions,
+                                             view.slot_mapping, inv_freq, self.num_heads, self.num_kv_heads,
+                                             self.head_dim, cache.k, cache.v)
         return ops.linear_rope_store(weighted, eps, stats, self.qkv.weight, self.qkv.bias, step.positions,
                                      view.slot_mapping, inv_freq, self.num_heads, self.num_kv_heads, self.head_dim,
                                      cache.k, cache.v)

@@ -821,6 +821,65 @@ def test_many_rows_product_into_the_stream_with_k_split_over_workgroups(m, n, k,
     torch.testing.assert_close(no_bias, h0 + F.linear(x.float(), w.float()), **tol)
 
 
+@pytest.mark.parametrize("scaled", [True, False], ids=["normed", "as-is"])
+@pytest.mark.parametrize("m, nq, nkv, d, hidden, page", [(65, 4, 2, 32, 1032, 16), (100, 12, 2, 64, 2056, 8),
+                                                         (128, 28, 4, 128, 3584, 16), (300, 6, 2, 96, 2056, 8),
+                                                         (513, 5, 1, 64, 1536, 32)])
+def test_qkv_product_of_many_rows_rotates_and_stores_where_it_adds_its_splits(m, nq, nkv, d, hidden, page, scaled):
+    """The q/k/v product of some hundred rows shares K among workgroups; the kernel that adds their sums scales the
+    rows, adds the bias, rotates q and k and stores k and v in their pages.  Against the float32 formulas and
+    against the same product followed by the rotation kernel (the same sums rounded at the same places)."""
+    eps, theta = 1e-5, 1e4
+    pages = (m + page - 1) // page + 3
+    n_out = (nq + 2 * nkv) * d
+    assert ops.linear_big_splits(m, n_out, hidden) > 1
+    w, b = rnd(n_out, hidden, dtype="bfloat16", seed=2, scale=0.05), rnd(n_out, seed=3)
+    positions = i32([(7 * t * t + 3) % 5000 for t in range(m)])
+    order = torch.randperm(pages * page, generator=torch.Generator().manual_seed(5)).tolist()[:m]
+    order[m // 2] = -1                                                        # a token without a slot is not stored
+    slots = i32(order)
+    inv_freq = plain.rope_inv_freq(d, theta).to(DEV)
+    if scaled:
+        h = rnd(m, hidden, seed=4, scale=2.0)
+        norm_w = 1.0 + rnd(hidden, seed=5, scale=0.1)
+        x = (norm_w * h).to(torch.bfloat16)
+        stats = torch.zeros(3, 16 * ((m + 15) // 16), device=DEV)
+        stats[1, :m] = h.pow(2).sum(dim=1)
+        exact_x = x.float() * torch.rsqrt(h.pow(2).mean(dim=1, keepdim=True) + eps)
+    else:
+        x, stats = rnd(m, hidden, dtype="bfloat16", seed=4), None
+        exact_x = x.float()
+    kc = torch.zeros(pages, nkv, page, d, dtype=torch.bfloat16, device=DEV)
+    vc = torch.zeros(pages, nkv, d, page, dtype=torch.bfloat16, device=DEV)
+    q = ops.linear_big_rope_store(x, eps, stats, w, b, positions, slots, inv_freq, nq, nkv, d, kc, vc)
+    heads = F.linear(exact_x, w.float(), b).view(m, nq + 2 * nkv, d).cpu()
+    cos, sin = plain.rope_cos_sin(positions.cpu(), d, theta)
+    want_q = plain.apply_rope(heads[:, :nq].transpose(0, 1), cos, sin).transpose(0, 1)
+    want_k = plain.apply_rope(heads[:, nq:nq + nkv].transpose(0, 1), cos, sin).transpose(0, 1)
+    tol = dict(atol=float(heads.abs().max()) * 2 ** -7, rtol=2 ** -7)
+    torch.testing.assert_close(q.float().view(m, nq, d).cpu(), want_q, **tol)
+    stored = [t for t, slot in enumerate(order) if slot >= 0]
+    at = torch.tensor([order[t] for t in stored])
+    torch.testing.assert_close(kc[at // page, :, at % page].float().cpu(), want_k[stored], **tol)
+    torch.testing.assert_close(vc[at // page, :, :, at % page].float().cpu(), heads[stored, nq + nkv:], **tol)
+    written = torch.zeros(pages * page, dtype=torch.bool)
+    written[at] = True
+    for cache in (kc.permute(0, 2, 1, 3), vc.permute(0, 3, 1, 2)):
+        assert float(cache.float().reshape(pages * page, -1).cpu()[~written].abs().sum()) == 0.0, \
+            "a slot that was not addressed was written"
+    # the separate kernels: the same product with its sums added by the plain kernel, then the rotation and the store
+    kc2, vc2 = torch.zeros_like(kc), torch.zeros_like(vc)
+    qkv = ops.linear_big(x, w, b, eps=eps, stats=stats) if scaled else ops.linear_big(x, w, b)
+    ops.rope_kv_store(qkv, positions, slots, inv_freq, d, nq, nkv, d, kc2, vc2)
+    assert torch.equal(q, qkv[:, :nq * d]) and torch.equal(kc, kc2) and torch.equal(vc, vc2)
+    with pytest.raises(KernelError, match="does not share K"):
+        big = rnd(2048, hidden, dtype="bfloat16", seed=6)
+        ops.linear_big_rope_store(big, eps, None, rnd(32 * 128 * 3, hidden, dtype="bfloat16"), None, i32([0] * 2048),
+                                  i32([-1] * 2048), plain.rope_inv_freq(128, theta).to(DEV), 32, 32, 128,
+                                  torch.zeros(1, 32, 16, 128, dtype=torch.bfloat16, device=DEV),
+                                  torch.zeros(1, 32, 128, 16, dtype=torch.bfloat16, device=DEV))
+
+
 STREAM = ops.BIG_TILE_STREAM
 STREAMED_TILES = [STREAM + 1, STREAM + 128, STREAM + 256]
 STREAMED_IDS = ["128-row", "256x128", "256x256"]
