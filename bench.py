@@ -288,22 +288,23 @@ class Workbench:
 
     # ----------------------------------------------------------------- serving
     def serving_run(self, count: int, max_concurrent: int, new_tokens: int = 256, chunk: int = 512,
-                    budget: int = 2048) -> dict:
-        """Continuous batching through the engine's own scheduler: everything arrives at once, prompts of 128 to
-        2,048 tokens are cut into portions of ``chunk`` under a budget of ``budget`` tokens a step, finished requests
+                    budget: int = 2048, prompt_range: tuple[int, int] = (128, 2048)) -> dict:
+        """Continuous batching through the engine's own scheduler: everything arrives at once, prompts of
+        ``prompt_range`` tokens (128 to 2,048) are cut into portions of ``chunk`` under a budget of ``budget`` tokens a step, finished requests
         free their pages.  Reported as a whole, with what a step held (the reference reports a run with its arrival
         trace: benchmarks/bench_engine.py:181-283)."""
         from somi_inference_amd.engine import Engine, Request, Scheduler
         from somi_inference_amd.engine.engine import full_collections_deferred
         torch, runner = self.torch, self.runner
-        lengths = torch.randint(128, 2049, (count,), generator=self.gen).tolist()
-        per_request = (2048 + new_tokens + self.block_size - 1) // self.block_size + 1
+        shortest, longest = prompt_range
+        lengths = torch.randint(shortest, longest + 1, (count,), generator=self.gen).tolist()
+        per_request = (longest + new_tokens + self.block_size - 1) // self.block_size + 1
         concurrent = max(1, min(count, max_concurrent, self.num_blocks // per_request))
         scheduler = Scheduler(runner.cache, max_concurrent=concurrent, max_num_batched_tokens=budget, chunk=chunk)
         engine = Engine(runner, scheduler, self.sampler, eos_token_id=-1)
         requests = [Request(f"s{i}", self.tokens(n), new_tokens, self.greedy, seed=i) for i, n in enumerate(lengths)]
         # as LLM.warm_up() does it: the decode graphs that the requests will replay are captured before they arrive
-        captured = runner.capture_decode_graphs(concurrent, 2048 + new_tokens)
+        captured = runner.capture_decode_graphs(concurrent, longest + new_tokens)
         prompt_mix, decode_mix, live_mix = [], [], []
         torch.cuda.synchronize()
         start = time.perf_counter()
