@@ -22,9 +22,11 @@
 //     cover 256 distinct bytes; the permutation is applied on the global side of the load (a lane's LDS
 //     position is fixed by the instruction);
 //   * a wavefront computes 128 x 64 of the tile as 4 x 2 products of 32 x 32 x 16 (128 accumulator
-//     registers); 8 wavefronts (wide) or 4 (narrow).  Two wavefronts on a SIMD matter: within one
-//     wavefront no instruction overlaps its own matrix instruction, so loads and LDS reads of one hide
-//     behind the products of the other;
+//     registers); 8 wavefronts (wide) or 4 (narrow).  (The wide tile on four wavefronts of 128 x 128 each, their
+//     sums in the accumulation registers, reads a third less from LDS per product and was measured slower:
+//     2,048 x 37,888 x 3,584 in 521 us against 455, x 3,584 x 18,944 in 368 against 349; a wavefront's own LDS
+//     reads do overlap its matrix instructions, but its waits at the barrier and for its loads leave the SIMD
+//     with nothing to run, and the gated end of 128 x 128 sums spills.);
 //   * fragment reads are software-pipelined one 16-deep sub-step ahead and issued between the products;
 //     the order of instructions in the loop is pinned (the compiler's own schedule waited for each read
 //     right after issuing it);
@@ -115,8 +117,11 @@ template <int N> __device__ __forceinline__ void big_wait_vmcnt() { asm volatile
 
 // S: 3 = a ring of three whole stages (narrow tile); 5 = five slots of 32 KB that hold one operand's stage each
 // (wide tile), filled in the order A0 B0 A1 B1 A2 ...: piece q goes to slot q % 5.  While stage kt is computed,
-// both pieces of stage kt + 1 and A of kt + 2 are in the ring or on their way; the barrier that ends the reads of
-// stage kt frees two slots, which take B of kt + 2 and A of kt + 3.
+// both pieces of stage kt + 1 are in the ring or on their way and A of kt + 2 is asked for; the barrier that ends the
+// reads of stage kt frees two slots, which take B of kt + 2 at once and A of kt + 3 during stage kt + 1.  No
+// wavefront asks for more than one load per product: every wavefront of a workgroup passes the barrier at the same
+// time, and eight loads each in a burst filled the unit that takes their addresses, so that the wavefronts waited
+// to issue and their matrix instructions with them (2,048 x 37,888 x 3,584: 526 us with the burst, 457 without).
 // The wide form is persistent: a workgroup walks its die's tiles 32 apart, and the first pieces of the next
 // tile are asked for before the finished tile is stored, so the stores and the first loads overlap.
 // BM: rows of a tile, 256 (two wavefronts along m) or 128 (one: for 65 to 128 rows, where a 256-row tile would
@@ -138,10 +143,13 @@ linear_big_kernel(const BigArgs p) {
     static_assert(HALF || (S == 3 && L % KK == 0), "three whole stages, loads divisible over the sub-steps");
     static_assert(!HALF || (LA == LB && BN == 256 && BM == 256), "halves of equal size");
     constexpr int LPS = HALF ? 0 : L / KK;
+    constexpr int SYNC_AFTER = 2;                                 // products of the last sub-step issued before the barrier
+    constexpr int LSUB = HALF ? LA / KK : 1;                      // wide ring: loads of the far piece per sub-step
+    static_assert(!HALF || (LA % KK == 0 && NM % LSUB == 0 && NM / LSUB > SYNC_AFTER && LA <= NF),
+                  "the wide ring's loads spread over the sub-steps and the read slots");
     constexpr int HB = 256 * ROW_BYTES;                           // bytes of a slot of the wide ring
     constexpr int STG = HALF ? 3 * HB : 0;                        // where the epilogue stages: slots 3 and 4, or the ring
     constexpr int STG_WAVE = 8192;
-    constexpr int SYNC_AFTER = 2;                                 // products of the last sub-step issued before the barrier
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -301,6 +309,7 @@ linear_big_kernel(const BigArgs p) {
             int sa = 0, sb = 1;                // slots of the stage computed on
             for (int kt = 0; kt < KT; ++kt) {
                 const int na = sa + 2 >= 5 ? sa - 3 : sa + 2, nb = sb + 2 >= 5 ? sb - 3 : sb + 2;     // slots of the next stage
+                const int sp = sa == 0 ? 4 : sa - 1;                                                   // the slot B of kt - 1 had
                 BIG_FENCE();
 #pragma unroll
                 for (int kk = 0; kk < KK; ++kk) {
@@ -314,26 +323,24 @@ linear_big_kernel(const BigArgs p) {
 #pragma unroll
                     for (int q = 0; q < NM; ++q) {
                         if (last && q == SYNC_AFTER) {
-                            // stage kt + 1 has landed (only A of kt + 2 may still be on its way); everybody has read stage kt
-                            big_wait_vmcnt<LA>();
+                            // stage kt + 1 has landed (only what this iteration has asked for of A of kt + 2 may still be
+                            // on its way); everybody has read stage kt
+                            big_wait_vmcnt<(KK - 1) * LSUB + 1>();
                             __builtin_amdgcn_s_barrier();
                             BIG_FENCE();
                         }
                         if (kk & 1) product(a1, b1, q); else product(a0, b0, q);
                         BIG_FENCE();
+                        // A of stage kt + 2 (piece 2 kt + 4) into the slot that B of kt - 1 had: over the sub-steps
+                        if (q % (NM / LSUB) == 0) {
+                            issue_piece(2 * kt + 4, sp, kk * LSUB + q / (NM / LSUB));
+                            BIG_FENCE();
+                        }
                         if ((!last || q >= SYNC_AFTER) && reads < NF) {
                             if (kk & 1) read_one(a0, b0, aa, ab, reads); else read_one(a1, b1, aa, ab, reads);
                             ++reads;
-                            if (last) {
-                                // B of stage kt + 2 into the slot A of kt had, then A of kt + 3 into the slot B of kt had
-#pragma unroll
-                                for (int e = 0; e < 2; ++e)
-                                    if (loads < 2 * LA) {
-                                        if (loads < LA) issue_piece(2 * kt + 5, sa, loads);
-                                        else issue_piece(2 * kt + 6, sb, loads - LA);
-                                        ++loads;
-                                    }
-                            }
+                            // B of stage kt + 2 into the slot A of kt had, which the barrier has just freed
+                            if (last && loads < LA) { issue_piece(2 * kt + 5, sa, loads); ++loads; }
                             BIG_FENCE();
                         }
                     }
