@@ -105,6 +105,10 @@ struct BigArgs {
 // silu(gate) * up = gate * up / (1 + e^-gate) with the hardware's base-2 exponential and reciprocal (each within
 // one unit in the last place of float32; the result is rounded to bfloat16): nine instructions a value where expf and
 // a float32 division take twenty-five, which a 2,048-row gate_up product feels (its end is 38.8 million values).
+// The plain form's end, s * sum + bias, as one fused multiply-add in every kernel that computes it, so that a product
+// gives the same bits whichever of them ends it (the compiler fuses the plain expression in some and not in others).
+__device__ __forceinline__ float big_scale_bias(float scale, float sum, float bias) { return __builtin_fmaf(scale, sum, bias); }
+
 __device__ __forceinline__ float big_silu_mul(float gate, float up) {
     return gate * up * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(-1.44269504088896341f * gate));
 }
@@ -482,7 +486,7 @@ linear_big_kernel(const BigArgs p) {
                         for (int g = 0; g < 4; ++g) {
                             bf16x4 v;
 #pragma unroll
-                            for (int c = 0; c < 4; ++c) v[c] = (bf16)(s * t[4 * g + c] + bv[j][4 * g + c]);
+                            for (int c = 0; c < 4; ++c) v[c] = (bf16)big_scale_bias(s, t[4 * g + c], bv[j][4 * g + c]);
                             *(bf16x4*)(stg + ml * SROW + (j * 32 + 8 * g + 4 * nh) * 2) = v;
                         }
                     }
@@ -704,11 +708,11 @@ big_split_reduce_plain_kernel(const BigArgs p) {
     if (four) {
         bf16x4 v;
 #pragma unroll
-        for (int c = 0; c < 4; ++c) v[c] = (bf16)(scale * sum[c] + (p.bias != nullptr ? p.bias[gn + c] : 0.f));
+        for (int c = 0; c < 4; ++c) v[c] = (bf16)big_scale_bias(scale, sum[c], p.bias != nullptr ? p.bias[gn + c] : 0.f);
         *(bf16x4*)op = v;
     } else {
         for (int c = 0; c < 4; ++c)
-            if (gn + c < N) op[c] = (bf16)(scale * sum[c] + (p.bias != nullptr ? p.bias[gn + c] : 0.f));
+            if (gn + c < N) op[c] = (bf16)big_scale_bias(scale, sum[c], p.bias != nullptr ? p.bias[gn + c] : 0.f);
     }
 }
 
@@ -779,7 +783,7 @@ big_stream_finish_kernel(const BigArgs p, int epi) {
             } else {
                 gc = gn;
 #pragma unroll
-                for (int e = 0; e < 4; ++e) v[e] = (bf16)(scale * sum[q][e] + (p.bias != nullptr && gn + e < N ? p.bias[gn + e] : 0.f));
+                for (int e = 0; e < 4; ++e) v[e] = (bf16)big_scale_bias(scale, sum[q][e], p.bias != nullptr && gn + e < N ? p.bias[gn + e] : 0.f);
             }
             bf16* dst = p.out + (int64_t)gm * out_n + gc;
             if (aligned && gc + 4 <= out_n) *(bf16x4*)dst = v;
@@ -859,8 +863,8 @@ big_split_reduce_rope_kernel(const BigArgs p) {
         bf16x4 first, second;
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-            const float x1 = (float)(bf16)(scale * lo[e] + (p.bias != nullptr ? p.bias[gn + e] : 0.f));
-            const float x2 = (float)(bf16)(scale * hi[e] + (p.bias != nullptr ? p.bias[gn + half + e] : 0.f));
+            const float x1 = (float)(bf16)big_scale_bias(scale, lo[e], p.bias != nullptr ? p.bias[gn + e] : 0.f);
+            const float x2 = (float)(bf16)big_scale_bias(scale, hi[e], p.bias != nullptr ? p.bias[gn + half + e] : 0.f);
             if (head < nq + nkv) {
                 const float angle = pos * p.inv_freq[j + e];
                 const float c = cosf(angle), sn = sinf(angle);
@@ -988,8 +992,10 @@ static int big_launch_one(const BigArgs& args, hipStream_t stream) {
 // How many workgroups share a tile's K in the residual form (tiles of three whole stages): as many as give about
 // every compute unit a workgroup, with at least BIG_SPLIT_MIN_STAGES stages each, within the workspace; 1 where the
 // tiles alone fill half of the device.  (7B down projection at 192 rows: 28 tiles of 256 x 128, 296 stages: 227 us
-// unsplit, 62 in 9 splits.)
-#define BIG_SPLIT_MIN_STAGES 8
+// unsplit, 62 in 9 splits.  At least 4 stages, not 8: a K of 896 has 14, and with 8 the products of a 0.5B layer at
+// 65 to 128 rows ran on the 4 or 5 workgroups of their tiles: steps of 96 / 128 requests 3.09 -> 2.63 / 3.30 -> 2.74
+// ms; at 7B sizes nothing changes.)
+#define BIG_SPLIT_MIN_STAGES 4
 static int big_splits(int tiles, int m, int n, int k, int64_t workspace_floats) {
     const int cus = big_compute_units();
     const int stages = ceil_div(k, BIG_BK);

@@ -496,15 +496,12 @@ def residual_stats_blocks(m: int, n: int, k: int, mid: bool) -> int:
 
 
 def linear_residual(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, h: torch.Tensor,
-                    next_norm_weight: torch.Tensor | None = None, mid: bool = False,
-                    stats_out: torch.Tensor | None = None, weighted_out: torch.Tensor | None = None
+                    next_norm_weight: torch.Tensor | None = None, mid: bool = False
                     ) -> tuple[torch.Tensor, torch.Tensor | None]:
     """h += x @ weight.T (+ bias) in float32, in place, for at most 64 bfloat16 rows.  Returns the row statistics
     ``[workgroups, 16 ceil(M / 16)]`` (per workgroup and row the sum of squares of the new h over the workgroup's
     columns) and, with ``next_norm_weight``, the rows ``bfloat16(next_norm_weight * h)`` that :func:`linear_scaled`
-    reads.  ``mid``: by the kernel that shares x inside a workgroup and splits K over workgroups.  ``stats_out``
-    (these rows' columns in the table of more rows) and ``weighted_out`` take the two results where the caller
-    keeps them."""
+    reads.  ``mid``: by the kernel that shares x inside a workgroup and splits K over workgroups."""
     _need(x, "linear input", torch.bfloat16)
     m, k = x.shape
     _need(weight, "linear weight", torch.bfloat16)
@@ -516,25 +513,12 @@ def linear_residual(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | 
     _need(h, "residual stream", torch.float32, (m, n))
     lib = library()
     blocks = residual_stats_blocks(m, n, k, mid)
-    stats_stride = 0
-    if stats_out is None:
-        stats = torch.empty((blocks, _stats_width(m)), dtype=torch.float32, device=x.device)
-    else:
-        stats = stats_out
-        if (not isinstance(stats, torch.Tensor) or not stats.is_cuda or stats.dtype != torch.float32 or stats.dim() != 2
-                or tuple(stats.shape) != (blocks, _stats_width(m)) or stats.stride(1) != 1 or stats.stride(0) % 4
-                or stats.data_ptr() % 16):
-            raise KernelError(f"linear_residual: the statistics go to float32 [{blocks}, {_stats_width(m)}] on the GPU "
-                              "with rows of consecutive floats")
-        stats_stride = stats.stride(0)
+    stats_stride = 0                    # rows of the statistics follow each other
+    stats = torch.empty((blocks, _stats_width(m)), dtype=torch.float32, device=x.device)
     weighted = None
     if next_norm_weight is not None:
         _need(next_norm_weight, "norm weight", torch.float32, (n,))
-        if weighted_out is None:
-            weighted = torch.empty((m, n), dtype=torch.bfloat16, device=x.device)
-        else:
-            _need(weighted_out, "weighted rows", torch.bfloat16, (m, n))
-            weighted = weighted_out
+        weighted = torch.empty((m, n), dtype=torch.bfloat16, device=x.device)
     if mid:
         workspace = _mid_workspace(x.device)
         _check(lib.somi_linear_mid_residual(_ptr(x), _ptr(weight), _ptr(bias), _ptr(h), _ptr(stats), stats_stride,
