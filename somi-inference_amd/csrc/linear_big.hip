@@ -70,6 +70,7 @@ struct BigArgs {
     int tiles_m, tiles_n;
     // plain / swiglu
     bf16* out;                        // [M, N] or [M, N / 2]
+    int64_t ldo;                      // row stride of out in elements (a product over a range of columns writes into wider rows)
     const float* row_scale;           // [M] the rows' scales s, or null
     // residual
     float* h;                         // [M, N] float32, in and out
@@ -85,7 +86,8 @@ struct BigArgs {
                                       // (the splits of a tile run side by side and so read neighbouring lines of a row)
     int stats_rows;                   // rows of stats_out (one per 64 columns of the tiles)
     int reduce_plain;                 // the splits' sums end as the plain form does: out = s * sum + bias in bfloat16
-                                      // (2: and are then rotated and stored, see big_split_reduce_rope_kernel)
+                                      // (2: and are then rotated and stored, see big_split_reduce_rope_kernel; 3: they end as the
+                                      // gated form does, see big_split_reduce_swiglu_kernel)
     // Streamed: the (tile, stage) units of the whole product, tiles in launch order, stages within a tile, are dealt
     // out to `stream_wgs` workgroups in equal contiguous ranges, so any number of tiles keeps every compute unit busy
     // to the end.  A range may begin or end inside a tile: such a segment leaves its sums in one of the workgroup's
@@ -462,7 +464,7 @@ linear_big_kernel(const BigArgs p) {
             constexpr int LPR = CW * 2 / 16;                                   // lanes per row when reading back
             const int out_n = EPI == BIG_SWIGLU ? N / 2 : N;
             const int out_c0 = EPI == BIG_SWIGLU ? wave_n0 / 2 : wave_n0;
-            const bool aligned = (out_n & 7) == 0 && ((uintptr_t)p.out & 15) == 0;
+            const bool aligned = (out_n & 7) == 0 && (p.ldo & 7) == 0 && ((uintptr_t)p.out & 15) == 0;
 #pragma unroll
             for (int i = 0; i < WTM; ++i) {
                 const float s = scale[i];            // the row scale of the norm whose rows x holds
@@ -499,7 +501,7 @@ linear_big_kernel(const BigArgs p) {
                     const int gm = m0 + wm * 128 + i * 32 + row;
                     const int gc = out_c0 + piece * 8;
                     if (gm < M) {
-                        bf16* dst = p.out + (int64_t)gm * out_n + gc;
+                        bf16* dst = p.out + (int64_t)gm * p.ldo + gc;
                         if (aligned && gc + 8 <= out_n) *(u32x4*)dst = v;
                         else {
                             const bf16* e = (const bf16*)&v;
@@ -516,9 +518,29 @@ linear_big_kernel(const BigArgs p) {
             const bool aligned = (N & 3) == 0 && ((uintptr_t)p.h & 15) == 0 &&
                                  (p.weighted == nullptr || ((uintptr_t)p.weighted & 7) == 0);
             const int stats_row = tn * WAVES_N + wn;
+            // With four wavefronts (512 registers each) the stream's values are asked for ahead of their use, a block
+            // of 32 rows at a time (eight loads of 16 bytes a lane), the next block's while this one is added: a load
+            // that is asked for where it is used waits for memory 32 times a tile (2,048 x 3,584 x 64, where the end
+            // is all there is: 29 us, of which the stream's 73 MB would take 12).  The tile of eight wavefronts has no
+            // registers to spare for it.
+            constexpr bool DEEP = NW == 4;
+            const bool ahead = DEEP && (HALF || p.partial == nullptr) && aligned && !p.overwrite;
+            f32x4 hq[DEEP ? 2 : 1][WTN][4];
+            auto ask = [&](int i, f32x4 (&q)[WTN][4]) {
+#pragma unroll
+                for (int j = 0; j < WTN; ++j)
+#pragma unroll
+                    for (int pass = 0; pass < 4; ++pass) {
+                        const int gm = m0 + wm * 128 + i * 32 + pass * 8 + (lane >> 3);
+                        const int gn = wave_n0 + j * 32 + (lane & 7) * 4;
+                        q[j][pass] = gm < M && gn + 4 <= N ? *(const f32x4*)(p.h + (int64_t)gm * N + gn) : f32x4{0.f, 0.f, 0.f, 0.f};
+                    }
+            };
+            if (ahead) ask(0, hq[0]);
 #pragma unroll
             for (int i = 0; i < WTM; ++i) {
                 float sq[4] = {0.f, 0.f, 0.f, 0.f};            // of the rows this lane reads back, over both products
+                if (ahead && i + 1 < WTM) ask(i + 1, hq[DEEP ? (i + 1) & 1 : 0]);
 #pragma unroll
                 for (int j = 0; j < WTN; ++j) {
 #pragma unroll
@@ -546,7 +568,7 @@ linear_big_kernel(const BigArgs p) {
                         } else if (gm < M && gn < N) {
                             float* hp = p.h + (int64_t)gm * N + gn;
                             if (aligned && gn + 4 <= N) {
-                                f32x4 hv = p.overwrite ? f32x4{0.f, 0.f, 0.f, 0.f} : *(const f32x4*)hp;
+                                f32x4 hv = p.overwrite ? f32x4{0.f, 0.f, 0.f, 0.f} : ahead ? hq[DEEP ? i & 1 : 0][j][pass] : *(const f32x4*)hp;
 #pragma unroll
                                 for (int c = 0; c < 4; ++c) {
                                     hv[c] += v[c] + (p.bias != nullptr ? p.bias[gn + c] : 0.f);
@@ -683,7 +705,7 @@ big_split_reduce_plain_kernel(const BigArgs p) {
     const int gm = blockIdx.y * 16 + row, gn = blockIdx.x * 64 + cg * 4;
     const int M = p.M, N = p.N;
     if (gm >= M || gn >= N) return;
-    const bool four = (N & 3) == 0 && ((uintptr_t)p.out & 7) == 0 && gn + 4 <= N;
+    const bool four = (N & 3) == 0 && (p.ldo & 3) == 0 && ((uintptr_t)p.out & 7) == 0 && gn + 4 <= N;
     f32x4 sum = {0.f, 0.f, 0.f, 0.f};
     const float* pp = p.partial + (int64_t)gm * N + gn;
     const int64_t plane = (int64_t)M * N;
@@ -704,7 +726,7 @@ big_split_reduce_plain_kernel(const BigArgs p) {
                 if (gn + c < N) sum[c] += pp[s * plane + c];
     }
     const float scale = p.row_scale != nullptr ? p.row_scale[gm] : 1.f;
-    bf16* op = p.out + (int64_t)gm * N + gn;
+    bf16* op = p.out + (int64_t)gm * p.ldo + gn;
     if (four) {
         bf16x4 v;
 #pragma unroll
@@ -764,7 +786,7 @@ big_stream_finish_kernel(const BigArgs p, int epi) {
         if (gm >= M) return;
         const float scale = p.row_scale != nullptr ? p.row_scale[gm] : 1.f;
         const int out_n = epi == BIG_SWIGLU ? N / 2 : N;
-        const bool aligned = (out_n & 3) == 0 && ((uintptr_t)p.out & 7) == 0;
+        const bool aligned = (out_n & 3) == 0 && (p.ldo & 3) == 0 && ((uintptr_t)p.out & 7) == 0;
 #pragma unroll
         for (int q = 0; q < QUADS; ++q) {
             if (epi == BIG_SWIGLU && q >= QUADS / 2) break;
@@ -785,7 +807,7 @@ big_stream_finish_kernel(const BigArgs p, int epi) {
 #pragma unroll
                 for (int e = 0; e < 4; ++e) v[e] = (bf16)big_scale_bias(scale, sum[q][e], p.bias != nullptr && gn + e < N ? p.bias[gn + e] : 0.f);
             }
-            bf16* dst = p.out + (int64_t)gm * out_n + gc;
+            bf16* dst = p.out + (int64_t)gm * p.ldo + gc;
             if (aligned && gc + 4 <= out_n) *(bf16x4*)dst = v;
             else
                 for (int e = 0; e < 4; ++e)
@@ -832,6 +854,34 @@ big_stream_finish_kernel(const BigArgs p, int epi) {
             if (cg == 0 && gm < M) p.stats_out[(int64_t)(tn * QUADS + q) * p.stats_width + gm] = sq;
         }
     }
+}
+
+// The end of the gated form where K was split: out = silu(s g) * (s u) with g and u the sums over the splits (in split
+// order) of a channel's gate and up columns, which lie 16 apart in blocks of 32 columns.  A workgroup takes 16 rows x
+// 128 columns of the product (64 of the output); a lane adds four gate columns and their four up columns.
+__global__ void __launch_bounds__(256)
+big_split_reduce_swiglu_kernel(const BigArgs p) {
+    const int row = threadIdx.x >> 4, cg = threadIdx.x & 15;
+    const int gm = blockIdx.y * 16 + row;
+    const int gn = blockIdx.x * 128 + (cg >> 2) * 32 + (cg & 3) * 4;      // first of the four gate columns
+    const int M = p.M, N = p.N;
+    if (gm >= M || gn >= N) return;
+    f32x4 gate = {0.f, 0.f, 0.f, 0.f}, up = gate;
+    const float* pp = p.partial + (int64_t)gm * N + gn;
+    const int64_t plane = (int64_t)M * N;
+    for (int sp = 0; sp < p.splits; ++sp) {
+        gate += *(const f32x4*)(pp + sp * plane);
+        up += *(const f32x4*)(pp + sp * plane + 16);
+    }
+    const float scale = p.row_scale != nullptr ? p.row_scale[gm] : 1.f;
+    bf16x4 v;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[e] = (bf16)big_silu_mul(scale * gate[e], scale * up[e]);
+    const int gc = (gn >> 5) * 16 + (gn & 15);
+    bf16* dst = p.out + (int64_t)gm * p.ldo + gc;
+    if ((p.ldo & 3) == 0 && ((uintptr_t)p.out & 7) == 0) *(bf16x4*)dst = v;
+    else
+        for (int e = 0; e < 4; ++e) dst[e] = v[e];
 }
 
 // The end of the q/k/v product where K was split: the splits' sums, added in split order, scaled per row, plus the
@@ -970,6 +1020,8 @@ static int big_launch_once(const BigArgs& args, hipStream_t stream) {
     if (EPI == BIG_RESIDUAL && args.partial != nullptr) {
         if (args.reduce_plain == 2)
             hipLaunchKernelGGL(big_split_reduce_rope_kernel, dim3(args.nq + 2 * args.nkv, ceil_div(args.M, 16)), dim3(256), 0, stream, args);
+        else if (args.reduce_plain == 3)
+            hipLaunchKernelGGL(big_split_reduce_swiglu_kernel, dim3(ceil_div(args.N, 128), ceil_div(args.M, 16)), dim3(256), 0, stream, args);
         else if (args.reduce_plain)
             hipLaunchKernelGGL(big_split_reduce_plain_kernel, dim3(ceil_div(args.N, 64), ceil_div(args.M, 16)), dim3(256), 0, stream, args);
         else
@@ -996,8 +1048,8 @@ static int big_launch_one(const BigArgs& args, hipStream_t stream) {
 // 65 to 128 rows ran on the 4 or 5 workgroups of their tiles: steps of 96 / 128 requests 3.09 -> 2.63 / 3.30 -> 2.74
 // ms; at 7B sizes nothing changes.)
 #define BIG_SPLIT_MIN_STAGES 4
-static int big_splits(int tiles, int m, int n, int k, int64_t workspace_floats) {
-    const int cus = big_compute_units();
+static int big_splits(int tiles, int m, int n, int k, int64_t workspace_floats, int cus = 0) {
+    if (cus <= 0) cus = big_compute_units();
     const int stages = ceil_div(k, BIG_BK);
     if (workspace_floats <= 0 || tiles * 2 > cus) return 1;
     int64_t splits = cus / tiles;
@@ -1136,6 +1188,46 @@ extern "C" int somi_linear_big_streams(int m, int n, int k, int tile, int64_t wo
     return yes ? wgs : 0;
 }
 
+// The tail of a product whose 256 x 128 tiles do not come out even over the compute units: the whole rounds of tiles run
+// as they are, and the column tiles that are left, too few to fill the device, share their K among workgroups as a
+// product of their own over the last columns (float32 sums in the workspace, ended by a reduce kernel).  7B gate_up at
+// 512 rows: two rounds and 80 tiles in 3 splits instead of three rounds, 142 us against 151 (and 160 for two rounds of
+// 256 x 256 tiles).  Only from two whole rounds on: after one round the tail's two launches cost what they save, and
+// one round of 256 x 256 tiles is faster than either (q/k/v at 2,048 rows: 88 us with a tail, 89 in two rounds, 78 on
+// 144 tiles of 256 x 256; gate_up at 256 rows: 87, 97, 76).
+// Returns the columns of the tail (0: the product runs whole) and its splits.  Costs in rounds of 256 x 128 tiles:
+// a round of 256 x 256 tiles counts 1.72 (91 us against 53 over K = 3,584), the tail's launches 0.45.
+static int big_tail(int m, int n, int k, int64_t workspace_floats, int cus, int* splits_out) {
+    if (cus <= 0) cus = big_compute_units();
+    *splits_out = 1;
+    if (m <= 128 || workspace_floats <= 0) return 0;
+    const int tiles_m = ceil_div(m, BIG_BM), col_tiles = ceil_div(n, 128), tiles = tiles_m * col_tiles;
+    if (tiles <= cus) return 0;
+    const int main_cols = (tiles / cus) * cus / tiles_m;            // column tiles of the whole rounds
+    const int tail_cols = col_tiles - main_cols, tail_tiles = tail_cols * tiles_m;
+    if (tail_tiles == 0 || main_cols == 0) return 0;
+    const int tail_n = n - main_cols * 128;
+    const int splits = big_splits(tail_tiles, m, tail_n, k, workspace_floats, cus);
+    if (splits < 2) return 0;
+    if (tiles / cus < 2) return 0;
+    const double whole_wide = (double)ceil_div(tiles_m * ceil_div(n, 256), cus) * 1.72;
+    const double whole_narrow = (double)ceil_div(tiles, cus);
+    const double with_tail = (double)(main_cols * tiles_m) / cus + 1.0 / splits + 0.45;
+    if (with_tail >= 0.97 * (whole_wide < whole_narrow ? whole_wide : whole_narrow)) return 0;
+    *splits_out = splits;
+    return tail_n;
+}
+
+// What somi_linear_big does with the last columns of a product at tile code 0 on a device of `units` compute units
+// (0: the current device): the columns that run as a product of their own with K shared (0: none), and in how many
+// splits.
+extern "C" int somi_linear_big_tail(int m, int n, int k, int64_t workspace_floats, int units, int* splits) {
+    int s = 1;
+    const int tail = big_tail(m, n, k, workspace_floats, units, &s);
+    if (splits != nullptr) *splits = s;
+    return tail;
+}
+
 // out = s * (x . w^T) + bias -> bfloat16 [M, N]; with swiglu w is [N, K] with gate and up rows interleaved in blocks
 // of 16 and out is [M, N / 2] = silu(s g) * (s u).  row_scale (or null): s [M], see somi_row_scale.  workspace (or
 // null): as in somi_linear_big_residual, for the plain form (q/k/v of some hundred rows: 72 tiles at 7B sizes).
@@ -1148,10 +1240,28 @@ extern "C" int somi_linear_big(const void* x, int64_t ldx, const void* w, int64_
     SOMI_REQUIRE(big_tile_code_ok(tile), "linear_big: tile code %d (0, 1, 128 or 256, + 1000 or 2000)", tile);
     BigArgs args = {};
     args.x = (const bf16*)x; args.ldx = ldx; args.w = (const bf16*)w; args.ldw = ldw; args.bias = bias;
-    args.M = m; args.N = n; args.K = k; args.out = (bf16*)out;
+    args.M = m; args.N = n; args.K = k; args.out = (bf16*)out; args.ldo = swiglu ? n / 2 : n;
     args.row_scale = row_scale;
     SOMI_REQUIRE(workspace == nullptr || (((uintptr_t)workspace & 15) == 0 && workspace_floats >= 0),
                  "linear_big: the workspace must be aligned to 16 bytes");
+    int tail_splits = 1;
+    const int tail_n = tile == 0 && workspace != nullptr ? big_tail(m, n, k, workspace_floats, 0, &tail_splits) : 0;
+    if (tail_n > 0) {
+        // whole rounds of 256 x 128 tiles over the first columns, then the last columns with their K shared
+        const int main_n = n - tail_n;
+        BigArgs head = args;
+        head.N = main_n;
+        const int rc = swiglu ? big_launch<BIG_SWIGLU>(head, 128 + BIG_TILE_NO_STREAM, stream)
+                              : big_launch<BIG_PLAIN>(head, 128 + BIG_TILE_NO_STREAM, stream);
+        if (rc != 0) return rc;
+        BigArgs tail = args;
+        tail.w = args.w + (int64_t)main_n * ldw;
+        tail.bias = bias != nullptr ? bias + main_n : nullptr;
+        tail.N = tail_n;
+        tail.out = args.out + (swiglu ? main_n / 2 : main_n);
+        tail.reduce_plain = swiglu ? 3 : 1;
+        return big_launch<BIG_RESIDUAL>(tail, 128 + BIG_TILE_NO_STREAM, stream, workspace, workspace_floats);
+    }
     if (!swiglu && workspace != nullptr && somi_linear_big_splits(m, n, k, tile, workspace_floats) > 1) {
         // the workgroups of a tile share its K and leave float32 sums; the reduce scales, adds the bias and rounds
         args.reduce_plain = 1;
@@ -1226,7 +1336,7 @@ extern "C" int somi_linear_big_rope_store(const void* x, int64_t ldx, const void
                  "linear_big_rope_store: at m=%d n=%d k=%d the product does not share K among workgroups", m, n, k);
     BigArgs args = {};
     args.x = (const bf16*)x; args.ldx = ldx; args.w = (const bf16*)w; args.ldw = ldw; args.bias = bias;
-    args.M = m; args.N = n; args.K = k; args.out = (bf16*)q; args.row_scale = row_scale;
+    args.M = m; args.N = n; args.K = k; args.out = (bf16*)q; args.ldo = (int64_t)nq * D; args.row_scale = row_scale;
     args.positions = positions; args.cache_slots = slots; args.inv_freq = inv_freq;
     args.k_cache = (bf16*)k_cache; args.v_cache = (bf16*)v_cache;
     args.nq = nq; args.nkv = nkv; args.D = D; args.page_size = page_size;

@@ -489,6 +489,15 @@ def linear_big_streams(m: int, n: int, k: int, tile: int = 0, units: int = 0) ->
     return library().somi_linear_big_streams(m, n, k, int(tile), ctypes.c_int64(MID_WORKSPACE_FLOATS), int(units))
 
 
+def linear_big_tail(m: int, n: int, k: int, units: int = 0) -> tuple[int, int]:
+    """(columns, splits): the last columns of a many-rows product (plain or gated, tile code 0) that run as a product
+    of their own with K shared among workgroups, where whole rounds of 256 x 128 tiles leave a tail too small to fill
+    the device; (0, 1) where the product runs whole.  ``units``: the device's compute units (0: the current device)."""
+    splits = ctypes.c_int(1)
+    columns = library().somi_linear_big_tail(m, n, k, ctypes.c_int64(MID_WORKSPACE_FLOATS), int(units), ctypes.byref(splits))
+    return columns, splits.value
+
+
 def residual_stats_blocks(m: int, n: int, k: int, mid: bool) -> int:
     """Rows of the statistics that :func:`linear_residual` writes for these sizes."""
     lib = library()

@@ -717,6 +717,39 @@ def test_many_rows_product_with_the_gate_in_its_end(m, inter, k, tile):
     torch.testing.assert_close(got.float(), want, atol=0.02 * float(want.abs().max()) + 1e-3, rtol=2e-2)
 
 
+@pytest.mark.parametrize("m,n,k", [(300, 2 * 17920 + 96, 1032), (129, 2 * 33000, 1032), (1000, 18016, 1032)])
+def test_many_rows_product_whose_last_columns_share_k(m, n, k):
+    """More 256 x 128 tiles than compute units, with a tail that is small: the whole rounds run as they are and the
+    last columns as a product of their own with K shared (a row stride of the output that is not its width, the
+    weight and bias from an offset).  Plain with bias and row scale and gated, against float32 and against the same
+    product on whole tiles."""
+    columns, splits = ops.linear_big_tail(m, n, k)
+    if ops.compute_units() == 256:
+        assert columns > 0 and splits > 1
+    x, w, bias = rnd(m, k, dtype="bfloat16", seed=1), rnd(n, k, dtype="bfloat16", seed=2, scale=0.3), rnd(n, seed=3)
+    eps, width = 1e-5, 16 * ((m + 15) // 16)
+    stats = torch.zeros(3, width, device=DEV)
+    stats[:, :m] = torch.rand(3, m, device=DEV) * k
+    scale = torch.rsqrt(stats[:, :m].sum(0) / k + eps)
+    want = scale[:, None] * F.linear(x.float(), w.float()) + bias
+    got = ops.linear_big(x, w, bias, eps=eps, stats=stats)
+    whole = ops.linear_big(x, w, bias, eps=eps, stats=stats, tile=128)
+    tol = dict(atol=0.02 * float(want.abs().max()), rtol=2e-2)
+    torch.testing.assert_close(got.float(), want, **tol)
+    assert torch.equal(got[:, :n - columns], whole[:, :n - columns])          # the whole rounds are the same launch
+    torch.testing.assert_close(got.float(), whole.float(), atol=float(want.abs().max()) * 2 ** -7, rtol=2 ** -7)
+    inter = n // 32 * 16
+    gate, up = w[:inter], rnd(inter, k, dtype="bfloat16", seed=8, scale=0.3)
+    mixed = _interleave16(gate, up)
+    assert ops.linear_big_tail(m, 2 * inter, k) == (columns - (n - 2 * inter), splits) or columns == 0
+    s = scale[:, None]
+    want = F.silu(s * (x.float() @ gate.float().t())) * (s * (x.float() @ up.float().t()))
+    got = ops.linear_big(x, mixed, swiglu=True, eps=eps, stats=stats)
+    whole = ops.linear_big(x, mixed, swiglu=True, eps=eps, stats=stats, tile=128)
+    torch.testing.assert_close(got.float(), want, atol=0.02 * float(want.abs().max()) + 1e-3, rtol=2e-2)
+    torch.testing.assert_close(got.float(), whole.float(), atol=float(want.abs().max()) * 2 ** -6, rtol=2 ** -6)
+
+
 @pytest.mark.parametrize("tile", [0, 1, 128, 256])
 @pytest.mark.parametrize("m,n,k", [(65, 132, 64), (128, 600, 264), (300, 520, 200), (1024, 72, 1032), (257, 256, 136)])
 def test_many_rows_product_into_the_residual_stream(m, n, k, tile):

@@ -125,3 +125,21 @@ def test_the_many_rows_product_deals_out_units_only_where_it_is_asked_to():
     assert streams(2048, 4608, 3584, asked, units=500) == 0       # more workgroups than the workspace has slots for
     assert streams(64, 256, 64, asked) == 0                        # fewer units than workgroups
     assert streams(2048, 4608, 3584, ops.BIG_TILE_NO_STREAM + 256) == 0
+
+
+def test_the_last_columns_of_a_many_rows_product_share_k_where_whole_rounds_leave_a_small_tail():
+    """A product whose 256 x 128 tiles are two or more whole rounds over the compute units and a tail that would
+    leave most of them idle runs the tail as a product of its own with K shared; after one round (a single round of
+    256 x 256 tiles is faster), where the tail is large, or up to 128 rows, the product runs whole."""
+    tail = lambda m, n, k, units=256: ops.linear_big_tail(m, n, k, units)
+    # gate_up at 512 rows: 2 x 296 tiles = two rounds and 80 tiles (40 column tiles) in 3 splits
+    assert tail(512, 37888, 3584) == (5120, 3)
+    # one whole round and a tail: 7B q/k/v at 2,048 rows (8 x 36 tiles), gate_up at 256 rows (296 tiles)
+    assert tail(2048, 4608, 3584) == (0, 1) and tail(256, 37888, 3584) == (0, 1)
+    # at 2,048 rows five rounds of 256 x 256 tiles cost less than nine rounds of 256 x 128 and a tail
+    assert tail(2048, 37888, 3584) == (0, 1)
+    # o and down (224 tiles), up to 128 rows, and a tail of more than half of the units: whole
+    assert tail(2048, 3584, 18944) == (0, 1) and tail(128, 37888, 3584) == (0, 1)
+    assert tail(1024, 37888, 3584) == (0, 1)                       # 4 x 296 = 1,184 tiles: a tail of 160
+    # half the device: 1 x 296 tiles are two rounds of 128 and 40 tiles in 3 splits
+    assert tail(256, 37888, 3584, units=128) == (5120, 3)
