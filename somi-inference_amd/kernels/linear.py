@@ -7,7 +7,6 @@ import torch
 from . import ops
 
 SKINNY_MAX_ROWS = 64   # what the skinny MFMA kernel takes
-MID_PASSES_ROWS = 128  # up to here a product with long K and few columns runs the split-K kernel in passes of 64 rows
 SKINNY_ROWS = 64       # up to here the few-rows kernels run; beyond, the many-rows kernel (ops.linear_big)
 
 
@@ -26,15 +25,6 @@ def _mid_is_faster(m: int, n: int, k: int) -> bool:
         return False
     units = ops.compute_units()
     return (k >= LONG_K and n <= FEW_COLUMNS_PER_UNIT * units) or n >= MANY_COLUMNS_PER_UNIT * units
-
-
-def prefers_mid_passes(m: int, n: int, k: int) -> bool:
-    """More than SKINNY_ROWS rows, but few enough that a product with a long K and few columns (down) runs faster
-    as passes of the split-K kernel over 64 rows each than on the 256-row tiles of the many-rows kernel, which are
-    too few to fill the device there (7B down projection: 62 to 67 us at 65 to 128 rows against 157).  The product
-    into the residual stream has ways of its own (passes that add into the stream up to 128 rows, the many-rows
-    kernel with K split over workgroups beyond); this is for a product that is kept."""
-    return SKINNY_ROWS < m <= MID_PASSES_ROWS and k >= LONG_K and n <= FEW_COLUMNS_PER_UNIT * ops.compute_units()
 
 
 def linear_swiglu(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
@@ -91,11 +81,6 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = No
         if _mid_is_faster(m, weight.shape[0], k):
             return ops.linear_mid(x, weight, bias, out_dtype)
         return ops.linear_skinny(x, weight, bias, out_dtype)
-    if prefers_mid_passes(m, weight.shape[0], k) and out_dtype == x.dtype:
-        out = torch.empty((m, weight.shape[0]), dtype=out_dtype, device=x.device)
-        for at in range(0, m, SKINNY_MAX_ROWS):
-            ops.linear_mid(x[at:at + SKINNY_MAX_ROWS], weight, bias, out_dtype, out=out[at:at + SKINNY_MAX_ROWS])
-        return out
     if out_dtype == x.dtype and ops.big_supported(x, weight):
         return ops.linear_big(x, weight, bias)
     if out_dtype == torch.float32 and ops.big_supported(x, weight):

@@ -611,8 +611,7 @@ def linear_rope_store(x: torch.Tensor, eps: float, stats: torch.Tensor | None, w
 
 
 def linear_mid(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None,
-               out_dtype: torch.dtype | None = None, swiglu: bool = False,
-               out: torch.Tensor | None = None) -> torch.Tensor:
+               out_dtype: torch.dtype | None = None, swiglu: bool = False) -> torch.Tensor:
     """x @ weight.T (+ bias) for at most 64 bfloat16 rows, x shared by the wavefronts of a workgroup, K split
     over workgroups where the columns do not fill the device.  With ``swiglu`` weight is [2 I, K] with gate and
     up rows interleaved in blocks of 16 and the result is silu(x @ gate.T) * (x @ up.T)."""
@@ -625,9 +624,7 @@ def linear_mid(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None 
     if bias is not None:
         _need(bias, "linear bias", torch.float32, (n,))
     out_dtype = out_dtype or x.dtype
-    if out is None:
-        out = torch.empty((m, n // 2 if swiglu else n), dtype=out_dtype, device=x.device)
-    _need(out, "linear_mid out", out_dtype, (m, n // 2 if swiglu else n))
+    out = torch.empty((m, n // 2 if swiglu else n), dtype=out_dtype, device=x.device)
     workspace = _mid_workspace(x.device)
     _check(library().somi_linear_mid(_ptr(x), _ptr(weight), _ptr(bias), _ptr(out), dtype_code(out_dtype), m, n, k,
                                      1 if swiglu else 0, _ptr(workspace), ctypes.c_int64(workspace.numel()), _stream()))

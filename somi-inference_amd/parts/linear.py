@@ -77,21 +77,15 @@ class Projection:
                 x = x.materialize()
             return linear_kernels.linear(x, self.weight, self.bias, out_dtype)
 
-    def _takes_fused_kernels(self, rows: int) -> bool:
+    def fusable(self, rows: int) -> bool:
+        """The kernels that fuse this product with the norm before it, or with the add into the stream after it, take
+        it."""
         return (self.weight.dtype == torch.bfloat16 and rows > 0 and self.in_features % 8 == 0
                 and self.weight.data_ptr() % 16 == 0)
-
-    def fusable(self, rows: int) -> bool:
-        """The kernels that fuse this product with the norm before it take it, and are the fastest way to it."""
-        if not self._takes_fused_kernels(rows):
-            return False
-        # some dozens of rows beyond what the few-rows kernels take, over a long K and few columns: the split-K
-        # kernel in passes of 64 rows (kernels.linear.linear) is faster there than one 256-row tile per column tile
-        return not linear_kernels.prefers_mid_passes(rows, self.out_features, self.in_features)
 
     def deferred(self, x: torch.Tensor) -> "torch.Tensor | DeferredProduct":
         """The product, or a promise of it where the residual stream can compute and add it in one kernel (any number
         of bfloat16 rows: the few-rows kernels, or the many-rows kernel, which shares a tile's K where tiles are few)."""
-        if x.dtype == torch.bfloat16 and x.data_ptr() % 16 == 0 and self._takes_fused_kernels(x.shape[0]):
+        if x.dtype == torch.bfloat16 and x.data_ptr() % 16 == 0 and self.fusable(x.shape[0]):
             return DeferredProduct(self, x)
         return self(x)

@@ -46,9 +46,6 @@ def test_a_split_is_no_longer_than_the_page_list_in_lds_holds(device_of_256_unit
 
 
 def test_rows_of_a_product_into_the_stream_choose_their_kernel(device_of_256_units):
-    # a kept product with a long K and few columns: passes of the split-K kernel up to 128 rows
-    assert products.prefers_mid_passes(100, 3584, 18944) and not products.prefers_mid_passes(129, 3584, 18944)
-    assert not products.prefers_mid_passes(100, 37888, 3584)
     # the few-rows choice between the kernel that splits K and the one that does not goes with the device's units
     assert products._mid_is_faster(32, 3584, 18944) and products._mid_is_faster(64, 37888, 3584)
     assert not products._mid_is_faster(16, 3584, 18944) and not products._mid_is_faster(64, 4608, 3584)
