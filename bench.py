@@ -149,12 +149,16 @@ def measure_peaks(device) -> dict:
     shapes = {}
     for shape in ops.probe_stream_shapes():
         shapes[shape] = round((2 << 30) / 1e9 / timed(lambda: ops.probe_stream_read(buffer, shape), 5), 1)
+    # matrix instructions on operands as a product has them, and on small integers (most bits zero: the clock under
+    # matrix instructions goes with what the operands toggle, so this loop runs faster than any product can)
     flops = ops.probe_mfma(20000, device)
     mfma_s = timed(lambda: ops.probe_mfma(20000, device), 3)
+    sparse_s = timed(lambda: ops.probe_mfma(20000, device, dense=False), 3)
     del buffer
     best = max(shapes, key=shapes.get)
     return {"stream_read_gbs": shapes[best], "stream_read_shape": best, "stream_read_by_shape": shapes,
-            "mfma_bf16_tflops": round(flops / mfma_s / 1e12, 1)}
+            "mfma_bf16_tflops": round(flops / mfma_s / 1e12, 1),
+            "mfma_bf16_tflops_small_integers": round(flops / sparse_s / 1e12, 1)}
 
 
 def qwen2_config_dict(sizes: str, layers: int | None) -> dict:

@@ -97,13 +97,24 @@ probe_tile_rows_kernel(const char* __restrict__ src, int row_groups, int row_byt
 }
 
 // Every wavefront multiplies `iters` times four independent 32 x 32 x 16 bfloat16 products (32,768 flops each).
+// dense: operands with every mantissa bit in use (hashed values in [-1, 1)), as a product of real activations and
+// weights has them; otherwise small integers, most of whose bits are zero.  The part's clock under matrix
+// instructions goes with what the operands toggle: the same loop runs a third slower on dense operands, and that is
+// the rate a product can be held against.
 __global__ void __launch_bounds__(512)
-probe_mfma_kernel(int iters, float* __restrict__ out) {
+probe_mfma_kernel(int iters, int dense, float* __restrict__ out) {
     bf16x8 a, b;
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-        a[e] = (bf16)(float)((threadIdx.x + e) & 3);
-        b[e] = (bf16)(float)((threadIdx.x * 3 + e) & 1);
+        if (dense) {
+            unsigned ha = (threadIdx.x * 8u + e + blockIdx.x * 4099u) * 2654435761u, hb = (ha ^ 0x9e3779b9u) * 2246822519u;
+            ha ^= ha >> 15; hb ^= hb >> 13;
+            a[e] = (bf16)((float)(int)(ha & 0xffff) * (1.f / 32768.f) - 1.f);
+            b[e] = (bf16)((float)(int)(hb & 0xffff) * (1.f / 32768.f) - 1.f);
+        } else {
+            a[e] = (bf16)(float)((threadIdx.x + e) & 3);
+            b[e] = (bf16)(float)((threadIdx.x * 3 + e) & 1);
+        }
     }
     f32x16 c0 = {0}, c1 = {0}, c2 = {0}, c3 = {0};
     for (int i = 0; i < iters; ++i) {
@@ -199,14 +210,15 @@ extern "C" int somi_probe_stream_read(const void* src, int64_t bytes, int shape,
 }
 
 // Runs the products on every compute unit (two wavefronts per SIMD); returns the number of flops through *flops.
-extern "C" int somi_probe_mfma(int iters, float* out, double* flops, hipStream_t stream) {
+// dense: see probe_mfma_kernel.
+extern "C" int somi_probe_mfma(int iters, int dense, float* out, double* flops, hipStream_t stream) {
     SOMI_REQUIRE(iters > 0 && out != nullptr, "probe_mfma: bad arguments");
     int device = 0;
     hipDeviceProp_t prop;
     SOMI_REQUIRE(hipGetDevice(&device) == hipSuccess && hipGetDeviceProperties(&prop, device) == hipSuccess,
                  "probe_mfma: no device properties");
     const int blocks = prop.multiProcessorCount;
-    hipLaunchKernelGGL(probe_mfma_kernel, dim3(blocks), dim3(512), 0, stream, iters, out);
+    hipLaunchKernelGGL(probe_mfma_kernel, dim3(blocks), dim3(512), 0, stream, iters, dense, out);
     SOMI_LAUNCH_CHECK("probe_mfma");
     if (flops != nullptr) *flops = (double)blocks * 8.0 * (double)iters * 4.0 * 32768.0;
     return 0;

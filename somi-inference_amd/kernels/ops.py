@@ -699,10 +699,12 @@ def probe_stream_read(buffer: torch.Tensor, shape: str | int = 0) -> None:
     _check(lib.somi_probe_stream_read(_ptr(buffer), ctypes.c_int64(size), index, _ptr(sink), _stream()))
 
 
-def probe_mfma(iters: int, device: torch.device | str = "cuda:0") -> float:
+def probe_mfma(iters: int, device: torch.device | str = "cuda:0", dense: bool = True) -> float:
     """Runs ``iters`` rounds of four bfloat16 32 x 32 x 16 matrix instructions on every wavefront slot the launch
-    fills (two per SIMD); returns the flops the launch does."""
+    fills (two per SIMD); returns the flops the launch does.  ``dense``: operands with every mantissa bit in use, as
+    real activations and weights have them (the clock under matrix instructions goes with what the operands toggle);
+    otherwise small integers."""
     sink = torch.zeros((1,), dtype=torch.float32, device=device)
     flops = ctypes.c_double(0.0)
-    _check(library().somi_probe_mfma(int(iters), _ptr(sink), ctypes.byref(flops), _stream()))
+    _check(library().somi_probe_mfma(int(iters), 1 if dense else 0, _ptr(sink), ctypes.byref(flops), _stream()))
     return float(flops.value)
