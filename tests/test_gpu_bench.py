@@ -84,3 +84,18 @@ def test_bench_line_of_a_tiny_configuration_from_a_config_json(tmp_path):
     many = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True,
                           timeout=120)
     assert many.returncode == 2 and "one GPU" in many.stdout
+
+
+def test_the_machines_own_peaks_are_measured_with_the_probes():
+    """The probes behind the measured peaks run: every launch shape of the streaming read over a small buffer, and the
+    loop of matrix instructions on dense operands and on small integers (the same number of operations either way)."""
+    import torch
+    from somi_inference_amd.kernels import ops
+    buffer = torch.zeros(1 << 22, dtype=torch.int32, device="cuda:0")
+    shapes = ops.probe_stream_shapes()
+    assert len(shapes) >= 8 and any("non-temporal" in s for s in shapes)
+    for shape in shapes:
+        ops.probe_stream_read(buffer, shape)
+    dense = ops.probe_mfma(50, "cuda:0")
+    assert dense == ops.probe_mfma(50, "cuda:0", dense=False) > 0
+    torch.cuda.synchronize()
