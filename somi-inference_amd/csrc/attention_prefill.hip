@@ -239,7 +239,7 @@ attention_prefill_kernel(const bf16* __restrict__ q, int64_t q_stride, const bf1
 // units (the figures in brackets: on the 256 units of an MI355X, where they were measured at 28 query heads).
 static int prefill_wide_groups(int units) { return units * 75 / 32; }        // [600] from this many 128-query groups on, workgroups take 128 queries, else 64 (448 groups 72 against 82 us with 64 queries, 672 groups 136 against 119)
 static int prefill_wide_groups_cached(int units) { return units; }           // [256] the same where at least half of the keys were cached before the step
-static int prefill_tile_wide_groups(int units) { return 2 * units; }         // [512] from this many 256-query groups on the tile kernel takes 256 queries a workgroup
+static int prefill_tile_wide_groups(int units) { return 3 * units / 2; }     // [384] from this many 256-query groups on the tile kernel takes 256 queries a workgroup (336 groups, 3,072 tokens: 118 us either way; 448 groups, 4,096 tokens: 166 against 183)
 static int prefill_key_split_below(int units) { return 7 * units / 2; }      // [896] below this many 64-query workgroups two wavefronts share a query block's keys
                                                                              // (448 workgroups 29 against 33 us, 512 tokens after 3,584 cached 83 against 108; 896 workgroups the same; 1,120 workgroups 94 against 89)
 // The launch shapes of the LDS kernel; a caller may ask for one (tests do, to reach each at small sizes).

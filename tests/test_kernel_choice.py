@@ -106,9 +106,10 @@ def test_launch_shapes_inside_the_library_go_with_the_devices_compute_units():
     assert shape(1, 512, 4096, 28, 256) == SPLIT and shape(12, 512, 4096, 28, 256) == WIDE
     # a short context (no workgroup walks 1,024 keys) keeps the plain shape
     assert shape(1, 512, 512, 28, 256) == NARROW
-    # the tile kernel: 256 queries a workgroup from two groups a unit on
+    # the tile kernel: 256 queries a workgroup from three groups for two units on
     assert shape(1, 2048, 2048, 28, 256, tile=1) == TILE and shape(1, 8192, 8192, 28, 256, tile=1) == TILE_WIDE
-    assert shape(1, 8192, 8192, 28, 512, tile=1) == TILE
+    assert shape(1, 3072, 3072, 28, 256, tile=1) == TILE and shape(1, 4096, 4096, 28, 256, tile=1) == TILE_WIDE
+    assert shape(1, 4096, 4096, 28, 512, tile=1) == TILE
 
 
 def test_the_many_rows_product_deals_out_units_only_where_it_is_asked_to():
